@@ -1,0 +1,194 @@
+/*
+ * minit_hip.h -- C ABI of the MI355X (gfx950) quantized-linear hot path.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers and sizes, never
+ * throws and never allocates device memory behind the caller's back (the
+ * mh_malloc family aside, which *is* the allocator).  Device pointers are
+ * caller-owned.  `stream` is a hipStream_t passed as void*; NULL is the null
+ * stream, which is what the reference's Python host passes to every kernel
+ * (`kernel(None, ...)`, e.g. minit/cuda/dispatch.py:442).
+ *
+ * Return value: 0 on success, non-zero on failure; mh_last_error() then
+ * returns a thread-local, NUL-terminated description.  The reference instead
+ * throws std::runtime_error through its extern "C" launchers
+ * (minit/cuda/allocator.py:21-27), which terminates the process.
+ *
+ * All matrices are dense row-major.  fp16 is IEEE binary16.
+ */
+#ifndef MINIT_HIP_H
+#define MINIT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mh_stream_t;
+typedef void* mh_event_t;
+
+#define MH_OK 0
+#define MH_ERR_INVALID 1   /* bad argument / shape contract violated */
+#define MH_ERR_HIP 2       /* a HIP runtime call failed              */
+#define MH_ERR_WORKSPACE 3 /* workspace missing or too small         */
+
+/* ---- library ------------------------------------------------------------ */
+
+int mh_abi_version(void);
+const char* mh_last_error(void);
+
+/* ---- device runtime ------------------------------------------------------
+ * Replaces the allocator shim minit/cuda/allocator.py:30-50
+ * (allocate_cuda_memory / copy_cuda_memory / free_cuda_memory / sync_cuda /
+ * reset), with an explicit stream and error codes.
+ */
+int mh_device_count(int* count);
+int mh_device_info(int* compute_units, int* wavefront_size, size_t* total_mem,
+                   size_t* lds_per_block, int* clock_khz, char* name, size_t name_len);
+int mh_malloc(void** ptr, size_t bytes);
+int mh_free(void* ptr);
+int mh_host_malloc(void** ptr, size_t bytes); /* pinned host memory */
+int mh_host_free(void* ptr);
+int mh_memcpy(void* dst, const void* src, size_t bytes, mh_stream_t stream); /* any direction, async */
+int mh_memset(void* dst, int value, size_t bytes, mh_stream_t stream);
+int mh_stream_create(mh_stream_t* stream);
+int mh_stream_destroy(mh_stream_t stream);
+int mh_stream_synchronize(mh_stream_t stream);
+int mh_device_synchronize(void);
+int mh_event_create(mh_event_t* event);
+int mh_event_destroy(mh_event_t event);
+int mh_event_record(mh_event_t event, mh_stream_t stream);
+int mh_event_synchronize(mh_event_t event);
+int mh_event_elapsed_ms(float* ms, mh_event_t start, mh_event_t stop);
+/* dst[i] = src[i], 16-byte vectors; the plain copy kernel the bandwidth
+ * counters are calibrated against. bytes must be a multiple of 16. */
+int mh_copy_kernel(mh_stream_t stream, const void* src, void* dst, size_t bytes);
+
+/* ---- GPTQ sub-word unpack -------------------------------------------------
+ * Replaces `unpack(x, axis)` (examples/qwen1_5_int8.py:40-50) and the
+ * RowPackedMatrix / ColPackedMatrix accessors (:97-138), generic in `bits`
+ * (4 or 8).  packed is int32 [rows, cols]; out is uint8
+ * [rows * (32/bits), cols] for axis 0, [rows, cols * (32/bits)] for axis 1.
+ */
+int mh_gptq_unpack(mh_stream_t stream, const int32_t* packed, uint8_t* out,
+                   size_t rows, size_t cols, int axis, int bits);
+
+/* ---- GPTQ dequantize --------------------------------------------------------
+ * Replaces dispatch_dequantize (minit/quantize/dispatch.py:14-20) applied to
+ * the packed checkpoint tensors: out[k, n] = fp16((q[k,n] - (z[g,n] + 1)) * s[g,n]),
+ * g = g_idx[k] (g_idx == NULL means g = k / group_size).
+ *   qweight int32 [K/P, N] (packed along K), qzeros int32 [G, N/P] (packed
+ *   along N), scales fp16 [G, N], g_idx int32 [K] or NULL, out fp16 [K, N];
+ *   P = 32 / bits, G = K / group_size.
+ */
+int mh_gptq_dequant(mh_stream_t stream, const int32_t* qweight, const int32_t* qzeros,
+                    const void* scales, const int32_t* g_idx, void* out,
+                    int N, int K, int group_size, int bits);
+
+/* ---- GPTQ quantized linear ---------------------------------------------------
+ * Replaces dispatch_quantized_matrix_multiply (minit/quantize/dispatch.py:8-11)
+ * and the fused kernel qmm_* / quantized_matrix_multiply
+ * (examples/qwen1_5_int8.py:202-203, :244-267):
+ *   out[m, n] = fp16( sum_k fp32(x[m,k]) * fp32(W[k,n]) ),  W as in mh_gptq_dequant.
+ * Shape contract (qwen1_5_int8.py:247-254): K == P * rows(qweight) == len(g_idx),
+ * N == P * cols(qzeros) == cols(scales).  Additionally N % 8 == 0,
+ * K % group_size == 0.
+ *
+ * workspace: device scratch of at least mh_gptq_workspace_bytes(M, N, K, ...)
+ * bytes, 256-byte aligned, zero-filled once by the caller before first use
+ * (the kernels leave it zeroed where it must be); may be shared by calls that
+ * are ordered on one stream, never by concurrent calls.
+ *
+ * mh_gptq_gemv   wave64 VALU path, no MFMA; M <= MH_GPTQ_GEMV_MAX_M.
+ * mh_gptq_gemm   fp16 MFMA path; any M >= 1.
+ * mh_gptq_matmul picks one of the two (or the act-order path when g_idx is a
+ *                non-trivial permutation).
+ */
+#define MH_GPTQ_GEMV_MAX_M 4
+size_t mh_gptq_workspace_bytes(int M, int N, int K, int group_size, int bits);
+int mh_gptq_gemv(mh_stream_t stream, const void* x, const int32_t* qweight,
+                 const int32_t* qzeros, const void* scales, const int32_t* g_idx,
+                 void* out, int M, int N, int K, int group_size, int bits,
+                 void* workspace, size_t workspace_bytes);
+int mh_gptq_gemm(mh_stream_t stream, const void* x, const int32_t* qweight,
+                 const int32_t* qzeros, const void* scales, const int32_t* g_idx,
+                 void* out, int M, int N, int K, int group_size, int bits,
+                 void* workspace, size_t workspace_bytes);
+int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight,
+                   const int32_t* qzeros, const void* scales, const int32_t* g_idx,
+                   void* out, int M, int N, int K, int group_size, int bits,
+                   void* workspace, size_t workspace_bytes);
+
+/* ---- dense fp16 product --------------------------------------------------------
+ * Replaces dispatch_matmul + minit_gemm (minit/cuda/dispatch.py:59-78,
+ * minit/cuda/kernel/cublas.py:68-111) for batch == 1:
+ *   out[m, n] = fp16( sum_k fp32(a[m,k]) * fp32(b[n,k]) ), b stored [N, K].
+ */
+int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out,
+                     int M, int N, int K);
+
+/* ---- W8A8 int8 GEMM --------------------------------------------------------------
+ * No counterpart in the reference (its "int8" model is weight-only,
+ * examples/qwen1_5_int8.py:156-200); operand orientation follows the
+ * reference's dense product, weight stored [N, K].
+ *   acc[m, n] = sum_k int32(a[m,k]) * int32(w[n,k])                (exact)
+ *   out[m, n] = fp16( fp32(acc[m,n]) * (a_scale[m] * w_scale[n]) )
+ * acc_i32 may be NULL (accumulators are then not written out); out_f16 may be
+ * NULL when only the accumulators are wanted.  K % 64 == 0.
+ */
+int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w,
+               const float* a_scale, const float* w_scale, void* out_f16,
+               int32_t* acc_i32, int M, int N, int K);
+/* out[n, k] = in[k, n]: one-time layout conversion for weights stored [K, N]. */
+int mh_i8_transpose(mh_stream_t stream, const int8_t* in, int8_t* out, int rows, int cols);
+
+/* ---- normalisation, rotary, softmax, reductions ---------------------------------------
+ * Same view convention as the reference: the tensor is seen as [a, b, c] and
+ * the operation runs along b.  dtype: 0 = fp16, 1 = bf16, 2 = fp32.
+ */
+#define MH_F16 0
+#define MH_BF16 1
+#define MH_F32 2
+
+/* minit_rms_norm (minit/cuda/kernel/cuda/rms_norm.py:94):
+ * out = T( x / sqrt(sum(x^2)/b + (float)eps) * w[b] ), fp32 internally. */
+int mh_rms_norm(mh_stream_t stream, const void* in, const void* weight, void* out,
+                size_t a, size_t b, size_t c, double eps, int dtype);
+
+/* minit_rope (minit/cuda/kernel/cuda/rope.py:75): x is [bs, seq, nh, hs],
+ * interleaved pairs rotated by fp32 tables.  positions == NULL: tables are
+ * [seq, hs/2] indexed by the sequence index (the reference form).
+ * positions != NULL: int32 [bs, seq]; tables are [nr_positions, hs/2] and row
+ * positions[b, s] is used (must be < nr_positions). */
+int mh_rope(mh_stream_t stream, const void* in, const float* freqs_cos,
+            const float* freqs_sin, const int32_t* positions, void* out,
+            size_t bs, size_t seq, size_t nh, size_t hs, int dtype);
+
+/* minit_softmax (minit/cuda/kernel/cuda/softmax.py:109): softmax along b. */
+int mh_softmax(mh_stream_t stream, const void* in, void* out,
+               size_t a, size_t b, size_t c, int dtype);
+
+/* Softmax with the models' causal mask and 1/sqrt(d) scale fused in
+ * (examples/llama3_70b.py:102-112): in is [rows_outer, s, t] with
+ * t == offset + s; out[., i, j] = softmax_j( T(in * scale) + m[i, j] ),
+ * m[i, j] = -inf iff j - offset > i.  scale == 1 skips the multiply. */
+int mh_softmax_causal(mh_stream_t stream, const void* in, void* out,
+                      size_t rows_outer, size_t s, size_t t, size_t offset,
+                      float scale, int dtype);
+
+/* minit_sum / minit_max (minit/cuda/kernel/cuda/reduce.py:95): [a,b,c] -> [a,1,c]. */
+int mh_sum(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype);
+int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype);
+
+/* silu(gate) * up in one pass (the models run sigmoid, multiply, multiply as
+ * three launches: examples/llama3_70b.py:44-45,126-130,
+ * minit/cuda/dispatch.py:137,143).  exact != 0 reproduces the three fp16
+ * roundings of that sequence; exact == 0 keeps fp32 until the store. */
+int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
+                size_t n, int exact, int dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINIT_HIP_H */

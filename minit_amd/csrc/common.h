@@ -1,0 +1,104 @@
+// Shared helpers for the gfx950 kernels: error plumbing, wave64 reductions,
+// 16-bit float vector types.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/minit_hip.h"
+
+namespace mh {
+
+// Records a message for mh_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define MH_CHECK_HIP(expr)                                                        \
+    do {                                                                          \
+        hipError_t _e = (expr);                                                   \
+        if (_e != hipSuccess)                                                     \
+            return ::mh::fail(MH_ERR_HIP, "%s: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+#define MH_REQUIRE(cond, ...)                                   \
+    do {                                                        \
+        if (!(cond)) return ::mh::fail(MH_ERR_INVALID, __VA_ARGS__); \
+    } while (0)
+
+// Launch-error check that does not synchronise.
+#define MH_CHECK_LAUNCH() MH_CHECK_HIP(hipGetLastError())
+
+inline hipStream_t as_stream(mh_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Number of compute units of the current device (cached per process).
+int compute_units();
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+typedef int int16_t_v __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Block-wide reductions over up to 16 waves; `smem` holds >= 16 floats and may
+// be reused after the call returns (the helper syncs on both sides).
+__device__ __forceinline__ float block_sum(float v, float* smem) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwaves = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float r = 0.f;
+    for (int i = 0; i < nwaves; ++i) r += smem[i];
+    return r;
+}
+
+__device__ __forceinline__ float block_max(float v, float* smem) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwaves = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float r = -INFINITY;
+    for (int i = 0; i < nwaves; ++i) r = fmaxf(r, smem[i]);
+    return r;
+}
+
+// 16-bit storage <-> fp32.
+template <typename T> struct Cvt;
+template <> struct Cvt<half_t> {
+    static __device__ __forceinline__ float to_f32(half_t v) { return (float)v; }
+    static __device__ __forceinline__ half_t from_f32(float v) { return (half_t)v; }
+};
+template <> struct Cvt<__hip_bfloat16> {
+    static __device__ __forceinline__ float to_f32(__hip_bfloat16 v) { return __bfloat162float(v); }
+    static __device__ __forceinline__ __hip_bfloat16 from_f32(float v) { return __float2bfloat16(v); }
+};
+template <> struct Cvt<float> {
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+    static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+
+}  // namespace mh

@@ -1,0 +1,114 @@
+// Dense fp16 product with the reference's operand orientation:
+//   out[m, n] = fp16( sum_k fp32(a[m, k]) * fp32(b[n, k]) ),  b stored [N, K]
+// (dispatch_matmul + minit_gemm, minit/cuda/dispatch.py:59-78,
+// minit/cuda/kernel/cublas.py:68-111).  Used for the unquantized lm_head at
+// decode and as the dense leg of the act-order path.
+//
+// Both operands are K-contiguous, which is the MFMA operand layout as is: lane l
+// of a 16x16x32 fp16 MFMA holds eight consecutive k of row l % 16, k-chunk l / 16,
+// i.e. one 16-byte load straight from global memory for either operand.  A wave
+// owns 16 rows of b (16 output columns) for all of K; b is streamed once, a is
+// small and served by the caches.
+#include "common.h"
+
+namespace mh {
+
+constexpr int kDenseDepth = 4;
+
+template <int MT>
+__global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __restrict__ a,
+                                                            const half_t* __restrict__ b,
+                                                            half_t* __restrict__ out, int M, int N, int K) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i16 = lane & 15, kq = lane >> 4;
+    const int n0 = (blockIdx.x * 4 + wave) * 16;
+    const int m0 = blockIdx.y * (16 * MT);
+    if (n0 >= N) return;
+    const int n = min(n0 + i16, N - 1);
+    const half_t* brow = b + (size_t)n * K + kq * 8;
+    const half_t* arow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = a + (size_t)min(m0 + mt * 16 + i16, M - 1) * K + kq * 8;
+
+    float4_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int steps = K / 32;
+    constexpr int D = kDenseDepth;
+    uint4_t bq[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        bq[d] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow + (size_t)min(d, steps - 1) * 32));
+    for (int s0 = 0; s0 < steps; s0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int s = s0 + d;
+            if (s < steps) {
+                const half8_t bf = __builtin_bit_cast(half8_t, bq[d]);
+                bq[d] = __builtin_nontemporal_load(
+                    reinterpret_cast<const uint4_t*>(brow + (size_t)min(s + D, steps - 1) * 32));
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const half8_t af = *reinterpret_cast<const half8_t*>(arow[mt] + (size_t)s * 32);
+                    // rows of the result are m (operand A), columns are n (operand B)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf, acc[mt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // acc[mt][r] is row m0 + mt*16 + kq*4 + r, column n0 + i16
+    if (n0 + i16 < N) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + mt * 16 + kq * 4 + r;
+                if (m < M) out[(size_t)m * N + n0 + i16] = (half_t)acc[mt][r];
+            }
+    }
+}
+
+// Any K (no divisibility or alignment assumptions): one thread per output.
+__global__ void f16_matmul_nk_generic_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
+                                             half_t* __restrict__ out, int M, int N, int K) {
+    const size_t total = (size_t)M * N;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int m = (int)(idx / N), n = (int)(idx % N);
+        float acc = 0.f;
+        for (int k = 0; k < K; ++k) acc = __builtin_fmaf((float)a[(size_t)m * K + k], (float)b[(size_t)n * K + k], acc);
+        out[idx] = (half_t)acc;
+    }
+}
+
+}  // namespace mh
+
+using namespace mh;
+
+extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out, int M, int N,
+                                int K) {
+    MH_REQUIRE(M >= 0 && N >= 0 && K >= 0, "mh_f16_matmul_nk: bad shape M=%d N=%d K=%d", M, N, K);
+    if (M == 0 || N == 0) return MH_OK;
+    MH_REQUIRE(a && b && out, "mh_f16_matmul_nk: null pointer");
+    hipStream_t st = as_stream(stream);
+    const bool fast = K > 0 && K % 32 == 0 && ((uintptr_t)a | (uintptr_t)b) % 16 == 0;
+    if (!fast) {
+        size_t blocks = ((size_t)M * N + 255) / 256;
+        const size_t cap = (size_t)compute_units() * 16;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(f16_matmul_nk_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                           (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K);
+        MH_CHECK_LAUNCH();
+        return MH_OK;
+    }
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    dim3 grid((N + 63) / 64, (M + 16 * mt - 1) / (16 * mt));
+    switch (mt) {
+        case 1: hipLaunchKernelGGL(f16_matmul_nk_kernel<1>, grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K); break;
+        case 2: hipLaunchKernelGGL(f16_matmul_nk_kernel<2>, grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K); break;
+        default: hipLaunchKernelGGL(f16_matmul_nk_kernel<4>, grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K); break;
+    }
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}

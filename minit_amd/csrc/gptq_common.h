@@ -1,0 +1,133 @@
+// In-register GPTQ sub-word extraction and dequantisation.
+//
+// Arithmetic contract (minit/quantize/dispatch.py:14-20 of the reference, in
+// fp16): W = (q - (z + 1)) * s.  q - (z + 1) is an exact small integer, so the
+// multiply is the only rounding.  The extraction below builds that integer
+// without int->float conversions: OR-ing a sub-word into the mantissa of the
+// fp16 constant 1024 (0x6400) yields 1024 + q exactly (or 1024 + 16 q when the
+// sub-word sits four bits up), and one packed subtract / fma against a
+// per-column constant removes both the bias and the zero point.  Sub-word i of
+// a word sits at bit i * bits (examples/qwen1_5_int8.py:107-116,129-136).
+#pragma once
+
+#include "common.h"
+
+namespace mh {
+
+#pragma clang fp contract(off)
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+template <int BITS> struct Packing;
+template <> struct Packing<4> {
+    static constexpr int kPerWord = 8;
+    static constexpr int kPairs = 4;
+    static constexpr uint32_t kMask = 0xFu;
+};
+template <> struct Packing<8> {
+    static constexpr int kPerWord = 4;
+    static constexpr int kPairs = 2;
+    static constexpr uint32_t kMask = 0xFFu;
+};
+
+// Per-(group, column) constants.
+struct ColumnConst {
+    half2_t scale;   // (s, s)
+    half2_t zero_lo; // (1024 + z + 1) twice
+    half2_t zero_hi; // (64 + z + 1) twice; 4-bit only
+};
+
+__device__ __forceinline__ ColumnConst make_column_const(half_t s, uint32_t z) {
+    ColumnConst c;
+    const half_t zp1 = (half_t)(float)(z + 1u);  // exact: z + 1 <= 256
+    c.scale = half2_t{s, s};
+    const half_t lo = (half_t)1024.0f + zp1;
+    const half_t hi = (half_t)64.0f + zp1;
+    c.zero_lo = half2_t{lo, lo};
+    c.zero_hi = half2_t{hi, hi};
+    return c;
+}
+
+// Bit masks and the fp16 bias kept in registers so that each extraction is a
+// single v_and_or_b32 (VOP3 on gfx9 takes no literals; left as literals the
+// compiler splits it into v_and + v_or).  Build once per kernel.
+struct DequantRegs {
+    uint32_t magic;    // 0x64006400: fp16 1024.0 twice
+    uint32_t mask_lo;  // sub-word in mantissa bits 0..3 (or 0..7)
+    uint32_t mask_hi;  // sub-word in mantissa bits 4..7; 4-bit only
+    __device__ __forceinline__ void init(int bits) {
+        magic = 0x64006400u;
+        mask_lo = bits == 4 ? 0x000F000Fu : 0x00FF00FFu;
+        mask_hi = 0x00F000F0u;
+        asm volatile("" : "+v"(magic));
+        asm volatile("" : "+s"(mask_lo));
+        asm volatile("" : "+s"(mask_hi));
+    }
+};
+
+// Dequantises one packed word of one column into kPairs half2 values.
+// Element order ("pair order") for 4 bits: (k0,k4) (k1,k5) (k2,k6) (k3,k7);
+// for 8 bits: (k0,k2) (k1,k3).  Callers pair the activations the same way.
+template <int BITS>
+__device__ __forceinline__ void dequant_word(uint32_t q, const ColumnConst& c, const DequantRegs& r,
+                                             half2_t* w);
+
+template <>
+__device__ __forceinline__ void dequant_word<4>(uint32_t q, const ColumnConst& c, const DequantRegs& r,
+                                                half2_t* w) {
+    const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+    const uint32_t q8 = q >> 8;
+    const half2_t p0 = as_half2((q & r.mask_lo) | r.magic);
+    const half2_t p1 = as_half2((q & r.mask_hi) | r.magic);
+    const half2_t p2 = as_half2((q8 & r.mask_lo) | r.magic);
+    const half2_t p3 = as_half2((q8 & r.mask_hi) | r.magic);
+    w[0] = (p0 - c.zero_lo) * c.scale;
+    w[1] = __builtin_elementwise_fma(p1, sixteenth, -c.zero_hi) * c.scale;
+    w[2] = (p2 - c.zero_lo) * c.scale;
+    w[3] = __builtin_elementwise_fma(p3, sixteenth, -c.zero_hi) * c.scale;
+}
+
+template <>
+__device__ __forceinline__ void dequant_word<8>(uint32_t q, const ColumnConst& c, const DequantRegs& r,
+                                                half2_t* w) {
+    const half2_t p0 = as_half2((q & r.mask_lo) | r.magic);
+    const half2_t p1 = as_half2(((q >> 8) & r.mask_lo) | r.magic);
+    w[0] = (p0 - c.zero_lo) * c.scale;
+    w[1] = (p1 - c.zero_lo) * c.scale;
+}
+
+// Re-orders 2*kPairs consecutive activations (as packed 32-bit words holding
+// two fp16 each) into the pair order of dequant_word.
+template <int BITS>
+__device__ __forceinline__ void pair_activations(const uint32_t* x, uint32_t* xp);
+
+template <>
+__device__ __forceinline__ void pair_activations<4>(const uint32_t* x, uint32_t* xp) {
+    // x[0]=(k0,k1) x[1]=(k2,k3) x[2]=(k4,k5) x[3]=(k6,k7)
+    xp[0] = (x[0] & 0xFFFFu) | (x[2] << 16);
+    xp[1] = (x[0] >> 16) | (x[2] & 0xFFFF0000u);
+    xp[2] = (x[1] & 0xFFFFu) | (x[3] << 16);
+    xp[3] = (x[1] >> 16) | (x[3] & 0xFFFF0000u);
+}
+
+template <>
+__device__ __forceinline__ void pair_activations<8>(const uint32_t* x, uint32_t* xp) {
+    // x[0]=(k0,k1) x[1]=(k2,k3)
+    xp[0] = (x[0] & 0xFFFFu) | (x[1] << 16);
+    xp[1] = (x[0] >> 16) | (x[1] & 0xFFFF0000u);
+}
+
+// Host-side argument validation shared by the GPTQ entry points.
+int check_gptq_args(const char* who, const void* x, const void* qweight, const void* qzeros,
+                    const void* scales, const void* out, int M, int N, int K, int group_size,
+                    int bits);
+
+// Split-K plan shared by the kernels and mh_gptq_workspace_bytes.
+struct SplitPlan {
+    int col_tiles;
+    int split_k;          // blocks along K
+    int groups_per_wave;  // groups each wave of a block walks
+};
+
+}  // namespace mh

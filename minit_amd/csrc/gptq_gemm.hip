@@ -1,0 +1,355 @@
+// GPTQ w4a16 / w8a16 dequant-GEMM on CDNA4 fp16 MFMA (v_mfma_f32_16x16x32_f16).
+//
+// Replaces the fused qmm kernel of the reference
+// (examples/qwen1_5_int8.py:156-216) for M above the GEMV range.
+//
+// Mapping.  The B operand of a 16x16x32 MFMA wants, in lane l, eight
+// consecutive k of column l % 16, k-chunk l / 16 -- for 4-bit GPTQ that is
+// exactly one packed word of qweight.  A lane therefore loads 16 bytes (four
+// adjacent columns of one packed row), dequantises each word in registers
+// (gptq_common.h) and feeds it to one of four MFMAs; the weights never touch
+// LDS.  The order of k inside a word that the extraction produces is applied to
+// the activations instead, when they are staged into LDS, so both operands
+// agree.  A block is four waves side by side along N (256 columns, 1 KiB
+// contiguous per packed row) sharing one activation tile [16*MT, KC] in LDS.
+// K is split over blockIdx.y with fp32 partials summed in split order by the
+// last block to arrive (deterministic).
+#include "gptq_common.h"
+
+namespace mh {
+
+#pragma clang fp contract(off)
+
+constexpr int kGemmCols = 256;
+constexpr int kGemmDepth = 4;  // weight prefetch distance in k-steps
+
+template <int MT> struct GemmStage { static constexpr int kSteps = MT <= 2 ? 16 : (MT == 4 ? 8 : 4); };
+
+template <int BITS, int MT>
+__global__ __launch_bounds__(256) void gptq_gemm_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
+    half_t* __restrict__ out, float* partial, unsigned* counters,
+    int M, int N, int K, int steps_per_group, int steps_total, int steps_per_block, int split_k) {
+    constexpr int P = Packing<BITS>::kPerWord;
+    constexpr int PAIRS = Packing<BITS>::kPairs;
+    constexpr uint32_t MASK = Packing<BITS>::kMask;
+    constexpr int BM = 16 * MT;
+    constexpr int ROWS_PER_STEP = 32 / P;     // packed rows per 32-k step
+    constexpr int LOADS = ROWS_PER_STEP / 4;  // 16-byte loads per lane per step
+    constexpr int SC = GemmStage<MT>::kSteps; // k-steps per LDS stage
+    constexpr int CHUNKS = SC * 4;            // 16-byte chunks per activation row per stage
+    constexpr int RS = CHUNKS + 1;            // padded row stride in chunks
+    constexpr int XLOADS = BM * CHUNKS / 256; // chunks each thread stages
+    constexpr int D = kGemmDepth;
+    static_assert(SC % D == 0, "stage must be a multiple of the prefetch depth");
+
+    __shared__ uint4 xs[BM * RS];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nl = lane & 15, kq = lane >> 4;
+    const int tile = blockIdx.x, split = blockIdx.y, mblock = blockIdx.z;
+    const int m0 = mblock * BM;
+    const int col = tile * kGemmCols + wave * 64 + nl * 4;
+    const bool active = col < N;
+    const int colc = active ? col : 0;
+
+    const int step_begin = split * steps_per_block;
+    const int step_end = min(steps_total, step_begin + steps_per_block);
+    const int last_step = step_end - 1;
+
+    DequantRegs regs;
+    regs.init(BITS);
+
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[mt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // ---- weight stream: ring of D steps in flight --------------------------------------
+    uint4_t qb[D][LOADS];
+    auto load_q = [&](int step, uint4_t* dst) {
+        const int s = min(step, last_step);
+        const size_t row = (size_t)s * ROWS_PER_STEP + kq * LOADS;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j)
+            dst[j] = __builtin_nontemporal_load(
+                reinterpret_cast<const uint4_t*>(qweight + (row + j) * N + colc));
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load_q(step_begin + d, qb[d]);
+
+    // ---- per-group constants, fetched one group ahead ------------------------------------
+    uint2 s_next;
+    uint32_t z_next;
+    auto load_consts = [&](int g) {
+        s_next = *reinterpret_cast<const uint2*>(scales + (size_t)g * N + colc);
+        z_next = qzeros[(size_t)g * (N / P) + colc / P];
+    };
+    const int g_last = last_step / steps_per_group;
+    int g_cur = step_begin / steps_per_group;
+    load_consts(g_cur);
+    ColumnConst cc[4];
+    auto take_consts = [&]() {
+        const uint32_t zword = z_next >> ((colc % P) * BITS);
+        const half2_t s01 = as_half2(s_next.x), s23 = as_half2(s_next.y);
+        cc[0] = make_column_const(s01.x, zword & MASK);
+        cc[1] = make_column_const(s01.y, (zword >> BITS) & MASK);
+        cc[2] = make_column_const(s23.x, (zword >> (2 * BITS)) & MASK);
+        cc[3] = make_column_const(s23.y, (zword >> (3 * BITS)) & MASK);
+    };
+    take_consts();
+    load_consts(min(g_cur + 1, g_last));
+
+    // ---- activation staging -----------------------------------------------------------------
+    uint4 xr[XLOADS];
+    auto load_x = [&](int stage_step) {
+#pragma unroll
+        for (int it = 0; it < XLOADS; ++it) {
+            const int idx = it * 256 + tid;
+            const int row = idx / CHUNKS, chunk = idx % CHUNKS;
+            const int m = m0 + row;
+            const int step = stage_step + chunk / 4;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (m < M && step < step_end)
+                v = *reinterpret_cast<const uint4*>(x + (size_t)m * K + (size_t)stage_step * 32 + chunk * 8);
+            xr[it] = v;
+        }
+    };
+    auto store_x = [&]() {
+#pragma unroll
+        for (int it = 0; it < XLOADS; ++it) {
+            const int idx = it * 256 + tid;
+            const int row = idx / CHUNKS, chunk = idx % CHUNKS;
+            const uint32_t in[4] = {xr[it].x, xr[it].y, xr[it].z, xr[it].w};
+            uint32_t o[4];
+            if constexpr (BITS == 4) {
+                pair_activations<4>(in, o);
+            } else {
+                pair_activations<8>(in, o);
+                pair_activations<8>(in + 2, o + 2);
+            }
+            xs[row * RS + chunk] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    };
+
+    load_x(step_begin);
+    for (int s0 = step_begin; s0 < step_end; s0 += SC) {
+        __syncthreads();  // the previous stage has been consumed
+        store_x();
+        __syncthreads();
+        if (s0 + SC < step_end) load_x(s0 + SC);
+
+#pragma unroll
+        for (int i = 0; i < SC; ++i) {
+            const int step = s0 + i;
+            const int g = min(step, last_step) / steps_per_group;
+            if (g != g_cur) {
+                g_cur = g;
+                take_consts();
+                load_consts(min(g + 1, g_last));
+            }
+            // B fragments: four columns, eight k each
+            half8_t b[4];
+            {
+                uint4_t* q = qb[i % D];
+                const uint32_t qa[4] = {q[0].x, q[0].y, q[0].z, q[0].w};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    half2_t w[4];
+                    if constexpr (BITS == 4) {
+                        dequant_word<BITS>(qa[t], cc[t], regs, w);
+                    } else {
+                        const uint32_t qc[4] = {q[LOADS - 1].x, q[LOADS - 1].y, q[LOADS - 1].z, q[LOADS - 1].w};
+                        dequant_word<BITS>(qa[t], cc[t], regs, w);
+                        dequant_word<BITS>(qc[t], cc[t], regs, w + PAIRS);
+                    }
+                    const uint4_t packed = {as_u32(w[0]), as_u32(w[1]), as_u32(w[2]), as_u32(w[3])};
+                    b[t] = __builtin_bit_cast(half8_t, packed);
+                }
+                load_q(step + D, q);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint4 av = xs[(mt * 16 + nl) * RS + i * 4 + kq];
+                const half8_t a = __builtin_bit_cast(half8_t, av);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[mt][t], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- epilogue --------------------------------------------------------------------------------
+    // acc[mt][t][r] is row m0 + mt*16 + kq*4 + r, column col + t.
+    if (split_k == 1) {
+        if (active) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int m = m0 + mt * 16 + kq * 4 + r;
+                    if (m < M) {
+                        const half4_t h = {(half_t)acc[mt][0][r], (half_t)acc[mt][1][r],
+                                           (half_t)acc[mt][2][r], (half_t)acc[mt][3][r]};
+                        *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
+                    }
+                }
+        }
+        return;
+    }
+
+    if (active) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + mt * 16 + kq * 4 + r;
+                if (m < M) {
+                    float* p = partial + ((size_t)split * M + m) * N + col;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        __hip_atomic_store(p + t, acc[mt][t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+    }
+    __threadfence();
+    __syncthreads();
+    __shared__ int is_last;
+    unsigned* counter = counters + (size_t)mblock * gridDim.x + tile;
+    if (tid == 0) {
+        const unsigned prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (prev == (unsigned)(split_k - 1));
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    if (active) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + mt * 16 + kq * 4 + r;
+                if (m < M) {
+                    float s[4] = {0.f, 0.f, 0.f, 0.f};
+                    for (int sp = 0; sp < split_k; ++sp) {
+                        const float* p = partial + ((size_t)sp * M + m) * N + col;
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            s[t] += __hip_atomic_load(p + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+                    *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
+                }
+            }
+    }
+    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- host side ---------------------------------------------------------------------------------------
+
+struct GemmPlan {
+    int mt;  // 16-row tiles per block: 1, 2, 4 or 8
+    int col_tiles;
+    int m_blocks;
+    int split_k;
+    int steps_total;
+    int steps_per_block;
+};
+
+static int env_int_gemm(const char* name, int fallback) {
+    const char* v = getenv(name);
+    if (!v || !*v) return fallback;
+    return atoi(v);
+}
+
+GemmPlan plan_gemm(int M, int N, int K) {
+    GemmPlan p;
+    p.mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
+    const int bm = 16 * p.mt;
+    const int sc = p.mt <= 2 ? 16 : (p.mt == 4 ? 8 : 4);
+    p.col_tiles = (N + kGemmCols - 1) / kGemmCols;
+    p.m_blocks = (M + bm - 1) / bm;
+    p.steps_total = K / 32;
+    static const int blocks_per_cu = env_int_gemm("MH_GEMM_BLOCKS_PER_CU", 2);
+    const long target_blocks = (long)compute_units() * blocks_per_cu;
+    long split = target_blocks / ((long)p.col_tiles * p.m_blocks);
+    // every block walks whole stages; partial sums cost 8*M*N bytes per split
+    const long max_split = (p.steps_total + sc - 1) / sc;
+    if (split > max_split) split = max_split;
+    if (split < 1) split = 1;
+    long spb = (p.steps_total + split - 1) / split;
+    spb = (spb + sc - 1) / sc * sc;
+    p.steps_per_block = (int)spb;
+    p.split_k = (int)((p.steps_total + spb - 1) / spb);
+    return p;
+}
+
+bool gemm_supported(int M, int N, int K, int group_size, int bits) {
+    return M >= 1 && (bits == 4 || bits == 8) && N % 8 == 0 && K % 32 == 0 && group_size % 32 == 0 &&
+           K % group_size == 0;
+}
+
+size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
+    (void)group_size;
+    (void)bits;
+    const GemmPlan p = plan_gemm(M, N, K);
+    size_t counters = ((size_t)p.col_tiles * p.m_blocks * sizeof(unsigned) + 255) / 256 * 256;
+    size_t partial = (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
+    return counters + partial;
+}
+
+template <int BITS, int MT>
+static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
+                        const int32_t* qzeros, const void* scales, void* out, void* workspace, int M, int N,
+                        int K, int group_size) {
+    const size_t counters_bytes = ((size_t)p.col_tiles * p.m_blocks * sizeof(unsigned) + 255) / 256 * 256;
+    unsigned* counters = reinterpret_cast<unsigned*>(workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters_bytes);
+    hipLaunchKernelGGL((gptq_gemm_kernel<BITS, MT>), dim3(p.col_tiles, p.split_k, p.m_blocks), dim3(256), 0,
+                       stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
+                       (const half_t*)scales, (half_t*)out, partial, counters, M, N, K, group_size / 32,
+                       p.steps_total, p.steps_per_block, p.split_k);
+}
+
+template <int BITS>
+static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
+                           const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
+                           int N, int K, int group_size) {
+    switch (p.mt) {
+        case 1: launch_gemm<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size); break;
+        case 2: launch_gemm<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size); break;
+        case 4: launch_gemm<BITS, 4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size); break;
+        default: launch_gemm<BITS, 8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size); break;
+    }
+}
+
+int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                     const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                     void* workspace, size_t workspace_bytes) {
+    const GemmPlan p = plan_gemm(M, N, K);
+    const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
+    if (p.split_k > 1) {
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
+                        workspace ? workspace_bytes : (size_t)0);
+        if ((uintptr_t)workspace % 256 != 0)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace must be 256-byte aligned");
+    }
+    if (bits == 4)
+        launch_gemm_mt<4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+    else
+        launch_gemm_mt<8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+int gemv_gemm_crossover() {
+    static const int m = env_int_gemm("MH_GEMV_MAX_M", MH_GPTQ_GEMV_MAX_M);
+    return m < MH_GPTQ_GEMV_MAX_M ? m : MH_GPTQ_GEMV_MAX_M;
+}
+
+}  // namespace mh

@@ -1,0 +1,266 @@
+// GPTQ w4a16 / w8a16 dequant-GEMV for decode (M <= 4), wave64 VALU, no MFMA.
+//
+// Replaces the fused qmm kernel of the reference
+// (examples/qwen1_5_int8.py:156-216) for small M.  Bandwidth-bound design:
+//
+//   * qweight [K/P, N] is N-contiguous, so lanes walk N: a lane owns four
+//     adjacent columns and fetches them with one 16-byte load per packed row;
+//     a wave therefore streams 1 KiB-contiguous row segments.
+//   * the packed rows a wave walks are wave-uniform, so the activations it
+//     needs are uniform too and live in scalar registers; each dequantised
+//     fp16 pair is consumed by one v_dot2_f32_f16 per output row.
+//   * K is split three ways: over the four waves of a block (reduced through
+//     LDS), over blockIdx.y (fp32 partials in the workspace, summed in a fixed
+//     order by whichever block finishes last -- deterministic, no atomics on
+//     data), and within a lane (private fp32 accumulators).
+//   * zero points and scales are fetched once per (group, column) and folded
+//     into packed fp16 constants (see gptq_common.h).
+#include "gptq_common.h"
+
+namespace mh {
+
+#pragma clang fp contract(off)
+
+constexpr int kGemvCols = 256;     // columns per block: 64 lanes x 4
+constexpr int kGemvWaves = 4;      // waves per block, splitting K
+
+template <int BITS, int M, int ROWS>
+__global__ __launch_bounds__(256) void gptq_gemv_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
+    half_t* __restrict__ out, float* partial, unsigned* counters,
+    int N, int K, int rows_per_group, int steps_total, int steps_per_wave, int split_k) {
+    constexpr int P = Packing<BITS>::kPerWord;
+    constexpr int PAIRS = Packing<BITS>::kPairs;
+    constexpr uint32_t MASK = Packing<BITS>::kMask;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tile = blockIdx.x;
+    const int split = blockIdx.y;
+    const int n = tile * kGemvCols + lane * 4;
+    const bool active = n < N;
+
+    DequantRegs regs;
+    regs.init(BITS);
+
+    float acc[M][4];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[m][c] = 0.f;
+
+    const int slot = split * kGemvWaves + wave;
+    const int step_begin = slot * steps_per_wave;
+    const int step_end = min(steps_total, step_begin + steps_per_wave);
+
+    if (active && step_begin < step_end) {
+        ColumnConst cc[4];
+        int g_cur = -1;
+        for (int step = step_begin; step < step_end; ++step) {
+            const int row = step * ROWS;
+            const uint32_t* wp = qweight + (size_t)row * N + n;
+            uint4_t q[ROWS];
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i)
+                q[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wp + (size_t)i * N));
+
+            const int g = row / rows_per_group;
+            if (g != g_cur) {
+                g_cur = g;
+                const uint2 sraw = *reinterpret_cast<const uint2*>(scales + (size_t)g * N + n);
+                const uint32_t zword = qzeros[(size_t)g * (N / P) + n / P] >> ((n % P) * BITS);
+                const half2_t s01 = as_half2(sraw.x), s23 = as_half2(sraw.y);
+                cc[0] = make_column_const(s01.x, zword & MASK);
+                cc[1] = make_column_const(s01.y, (zword >> BITS) & MASK);
+                cc[2] = make_column_const(s23.x, (zword >> (2 * BITS)) & MASK);
+                cc[3] = make_column_const(s23.y, (zword >> (3 * BITS)) & MASK);
+            }
+
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i) {
+                uint32_t xp[M][PAIRS];
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const uint32_t* xr =
+                        reinterpret_cast<const uint32_t*>(x + (size_t)m * K + (size_t)(row + i) * P);
+                    uint32_t xv[PAIRS];
+#pragma unroll
+                    for (int p = 0; p < PAIRS; ++p) xv[p] = xr[p];
+                    pair_activations<BITS>(xv, xp[m]);
+                }
+                const uint32_t qs[4] = {q[i].x, q[i].y, q[i].z, q[i].w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    half2_t w[PAIRS];
+                    dequant_word<BITS>(qs[c], cc[c], regs, w);
+#pragma unroll
+                    for (int m = 0; m < M; ++m)
+#pragma unroll
+                        for (int p = 0; p < PAIRS; ++p)
+                            acc[m][c] = __builtin_amdgcn_fdot2(as_half2(xp[m][p]), w[p], acc[m][c], false);
+                }
+            }
+        }
+    }
+
+    // K-reduction across the four waves of the block.
+    __shared__ float red[kGemvWaves][M][kGemvCols];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+        *reinterpret_cast<float4*>(&red[wave][m][lane * 4]) =
+            make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+    __syncthreads();
+
+    const int t = threadIdx.x;
+    const int nt = tile * kGemvCols + t;
+    float total[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) total[m] = (red[0][m][t] + red[1][m][t]) + (red[2][m][t] + red[3][m][t]);
+
+    if (split_k == 1) {
+        if (nt < N) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) out[(size_t)m * N + nt] = (half_t)total[m];
+        }
+        return;
+    }
+
+    // K-reduction across blocks: publish the partial, the last block to arrive
+    // for this column tile sums all of them in split order.
+    if (nt < N) {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            __hip_atomic_store(&partial[((size_t)split * M + m) * N + nt], total[m], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __threadfence();
+    __syncthreads();
+    __shared__ int is_last;
+    if (t == 0) {
+        const unsigned prev = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (prev == (unsigned)(split_k - 1));
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    if (nt < N) {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float s = 0.f;
+            for (int sp = 0; sp < split_k; ++sp)
+                s += __hip_atomic_load(&partial[((size_t)sp * M + m) * N + nt], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            out[(size_t)m * N + nt] = (half_t)s;
+        }
+    }
+    if (t == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- host side -----------------------------------------------------------------------
+
+struct GemvPlan {
+    int rows;            // packed rows per step (template ROWS)
+    int col_tiles;
+    int split_k;
+    int steps_total;
+    int steps_per_wave;
+};
+
+static int env_int(const char* name, int fallback) {
+    const char* v = getenv(name);
+    if (!v || !*v) return fallback;
+    return atoi(v);
+}
+
+GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
+    const int P = 32 / bits;
+    const int rows_per_group = group_size / P;
+    GemvPlan p;
+    p.rows = (rows_per_group % 8 == 0) ? 8 : (rows_per_group % 4 == 0) ? 4 : 1;
+    p.col_tiles = (N + kGemvCols - 1) / kGemvCols;
+    p.steps_total = (K / P) / p.rows;
+    // Enough waves to keep every SIMD busy with several loads in flight.
+    static const int waves_per_cu = env_int("MH_GEMV_WAVES_PER_CU", 16);
+    const long target_waves = (long)compute_units() * waves_per_cu;
+    long split = target_waves / ((long)p.col_tiles * kGemvWaves);
+    const long max_split = (p.steps_total + kGemvWaves - 1) / kGemvWaves;
+    if (split > max_split) split = max_split;
+    if (split < 1) split = 1;
+    p.steps_per_wave = (int)((p.steps_total + split * kGemvWaves - 1) / (split * kGemvWaves));
+    p.split_k = (p.steps_total + p.steps_per_wave * kGemvWaves - 1) / (p.steps_per_wave * kGemvWaves);
+    return p;
+}
+
+size_t gemv_workspace_bytes(int M, int N, int K, int group_size, int bits) {
+    const GemvPlan p = plan_gemv(N, K, group_size, bits);
+    size_t counters = ((size_t)p.col_tiles * sizeof(unsigned) + 255) / 256 * 256;
+    size_t partial = (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
+    return counters + partial;
+}
+
+template <int BITS, int M, int ROWS>
+static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, const int32_t* qweight,
+                        const int32_t* qzeros, const void* scales, void* out, void* workspace,
+                        int N, int K, int group_size) {
+    constexpr int P = Packing<BITS>::kPerWord;
+    const size_t counters_bytes = ((size_t)p.col_tiles * sizeof(unsigned) + 255) / 256 * 256;
+    unsigned* counters = reinterpret_cast<unsigned*>(workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters_bytes);
+    hipLaunchKernelGGL((gptq_gemv_kernel<BITS, M, ROWS>), dim3(p.col_tiles, p.split_k), dim3(256), 0, stream,
+                       (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
+                       (const half_t*)scales, (half_t*)out, partial, counters, N, K, group_size / P,
+                       p.steps_total, p.steps_per_wave, p.split_k);
+}
+
+template <int BITS, int M>
+static void launch_gemv_rows(hipStream_t stream, const GemvPlan& p, const void* x, const int32_t* qweight,
+                             const int32_t* qzeros, const void* scales, void* out, void* workspace,
+                             int N, int K, int group_size) {
+    switch (p.rows) {
+        case 8: launch_gemv<BITS, M, 8>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+        case 4: launch_gemv<BITS, M, 4>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+        default: launch_gemv<BITS, M, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+    }
+}
+
+template <int BITS>
+static void launch_gemv_m(hipStream_t stream, const GemvPlan& p, const void* x, const int32_t* qweight,
+                          const int32_t* qzeros, const void* scales, void* out, void* workspace,
+                          int M, int N, int K, int group_size) {
+    switch (M) {
+        case 1: launch_gemv_rows<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+        case 2: launch_gemv_rows<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+        case 3: launch_gemv_rows<BITS, 3>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+        default: launch_gemv_rows<BITS, 4>(stream, p, x, qweight, qzeros, scales, out, workspace, N, K, group_size); break;
+    }
+}
+
+// Fast-path shape contract beyond check_gptq_args.
+bool gemv_supported(int M, int N, int K, int group_size, int bits) {
+    const int P = 32 / bits;
+    return M >= 1 && M <= MH_GPTQ_GEMV_MAX_M && (bits == 4 || bits == 8) && group_size % P == 0 &&
+           K % group_size == 0 && N % 8 == 0;
+}
+
+int gptq_gemv_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                     const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                     void* workspace, size_t workspace_bytes) {
+    const GemvPlan p = plan_gemv(N, K, group_size, bits);
+    const size_t need = gemv_workspace_bytes(M, N, K, group_size, bits);
+    if (p.split_k > 1) {
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemv: workspace of %zu bytes required, got %zu", need,
+                        workspace ? workspace_bytes : (size_t)0);
+        if ((uintptr_t)workspace % 256 != 0)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemv: workspace must be 256-byte aligned");
+    }
+    if (bits == 4)
+        launch_gemv_m<4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+    else
+        launch_gemv_m<8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+}  // namespace mh

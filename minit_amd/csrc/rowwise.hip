@@ -1,0 +1,469 @@
+// RMSNorm, softmax (+ fused causal mask), row reductions, RoPE and SiLU*up.
+//
+// All of these are HBM-bound: one pass over the data where the row fits in
+// registers, 16-byte loads, wave64 shuffle reductions (common.h), one row per
+// workgroup so a launch has as many workgroups as rows.  The view convention is
+// the reference's: a tensor is seen as [a, b, c] and the operation runs along b
+// (minit/cuda/dispatch.py:430-478).  c == 1 with 16-bit data takes the
+// vectorised path; anything else takes the strided path.
+#include "common.h"
+
+namespace mh {
+
+constexpr int kRowThreads = 256;
+constexpr int kRowVec = 8;        // 16-bit elements per 16-byte load
+constexpr int kRowMaxChunks = 4;  // register-resident rows: b <= 256 * 8 * 4 = 8192
+
+template <typename T> struct Vec8 { uint4 raw; };
+
+template <typename T>
+__device__ __forceinline__ void unpack8(const uint4& raw, float* f) {
+    const T* p = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = Cvt<T>::to_f32(p[i]);
+}
+
+template <typename T>
+__device__ __forceinline__ uint4 pack8(const float* f) {
+    uint4 raw;
+    T* p = reinterpret_cast<T*>(&raw);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) p[i] = Cvt<T>::from_f32(f[i]);
+    return raw;
+}
+
+// ---- RMSNorm ------------------------------------------------------------------------------
+// out = T( x / sqrt(sum(x^2)/b + eps) * w ), fp32 inside
+// (minit/cuda/kernel/cuda/rms_norm.py:69-89).
+
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
+    const T* __restrict__ in, const T* __restrict__ weight, T* __restrict__ out, size_t b, float eps) {
+    __shared__ float smem[16];
+    const size_t row = blockIdx.x;
+    const uint4* src = reinterpret_cast<const uint4*>(in + row * b);
+    const uint4* wsrc = reinterpret_cast<const uint4*>(weight);
+    uint4* dst = reinterpret_cast<uint4*>(out + row * b);
+    const int nvec = (int)(b / kRowVec);
+    uint4 regs[kRowMaxChunks];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < kRowMaxChunks; ++c) {
+        const int v = c * kRowThreads + threadIdx.x;
+        if (v < nvec) {
+            regs[c] = src[v];
+            float f[8];
+            unpack8<T>(regs[c], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += f[i] * f[i];
+        }
+    }
+    ss = block_sum(ss, smem);
+    const float rms = sqrtf(ss / (float)b + eps);
+#pragma unroll
+    for (int c = 0; c < kRowMaxChunks; ++c) {
+        const int v = c * kRowThreads + threadIdx.x;
+        if (v < nvec) {
+            float f[8], w[8];
+            unpack8<T>(regs[c], f);
+            const uint4 wr = wsrc[v];
+            unpack8<T>(wr, w);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = f[i] / rms * w[i];
+            dst[v] = pack8<T>(f);
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_strided_kernel(
+    const T* __restrict__ in, const T* __restrict__ weight, T* __restrict__ out,
+    size_t a, size_t b, size_t c, float eps) {
+    __shared__ float smem[16];
+    const size_t lines = a * c;
+    for (size_t line = blockIdx.x; line < lines; line += gridDim.x) {
+        const size_t base = (line / c) * b * c + line % c;
+        float ss = 0.f;
+        for (size_t j = threadIdx.x; j < b; j += blockDim.x) {
+            const float v = Cvt<T>::to_f32(in[base + j * c]);
+            ss += v * v;
+        }
+        ss = block_sum(ss, smem);
+        const float rms = sqrtf(ss / (float)b + eps);
+        for (size_t j = threadIdx.x; j < b; j += blockDim.x) {
+            const float v = Cvt<T>::to_f32(in[base + j * c]);
+            out[base + j * c] = Cvt<T>::from_f32(v / rms * Cvt<T>::to_f32(weight[j]));
+        }
+    }
+}
+
+// ---- softmax --------------------------------------------------------------------------------
+// p = exp(x - max) / sum(exp(x - max)), fp32 inside
+// (minit/cuda/kernel/cuda/softmax.py:71-105).  The causal variant applies the
+// models' scale and additive mask first (examples/llama3_70b.py:102-111): the
+// scaled score is rounded to T as the separate divide kernel would, and
+// positions j > offset + i contribute exp(-inf) = 0.
+
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
+    const T* __restrict__ in, T* __restrict__ out, size_t b, size_t s, size_t offset, float scale) {
+    __shared__ float smem[16];
+    const size_t row = blockIdx.x;
+    const uint4* src = reinterpret_cast<const uint4*>(in + row * b);
+    uint4* dst = reinterpret_cast<uint4*>(out + row * b);
+    const int nvec = (int)(b / kRowVec);
+    const long limit = CAUSAL ? (long)(offset + row % s) : (long)b;  // last visible column
+    float vals[kRowMaxChunks][8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < kRowMaxChunks; ++c) {
+        const int v = c * kRowThreads + threadIdx.x;
+        if (v < nvec) {
+            const uint4 raw = src[v];
+            unpack8<T>(raw, vals[c]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (CAUSAL) {
+                    float x = vals[c][i];
+                    if (scale != 1.f) x = Cvt<T>::to_f32(Cvt<T>::from_f32(x * scale));
+                    if ((long)v * 8 + i > limit) x = -INFINITY;
+                    vals[c][i] = x;
+                }
+                mx = fmaxf(mx, vals[c][i]);
+            }
+        }
+    }
+    mx = block_max(mx, smem);
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < kRowMaxChunks; ++c) {
+        const int v = c * kRowThreads + threadIdx.x;
+        if (v < nvec) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                vals[c][i] = expf(vals[c][i] - mx);
+                sum += vals[c][i];
+            }
+        }
+    }
+    sum = block_sum(sum, smem);
+#pragma unroll
+    for (int c = 0; c < kRowMaxChunks; ++c) {
+        const int v = c * kRowThreads + threadIdx.x;
+        if (v < nvec) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vals[c][i] = vals[c][i] / sum;
+            dst[v] = pack8<T>(vals[c]);
+        }
+    }
+}
+
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(kRowThreads) void softmax_strided_kernel(
+    const T* __restrict__ in, T* __restrict__ out, size_t a, size_t b, size_t c, size_t s, size_t offset,
+    float scale) {
+    __shared__ float smem[16];
+    const size_t lines = a * c;
+    for (size_t line = blockIdx.x; line < lines; line += gridDim.x) {
+        const size_t base = (line / c) * b * c + line % c;
+        const long limit = CAUSAL ? (long)(offset + line % s) : (long)b;
+        auto fetch = [&](size_t j) {
+            float x = Cvt<T>::to_f32(in[base + j * c]);
+            if (CAUSAL) {
+                if (scale != 1.f) x = Cvt<T>::to_f32(Cvt<T>::from_f32(x * scale));
+                if ((long)j > limit) x = -INFINITY;
+            }
+            return x;
+        };
+        float mx = -INFINITY;
+        for (size_t j = threadIdx.x; j < b; j += blockDim.x) mx = fmaxf(mx, fetch(j));
+        mx = block_max(mx, smem);
+        float sum = 0.f;
+        for (size_t j = threadIdx.x; j < b; j += blockDim.x) sum += expf(fetch(j) - mx);
+        sum = block_sum(sum, smem);
+        for (size_t j = threadIdx.x; j < b; j += blockDim.x)
+            out[base + j * c] = Cvt<T>::from_f32(expf(fetch(j) - mx) / sum);
+    }
+}
+
+// ---- reductions -------------------------------------------------------------------------------
+// [a, b, c] -> [a, 1, c], fp32 accumulate, cast at the store
+// (minit/cuda/kernel/cuda/reduce.py:76-92).
+
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kRowThreads) void reduce_rows_kernel(const T* __restrict__ in,
+                                                                 T* __restrict__ out, size_t b) {
+    __shared__ float smem[16];
+    const size_t row = blockIdx.x;
+    const T* src = in + row * b;
+    float acc = IS_MAX ? -INFINITY : 0.f;
+    const size_t nvec = (sizeof(T) == 2 && (uintptr_t)src % 16 == 0) ? b / kRowVec : 0;
+    const uint4* vsrc = reinterpret_cast<const uint4*>(src);
+    for (size_t v = threadIdx.x; v < nvec; v += blockDim.x) {
+        float f[8];
+        const uint4 raw = vsrc[v];
+        unpack8<T>(raw, f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = IS_MAX ? fmaxf(acc, f[i]) : acc + f[i];
+    }
+    for (size_t j = nvec * kRowVec + threadIdx.x; j < b; j += blockDim.x) {
+        const float f = Cvt<T>::to_f32(src[j]);
+        acc = IS_MAX ? fmaxf(acc, f) : acc + f;
+    }
+    acc = IS_MAX ? block_max(acc, smem) : block_sum(acc, smem);
+    if (threadIdx.x == 0) out[row] = Cvt<T>::from_f32(acc);
+}
+
+// c > 1: one thread per output element, coalesced across c.
+template <typename T, bool IS_MAX>
+__global__ void reduce_strided_kernel(const T* __restrict__ in, T* __restrict__ out, size_t a, size_t b,
+                                      size_t c) {
+    const size_t total = a * c;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const size_t base = (idx / c) * b * c + idx % c;
+        float acc = IS_MAX ? -INFINITY : 0.f;
+        for (size_t j = 0; j < b; ++j) {
+            const float f = Cvt<T>::to_f32(in[base + j * c]);
+            acc = IS_MAX ? fmaxf(acc, f) : acc + f;
+        }
+        out[idx] = Cvt<T>::from_f32(acc);
+    }
+}
+
+// ---- RoPE ----------------------------------------------------------------------------------------
+// o[2i] = x[2i] c - x[2i+1] s ; o[2i+1] = x[2i+1] c + x[2i] s, fp32 math, one
+// rounding (minit/cuda/kernel/cuda/rope.py:58-73).  One thread per complex pair.
+
+template <typename T>
+__global__ void rope_kernel(const T* __restrict__ in, const float* __restrict__ freqs_cos,
+                            const float* __restrict__ freqs_sin, const int32_t* __restrict__ positions,
+                            T* __restrict__ out, size_t bs, size_t seq, size_t nh, size_t half) {
+    const size_t total = bs * seq * nh * half;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const size_t i = idx % half;
+        const size_t bsq = idx / (half * nh);  // b * seq + s
+        const size_t pos = positions ? (size_t)positions[bsq] : bsq % seq;
+        const float c = freqs_cos[pos * half + i], s = freqs_sin[pos * half + i];
+        const float re = Cvt<T>::to_f32(in[idx * 2]), im = Cvt<T>::to_f32(in[idx * 2 + 1]);
+        out[idx * 2] = Cvt<T>::from_f32(re * c - im * s);
+        out[idx * 2 + 1] = Cvt<T>::from_f32(im * c + re * s);
+    }
+}
+
+// 16-bit fast path: one thread per four pairs (16 bytes of x, 16 bytes of each table).
+template <typename T>
+__global__ void rope_vec_kernel(const T* __restrict__ in, const float* __restrict__ freqs_cos,
+                                const float* __restrict__ freqs_sin, const int32_t* __restrict__ positions,
+                                T* __restrict__ out, size_t bs, size_t seq, size_t nh, size_t half) {
+    const size_t quads = half / 4;
+    const size_t total = bs * seq * nh * quads;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const size_t qd = idx % quads;
+        const size_t bsq = idx / (quads * nh);
+        const size_t pos = positions ? (size_t)positions[bsq] : bsq % seq;
+        const float4 c = *reinterpret_cast<const float4*>(freqs_cos + pos * half + qd * 4);
+        const float4 s = *reinterpret_cast<const float4*>(freqs_sin + pos * half + qd * 4);
+        const uint4 raw = reinterpret_cast<const uint4*>(in)[idx];
+        float f[8], o[8];
+        unpack8<T>(raw, f);
+        const float cs[4] = {c.x, c.y, c.z, c.w}, sn[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            o[2 * p] = f[2 * p] * cs[p] - f[2 * p + 1] * sn[p];
+            o[2 * p + 1] = f[2 * p + 1] * cs[p] + f[2 * p] * sn[p];
+        }
+        reinterpret_cast<uint4*>(out)[idx] = pack8<T>(o);
+    }
+}
+
+// ---- SiLU(gate) * up ---------------------------------------------------------------------------------
+// EXACT reproduces the three launches of the reference (sigmoid rounded to T,
+// T multiply, T multiply: minit/cuda/dispatch.py:137,143); otherwise fp32 until
+// the store.
+
+template <typename T, bool EXACT>
+__device__ __forceinline__ float silu_mul_one(float g, float u) {
+    if (EXACT) {
+        const float sig = Cvt<T>::to_f32(Cvt<T>::from_f32((float)(1.0 / (1.0 + (double)expf(-g)))));
+        const float a = Cvt<T>::to_f32(Cvt<T>::from_f32(g * sig));
+        return a * u;
+    }
+    return g / (1.f + expf(-g)) * u;
+}
+
+template <typename T, bool EXACT>
+__global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up, T* __restrict__ out,
+                                size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const bool aligned = (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)out) % 16 == 0) && sizeof(T) == 2;
+    const size_t nvec = aligned ? n / 8 : 0;
+    for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
+        float g[8], u[8];
+        const uint4 graw = reinterpret_cast<const uint4*>(gate)[v];
+        const uint4 uraw = reinterpret_cast<const uint4*>(up)[v];
+        unpack8<T>(graw, g);
+        unpack8<T>(uraw, u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) g[i] = silu_mul_one<T, EXACT>(g[i], u[i]);
+        reinterpret_cast<uint4*>(out)[v] = pack8<T>(g);
+    }
+    for (size_t j = nvec * 8 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += stride)
+        out[j] = Cvt<T>::from_f32(silu_mul_one<T, EXACT>(Cvt<T>::to_f32(gate[j]), Cvt<T>::to_f32(up[j])));
+}
+
+static unsigned grid_for(size_t work_items, int per_block) {
+    size_t blocks = (work_items + per_block - 1) / per_block;
+    const size_t cap = (size_t)compute_units() * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (unsigned)blocks;
+}
+
+static bool rows_fast_path(const void* in, const void* out, size_t b, size_t c, size_t elem) {
+    return c == 1 && elem == 2 && b % kRowVec == 0 && b <= (size_t)kRowThreads * kRowVec * kRowMaxChunks &&
+           ((uintptr_t)in | (uintptr_t)out) % 16 == 0;
+}
+
+template <typename T>
+static int rms_norm_t(hipStream_t st, const void* in, const void* weight, void* out, size_t a, size_t b,
+                      size_t c, float eps) {
+    if (rows_fast_path(in, out, b, c, sizeof(T)) && (uintptr_t)weight % 16 == 0) {
+        hipLaunchKernelGGL(rms_norm_rows_kernel<T>, dim3((unsigned)a), dim3(kRowThreads), 0, st, (const T*)in,
+                           (const T*)weight, (T*)out, b, eps);
+    } else {
+        hipLaunchKernelGGL(rms_norm_strided_kernel<T>, dim3(grid_for(a * c, 1)), dim3(kRowThreads), 0, st,
+                           (const T*)in, (const T*)weight, (T*)out, a, b, c, eps);
+    }
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+template <typename T, bool CAUSAL>
+static int softmax_t(hipStream_t st, const void* in, void* out, size_t a, size_t b, size_t c, size_t s,
+                     size_t offset, float scale) {
+    if (rows_fast_path(in, out, b, c, sizeof(T))) {
+        hipLaunchKernelGGL((softmax_rows_kernel<T, CAUSAL>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
+                           (const T*)in, (T*)out, b, s, offset, scale);
+    } else {
+        hipLaunchKernelGGL((softmax_strided_kernel<T, CAUSAL>), dim3(grid_for(a * c, 1)), dim3(kRowThreads), 0,
+                           st, (const T*)in, (T*)out, a, b, c, s, offset, scale);
+    }
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+template <typename T, bool IS_MAX>
+static int reduce_t(hipStream_t st, const void* in, void* out, size_t a, size_t b, size_t c) {
+    if (c == 1) {
+        hipLaunchKernelGGL((reduce_rows_kernel<T, IS_MAX>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
+                           (const T*)in, (T*)out, b);
+    } else {
+        hipLaunchKernelGGL((reduce_strided_kernel<T, IS_MAX>), dim3(grid_for(a * c, 256)), dim3(256), 0, st,
+                           (const T*)in, (T*)out, a, b, c);
+    }
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+}  // namespace mh
+
+using namespace mh;
+
+#define MH_DISPATCH_DTYPE(dtype, who, CALL)                                         \
+    switch (dtype) {                                                                \
+        case MH_F16: { typedef half_t T; CALL; }                                    \
+        case MH_BF16: { typedef __hip_bfloat16 T; CALL; }                           \
+        case MH_F32: { typedef float T; CALL; }                                     \
+        default: return fail(MH_ERR_INVALID, who ": unknown dtype %d", dtype);      \
+    }
+
+extern "C" {
+
+int mh_rms_norm(mh_stream_t stream, const void* in, const void* weight, void* out, size_t a, size_t b,
+                size_t c, double eps, int dtype) {
+    if (a * b * c == 0) return MH_OK;
+    MH_REQUIRE(in && weight && out, "mh_rms_norm: null pointer");
+    MH_REQUIRE(a <= 0x7fffffffu, "mh_rms_norm: too many rows");
+    MH_DISPATCH_DTYPE(dtype, "mh_rms_norm",
+                      return rms_norm_t<T>(as_stream(stream), in, weight, out, a, b, c, (float)eps));
+}
+
+int mh_softmax(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype) {
+    if (a * b * c == 0) return MH_OK;
+    MH_REQUIRE(in && out, "mh_softmax: null pointer");
+    MH_REQUIRE(a <= 0x7fffffffu, "mh_softmax: too many rows");
+    MH_DISPATCH_DTYPE(dtype, "mh_softmax",
+                      return (softmax_t<T, false>(as_stream(stream), in, out, a, b, c, 1, 0, 1.f)));
+}
+
+int mh_softmax_causal(mh_stream_t stream, const void* in, void* out, size_t rows_outer, size_t s, size_t t,
+                      size_t offset, float scale, int dtype) {
+    if (rows_outer * s * t == 0) return MH_OK;
+    MH_REQUIRE(in && out, "mh_softmax_causal: null pointer");
+    MH_REQUIRE(t == offset + s, "mh_softmax_causal: t=%zu must equal offset=%zu + s=%zu", t, offset, s);
+    MH_REQUIRE(rows_outer * s <= 0x7fffffffu, "mh_softmax_causal: too many rows");
+    MH_DISPATCH_DTYPE(dtype, "mh_softmax_causal",
+                      return (softmax_t<T, true>(as_stream(stream), in, out, rows_outer * s, t, 1, s, offset, scale)));
+}
+
+int mh_sum(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype) {
+    if (a * c == 0) return MH_OK;
+    MH_REQUIRE(in && out, "mh_sum: null pointer");
+    MH_REQUIRE(a <= 0x7fffffffu, "mh_sum: too many rows");
+    MH_DISPATCH_DTYPE(dtype, "mh_sum", return (reduce_t<T, false>(as_stream(stream), in, out, a, b, c)));
+}
+
+int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype) {
+    if (a * c == 0) return MH_OK;
+    MH_REQUIRE(in && out, "mh_max: null pointer");
+    MH_REQUIRE(a <= 0x7fffffffu, "mh_max: too many rows");
+    MH_DISPATCH_DTYPE(dtype, "mh_max", return (reduce_t<T, true>(as_stream(stream), in, out, a, b, c)));
+}
+
+int mh_rope(mh_stream_t stream, const void* in, const float* freqs_cos, const float* freqs_sin,
+            const int32_t* positions, void* out, size_t bs, size_t seq, size_t nh, size_t hs, int dtype) {
+    if (bs * seq * nh * hs == 0) return MH_OK;
+    MH_REQUIRE(in && out && freqs_cos && freqs_sin, "mh_rope: null pointer");
+    MH_REQUIRE(hs % 2 == 0, "mh_rope: head size %zu must be even", hs);
+    const size_t half = hs / 2;
+    hipStream_t st = as_stream(stream);
+    const bool vec = dtype != MH_F32 && half % 4 == 0 &&
+                     (((uintptr_t)in | (uintptr_t)out | (uintptr_t)freqs_cos | (uintptr_t)freqs_sin) % 16 == 0);
+    const size_t items = bs * seq * nh * (vec ? half / 4 : half);
+    const unsigned grid = grid_for(items, 256);
+#define MH_ROPE_CALL                                                                                         \
+    if (vec)                                                                                                 \
+        hipLaunchKernelGGL(rope_vec_kernel<T>, dim3(grid), dim3(256), 0, st, (const T*)in, freqs_cos,        \
+                           freqs_sin, positions, (T*)out, bs, seq, nh, half);                                \
+    else                                                                                                     \
+        hipLaunchKernelGGL(rope_kernel<T>, dim3(grid), dim3(256), 0, st, (const T*)in, freqs_cos, freqs_sin, \
+                           positions, (T*)out, bs, seq, nh, half);                                           \
+    MH_CHECK_LAUNCH();                                                                                       \
+    return MH_OK;
+    MH_DISPATCH_DTYPE(dtype, "mh_rope", MH_ROPE_CALL);
+#undef MH_ROPE_CALL
+}
+
+int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out, size_t n, int exact,
+                int dtype) {
+    if (n == 0) return MH_OK;
+    MH_REQUIRE(gate && up && out, "mh_silu_mul: null pointer");
+    hipStream_t st = as_stream(stream);
+    const unsigned grid = grid_for(n / 8 + 1, 256);
+#define MH_SILU_CALL                                                                                  \
+    if (exact)                                                                                        \
+        hipLaunchKernelGGL((silu_mul_kernel<T, true>), dim3(grid), dim3(256), 0, st, (const T*)gate,  \
+                           (const T*)up, (T*)out, n);                                                 \
+    else                                                                                              \
+        hipLaunchKernelGGL((silu_mul_kernel<T, false>), dim3(grid), dim3(256), 0, st, (const T*)gate, \
+                           (const T*)up, (T*)out, n);                                                 \
+    MH_CHECK_LAUNCH();                                                                                \
+    return MH_OK;
+    MH_DISPATCH_DTYPE(dtype, "mh_silu_mul", MH_SILU_CALL);
+#undef MH_SILU_CALL
+}
+
+}  // extern "C"

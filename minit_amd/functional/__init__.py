@@ -1,0 +1,3 @@
+from .linalg import matrix_multiply
+from .reduce import max, sum
+from .special import rms_norm, rope, softmax

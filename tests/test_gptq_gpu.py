@@ -1,0 +1,198 @@
+"""GPU parity: GPTQ unpack / dequantize / quantized linear against the oracle.
+
+Integer work (unpack) and the dequantized matrix are bit-exact; products are
+within the fp16 tolerance stated in ``helpers.py``.  One-hot activations turn
+the product kernels into exact row-pickers of the dequantized matrix, which
+pins their k-ordering bit for bit.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from helpers import assert_fp16_close
+from oracle import gptq as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(hip, arr):
+    from minit_amd.hip.tensor import HIPTensor
+    return HIPTensor.from_numpy(np.ascontiguousarray(arr))
+
+
+def _weights(k, n, group_size, bits, seed, zero_range=(6, 9)):
+    from minit_amd import synthetic
+    return synthetic.gptq_weights(f"test{seed}", "w", k, n, group_size, bits, zero_range)
+
+
+def _run_linear(hip, entry, x, qweight, qzeros, scales, group_size, bits, g_idx=None):
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    m, k = x.shape
+    n = qweight.shape[1]
+    dx, dq, dz, ds = _dev(hip, x), _dev(hip, qweight), _dev(hip, qzeros), _dev(hip, scales)
+    dg = None if g_idx is None else _dev(hip, g_idx.astype(np.int32))
+    out = HIPTensor.allocate((m, n), "float16")
+    nbytes = hip.call("mh_gptq_workspace_bytes", m, n, k, group_size, bits)
+    ws = memory.workspace(max(nbytes, 256))
+    hip.call(entry, None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr,
+             None if dg is None else dg.data_ptr, out.data_ptr, m, n, k, group_size, bits,
+             ws._pointer, ws._size)
+    return out.numpy()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_unpack_bit_exact(hip, bits, axis):
+    from minit_amd.hip.tensor import HIPTensor
+    rng = np.random.default_rng(bits * 10 + axis)
+    packed = rng.integers(-2**31, 2**31, size=(37, 53), dtype=np.int64).astype(np.int32)
+    per_word = 32 // bits
+    shape = (37 * per_word, 53) if axis == 0 else (37, 53 * per_word)
+    out = HIPTensor.allocate(shape, "uint8")
+    hip.call("mh_gptq_unpack", None, _dev(hip, packed).data_ptr, out.data_ptr, 37, 53, axis, bits)
+    np.testing.assert_array_equal(out.numpy(), O.unpack(packed, axis, bits))
+
+
+@pytest.mark.parametrize("k,n,group_size,bits", [
+    (4096, 4096, 128, 4),     # config 0
+    (256, 136, 32, 4),        # N not a multiple of the column tile
+    (512, 64, 64, 8),         # the reference's own 8-bit layout
+    (384, 72, 128, 4),
+])
+def test_dequant_bit_exact(hip, k, n, group_size, bits):
+    from minit_amd.hip.tensor import HIPTensor
+    qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=1, zero_range=(0, (1 << bits) - 1))
+    out = HIPTensor.allocate((k, n), "float16")
+    hip.call("mh_gptq_dequant", None, _dev(hip, qweight).data_ptr, _dev(hip, qzeros).data_ptr,
+             _dev(hip, scales).data_ptr, None, out.data_ptr, n, k, group_size, bits)
+    ref = O.dequantize_packed(qweight, qzeros, scales, None, bits, group_size)
+    np.testing.assert_array_equal(out.numpy().view(np.uint16), ref.view(np.uint16))
+
+
+def test_dequant_act_order_bit_exact(hip):
+    from minit_amd.hip.tensor import HIPTensor
+    k, n, g = 512, 128, 128
+    qweight, qzeros, scales = _weights(k, n, g, 4, seed=2)
+    g_idx = np.random.default_rng(3).permutation(k).astype(np.int32) // g
+    out = HIPTensor.allocate((k, n), "float16")
+    hip.call("mh_gptq_dequant", None, _dev(hip, qweight).data_ptr, _dev(hip, qzeros).data_ptr,
+             _dev(hip, scales).data_ptr, _dev(hip, g_idx).data_ptr, out.data_ptr, n, k, g, 4)
+    ref = O.dequantize_packed(qweight, qzeros, scales, g_idx, 4)
+    np.testing.assert_array_equal(out.numpy().view(np.uint16), ref.view(np.uint16))
+
+
+LINEAR_SHAPES = [
+    # m, k, n, group_size, bits
+    (1, 4096, 4096, 128, 4),    # config 0
+    (2, 1024, 520, 128, 4),     # ragged N
+    (3, 768, 256, 64, 4),
+    (4, 512, 1032, 32, 4),
+    (1, 1024, 256, 128, 8),
+    (4, 512, 264, 64, 8),
+]
+
+
+@pytest.mark.parametrize("m,k,n,group_size,bits", LINEAR_SHAPES)
+def test_gemv_matches_oracle(hip, m, k, n, group_size, bits):
+    from minit_amd import synthetic
+    qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=4)
+    x = synthetic.activations("test4", "x", (m, k))
+    got = _run_linear(hip, "mh_gptq_gemv", x, qweight, qzeros, scales, group_size, bits)
+    ref = O.matmul_f64(x, qweight, qzeros, scales, None, bits, group_size)
+    assert_fp16_close(got, ref, what=f"gemv {m}x{k}x{n}")
+
+
+@pytest.mark.parametrize("entry,m", [("mh_gptq_gemv", 1), ("mh_gptq_gemv", 4), ("mh_gptq_gemm", 1),
+                                     ("mh_gptq_gemm", 16), ("mh_gptq_gemm", 40)])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_one_hot_rows_are_exact(hip, entry, m, bits):
+    """x = e_k picks row k of dequant(W): any wrong k-ordering or zero/scale
+    indexing changes bits."""
+    k, n, g = 512, 520, 128
+    qweight, qzeros, scales = _weights(k, n, g, bits, seed=5, zero_range=(0, (1 << bits) - 1))
+    w = O.dequantize_packed(qweight, qzeros, scales, None, bits, g)
+    rows = np.random.default_rng(6).choice(k, size=m, replace=False)
+    x = np.zeros((m, k), dtype=np.float16)
+    x[np.arange(m), rows] = 1.0
+    got = _run_linear(hip, entry, x, qweight, qzeros, scales, g, bits)
+    np.testing.assert_array_equal(got.view(np.uint16), w[rows].view(np.uint16))
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 16, 17, 32, 64, 128, 200])
+def test_gemm_matches_oracle(hip, m):
+    from minit_amd import synthetic
+    k, n, g = 1024, 776, 128
+    qweight, qzeros, scales = _weights(k, n, g, 4, seed=7)
+    x = synthetic.activations("test7", f"x{m}", (m, k))
+    got = _run_linear(hip, "mh_gptq_gemm", x, qweight, qzeros, scales, g, 4)
+    ref = O.matmul_f64(x, qweight, qzeros, scales, None, 4, g)
+    assert_fp16_close(got, ref, what=f"gemm M={m}")
+
+
+@pytest.mark.parametrize("m,k,n,group_size,bits", [(8, 1536, 512, 64, 8), (33, 4096, 256, 32, 4)])
+def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
+    from minit_amd import synthetic
+    qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=8)
+    x = synthetic.activations("test8", "x", (m, k))
+    got = _run_linear(hip, "mh_gptq_gemm", x, qweight, qzeros, scales, group_size, bits)
+    ref = O.matmul_f64(x, qweight, qzeros, scales, None, bits, group_size)
+    assert_fp16_close(got, ref, what=f"gemm {m}x{k}x{n} b{bits}")
+
+
+def test_repeated_calls_are_deterministic(hip):
+    """Split-K partials are summed in a fixed order: bitwise repeatable, and the
+    arrival counters are left zeroed for the next call."""
+    from minit_amd import synthetic
+    k, n, g = 4096, 1024, 128
+    qweight, qzeros, scales = _weights(k, n, g, 4, seed=9)
+    for entry, m in (("mh_gptq_gemv", 2), ("mh_gptq_gemm", 24)):
+        x = synthetic.activations("test9", f"x{m}", (m, k))
+        first = _run_linear(hip, entry, x, qweight, qzeros, scales, g, 4)
+        for _ in range(3):
+            again = _run_linear(hip, entry, x, qweight, qzeros, scales, g, 4)
+            np.testing.assert_array_equal(first.view(np.uint16), again.view(np.uint16))
+
+
+def test_act_order_through_matmul(hip):
+    from minit_amd import synthetic
+    m, k, n, g = 3, 512, 128, 128
+    qweight, qzeros, scales = _weights(k, n, g, 4, seed=10)
+    g_idx = np.random.default_rng(11).permutation(k).astype(np.int32) // g
+    x = synthetic.activations("test10", "x", (m, k))
+    got = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, 4, g_idx=g_idx)
+    ref = O.matmul_f64(x, qweight, qzeros, scales, g_idx, 4)
+    assert_fp16_close(got, ref, what="act-order")
+
+
+def test_bad_arguments_are_reported(hip):
+    from minit_amd.lib import HipError
+    with pytest.raises(HipError, match="bits"):
+        hip.call("mh_gptq_gemv", None, 256, 256, 256, 256, None, 256, 1, 64, 64, 32, 3, None, 0)
+    with pytest.raises(HipError, match="group_size"):
+        hip.call("mh_gptq_gemv", None, 256, 256, 256, 256, None, 256, 1, 64, 96, 64, 4, None, 0)
+    with pytest.raises(HipError, match="M <="):
+        hip.call("mh_gptq_gemv", None, 256, 256, 256, 256, None, 256, 9, 64, 128, 128, 4, None, 0)
+
+
+def test_operator_api_drop_in(hip):
+    """F.matrix_multiply(x, QuantizedTensor) with leading dims folded, and
+    QuantizedTensor.dequantize(), as the reference's callers use them."""
+    import minit_amd.functional as F
+    from minit_amd import synthetic
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.quantize.gptq import quantized_tensor_from_host
+    k, n, g = 1024, 512, 128
+    qweight, qzeros, scales = _weights(k, n, g, 4, seed=12)
+    g_idx = (np.arange(k) // g).astype(np.int32)
+    w = quantized_tensor_from_host(qweight, qzeros, scales, g_idx)
+    assert w._group is None and w.dtype == "quint4" and tuple(d.item() for d in w.shape) == (k, n)
+    x = synthetic.activations("test12", "x", (2, 3, k))
+    y = F.matrix_multiply(HIPTensor.from_numpy(x), w)
+    assert tuple(d.item() for d in y.shape) == (2, 3, n)
+    ref = O.matmul_f64(x.reshape(6, k), qweight, qzeros, scales, None, 4, g).reshape(2, 3, n)
+    assert_fp16_close(y.numpy(), ref, what="F.matrix_multiply")
+    wd = w.dequantize().numpy()
+    np.testing.assert_array_equal(wd.view(np.uint16),
+                                  O.dequantize_packed(qweight, qzeros, scales, None, 4, g).view(np.uint16))
