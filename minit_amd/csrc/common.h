@@ -86,6 +86,37 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
     return r;
 }
 
+// ---- cross-workgroup hand-off without device-wide cache flushes ---------------------
+// Split-K partial sums go from many workgroups to the one that finishes last.
+// A release/acquire fence pair at agent scope would do, but on a multi-XCD part
+// it writes back and invalidates a whole L2 per fence, once per workgroup.  The
+// data are instead moved with agent-scope relaxed atomic stores and loads, which
+// are written through to / fetched from the device-coherent level individually,
+// and ordered by hand: every thread waits until its stores are acknowledged
+// (s_waitcnt 0), the workgroup meets at a barrier, then one thread bumps the
+// arrival counter with an agent-scope atomic.
+__device__ __forceinline__ void store_agent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// True, in every thread, for the workgroup that arrives last of `expected`; that
+// workgroup also resets the counter for the next launch.  All threads of the
+// workgroup must call it.
+__device__ __forceinline__ bool arrive_and_check_last(unsigned* counter, unsigned expected, int* flag) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = prev == expected - 1;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = last;
+    }
+    __syncthreads();
+    return *flag != 0;
+}
+
 // 16-bit storage <-> fp32.
 template <typename T> struct Cvt;
 template <> struct Cvt<half_t> {

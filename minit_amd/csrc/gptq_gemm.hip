@@ -211,22 +211,13 @@ __global__ __launch_bounds__(256) void gptq_gemm_kernel(
                 if (m < M) {
                     float* p = partial + ((size_t)split * M + m) * N + col;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        __hip_atomic_store(p + t, acc[mt][t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int t = 0; t < 4; ++t) store_agent(p + t, acc[mt][t][r]);
                 }
             }
     }
-    __threadfence();
-    __syncthreads();
     __shared__ int is_last;
-    unsigned* counter = counters + (size_t)mblock * gridDim.x + tile;
-    if (tid == 0) {
-        const unsigned prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (prev == (unsigned)(split_k - 1));
-    }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
+    if (!arrive_and_check_last(counters + (size_t)mblock * gridDim.x + tile, (unsigned)split_k, &is_last))
+        return;
     if (active) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -235,18 +226,27 @@ __global__ __launch_bounds__(256) void gptq_gemm_kernel(
                 const int m = m0 + mt * 16 + kq * 4 + r;
                 if (m < M) {
                     float s[4] = {0.f, 0.f, 0.f, 0.f};
-                    for (int sp = 0; sp < split_k; ++sp) {
-                        const float* p = partial + ((size_t)sp * M + m) * N + col;
+                    const float* p = partial + (size_t)m * N + col;
+                    int sp = 0;
+                    for (; sp + 4 <= split_k; sp += 4) {
+                        float v[4][4];
 #pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            s[t] += __hip_atomic_load(p + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) v[u][t] = load_agent(p + (size_t)(sp + u) * M * N + t);
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) s[t] += v[u][t];
                     }
+                    for (; sp < split_k; ++sp)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) s[t] += load_agent(p + (size_t)sp * M * N + t);
                     const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
                 }
             }
     }
-    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- host side ---------------------------------------------------------------------------------------
@@ -278,7 +278,11 @@ GemmPlan plan_gemm(int M, int N, int K) {
     const long target_blocks = (long)compute_units() * blocks_per_cu;
     long split = target_blocks / ((long)p.col_tiles * p.m_blocks);
     // every block walks whole stages; partial sums cost 8*M*N bytes per split
-    const long max_split = (p.steps_total + sc - 1) / sc;
+    long max_split = (p.steps_total + sc - 1) / sc;
+    // fp32 partials cost 8*M*N bytes per split against K*N/2 bytes of weights:
+    // keep them under about a quarter of the weight traffic
+    const long traffic_cap = K / (64L * M) > 1 ? K / (64L * M) : 1;
+    if (max_split > traffic_cap) max_split = traffic_cap;
     if (split > max_split) split = max_split;
     if (split < 1) split = 1;
     long spb = (p.steps_total + split - 1) / split;

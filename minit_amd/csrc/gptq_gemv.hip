@@ -34,12 +34,35 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
     constexpr int PAIRS = Packing<BITS>::kPairs;
     constexpr uint32_t MASK = Packing<BITS>::kMask;
 
+    // activations of this block's K range, in pair order: [M][rows_blk * PAIRS] words
+    extern __shared__ uint32_t xs[];
+
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tile = blockIdx.x;
     const int split = blockIdx.y;
     const int n = tile * kGemvCols + lane * 4;
     const bool active = n < N;
+
+    const int rows_total = steps_total * ROWS;
+    const int rows_blk = kGemvWaves * steps_per_wave * ROWS;
+    const int row_base = split * rows_blk;
+    for (int idx = threadIdx.x; idx < rows_blk * M; idx += 256) {
+        const int m = idx / rows_blk, rl = idx % rows_blk;
+        const int row = row_base + rl;
+        uint32_t xv[PAIRS], xp[PAIRS];
+#pragma unroll
+        for (int p = 0; p < PAIRS; ++p) xv[p] = 0;
+        if (row < rows_total) {
+            const uint32_t* xr = reinterpret_cast<const uint32_t*>(x + (size_t)m * K + (size_t)row * P);
+#pragma unroll
+            for (int p = 0; p < PAIRS; ++p) xv[p] = xr[p];
+        }
+        pair_activations<BITS>(xv, xp);
+#pragma unroll
+        for (int p = 0; p < PAIRS; ++p) xs[(m * rows_blk + rl) * PAIRS + p] = xp[p];
+    }
+    __syncthreads();
 
     DequantRegs regs;
     regs.init(BITS);
@@ -77,18 +100,14 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
                 cc[3] = make_column_const(s23.y, (zword >> (3 * BITS)) & MASK);
             }
 
+            const int rl0 = row - row_base;
 #pragma unroll
             for (int i = 0; i < ROWS; ++i) {
                 uint32_t xp[M][PAIRS];
 #pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    const uint32_t* xr =
-                        reinterpret_cast<const uint32_t*>(x + (size_t)m * K + (size_t)(row + i) * P);
-                    uint32_t xv[PAIRS];
+                for (int m = 0; m < M; ++m)
 #pragma unroll
-                    for (int p = 0; p < PAIRS; ++p) xv[p] = xr[p];
-                    pair_activations<BITS>(xv, xp[m]);
-                }
+                    for (int p = 0; p < PAIRS; ++p) xp[m][p] = xs[(m * rows_blk + rl0 + i) * PAIRS + p];
                 const uint32_t qs[4] = {q[i].x, q[i].y, q[i].z, q[i].w};
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -126,35 +145,37 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
         return;
     }
 
-    // K-reduction across blocks: publish the partial, the last block to arrive
-    // for this column tile sums all of them in split order.
+    // K-reduction across blocks: publish the partial; the last block to arrive
+    // for this column tile sums all of them in split order (deterministic).
     if (nt < N) {
 #pragma unroll
-        for (int m = 0; m < M; ++m)
-            __hip_atomic_store(&partial[((size_t)split * M + m) * N + nt], total[m], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+        for (int m = 0; m < M; ++m) store_agent(&partial[((size_t)split * M + m) * N + nt], total[m]);
     }
-    __threadfence();
-    __syncthreads();
     __shared__ int is_last;
-    if (t == 0) {
-        const unsigned prev = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (prev == (unsigned)(split_k - 1));
-    }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
+    if (!arrive_and_check_last(&counters[tile], (unsigned)split_k, &is_last)) return;
     if (nt < N) {
+        float s[M];
 #pragma unroll
-        for (int m = 0; m < M; ++m) {
-            float s = 0.f;
-            for (int sp = 0; sp < split_k; ++sp)
-                s += __hip_atomic_load(&partial[((size_t)sp * M + m) * N + nt], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-            out[(size_t)m * N + nt] = (half_t)s;
+        for (int m = 0; m < M; ++m) s[m] = 0.f;
+        const float* p = partial + nt;
+        int sp = 0;
+        for (; sp + 8 <= split_k; sp += 8) {
+            float v[8][M];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int m = 0; m < M; ++m) v[u][m] = load_agent(p + ((size_t)(sp + u) * M + m) * N);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int m = 0; m < M; ++m) s[m] += v[u][m];
         }
+        for (; sp < split_k; ++sp)
+#pragma unroll
+            for (int m = 0; m < M; ++m) s[m] += load_agent(p + ((size_t)sp * M + m) * N);
+#pragma unroll
+        for (int m = 0; m < M; ++m) out[(size_t)m * N + nt] = (half_t)s[m];
     }
-    if (t == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- host side -----------------------------------------------------------------------
@@ -185,7 +206,11 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
     const long target_waves = (long)compute_units() * waves_per_cu;
     long split = target_waves / ((long)p.col_tiles * kGemvWaves);
     const long max_split = (p.steps_total + kGemvWaves - 1) / kGemvWaves;
+    // a block stages the activations of its K range in LDS: at most 512 packed rows
+    const long max_steps_per_wave = 512 / (kGemvWaves * p.rows);
+    const long min_split = (p.steps_total + kGemvWaves * max_steps_per_wave - 1) / (kGemvWaves * max_steps_per_wave);
     if (split > max_split) split = max_split;
+    if (split < min_split) split = min_split;
     if (split < 1) split = 1;
     p.steps_per_wave = (int)((p.steps_total + split * kGemvWaves - 1) / (split * kGemvWaves));
     p.split_k = (p.steps_total + p.steps_per_wave * kGemvWaves - 1) / (p.steps_per_wave * kGemvWaves);
@@ -207,7 +232,8 @@ static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, co
     const size_t counters_bytes = ((size_t)p.col_tiles * sizeof(unsigned) + 255) / 256 * 256;
     unsigned* counters = reinterpret_cast<unsigned*>(workspace);
     float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters_bytes);
-    hipLaunchKernelGGL((gptq_gemv_kernel<BITS, M, ROWS>), dim3(p.col_tiles, p.split_k), dim3(256), 0, stream,
+    const size_t lds = (size_t)M * kGemvWaves * p.steps_per_wave * ROWS * Packing<BITS>::kPairs * sizeof(uint32_t);
+    hipLaunchKernelGGL((gptq_gemv_kernel<BITS, M, ROWS>), dim3(p.col_tiles, p.split_k), dim3(256), lds, stream,
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, counters, N, K, group_size / P,
                        p.steps_total, p.steps_per_wave, p.split_k);
