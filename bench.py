@@ -1,0 +1,275 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+One *step* is one pass of the decode hot path over one layer's worth of
+Llama-3-70B-shape GPTQ 4-bit weights at M = 1: the four quantized linears
+(qkv 8192x10240, o 8192x8192, gate|up 8192x57344, down 28672x8192, group 128)
+through ``mh_gptq_gemv``.  ``--layers`` distinct weight sets (default 6,
+2.6 GB -- ten times the 256 MB Infinity Cache) are generated on the device and
+cycled, so every step streams its weights from HBM.  The value reported is
+algorithmic bytes per second: packed weights + scales + zero points +
+activations + outputs, each counted once.
+
+Prints ONE JSON line with the headline metric, its roofline fraction (HBM,
+8 TB/s) and the CPU baseline: the C restatement of the reference's arithmetic
+(``oracle/c``) timed on this machine's host cores on the same layer, whose
+result the GPU output is also checked against.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+INT8_PEAK_TOPS = 5000.0
+
+# (name, K, N) of the fused per-layer projections at Llama-3-70B shape
+HIDDEN, Q_HEADS, KV_HEADS, HEAD, FFN = 8192, 64, 8, 128, 28672
+LINEARS = [
+    ("qkv_proj", HIDDEN, (Q_HEADS + 2 * KV_HEADS) * HEAD),
+    ("o_proj", Q_HEADS * HEAD, HIDDEN),
+    ("gate_up_proj", HIDDEN, 2 * FFN),
+    ("down_proj", FFN, HIDDEN),
+]
+GROUP, BITS = 128, 4
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def linear_bytes(m, k, n, group=GROUP, bits=BITS):
+    """Algorithmic bytes of one quantized linear (every operand once)."""
+    groups = k // group
+    return k * n * bits // 8 + groups * n * 2 + groups * (n * bits // 32) * 4 + m * k * 2 + m * n * 2
+
+
+class DeviceLinear:
+    """One GPTQ weight set generated on the device."""
+
+    def __init__(self, lib, HIPTensor, k, n, seed):
+        per = 32 // BITS
+        groups = k // GROUP
+        self.k, self.n = k, n
+        self.qweight = HIPTensor.allocate((k // per, n), "int32")
+        self.qzeros = HIPTensor.allocate((groups, n // per), "int32")
+        self.scales = HIPTensor.allocate((groups, n), "float16")
+        lib.call("mh_synth_u32", None, self.qweight.data_ptr, (k // per) * n, seed * 3 + 0)
+        lib.call("mh_synth_subwords", None, self.qzeros.data_ptr, groups * (n // per), BITS, 6, 9, seed * 3 + 1)
+        lib.call("mh_synth_normal", None, self.scales.data_ptr, groups * n, 0.0, 0.02, 1, 1e-3, seed * 3 + 2, 0)
+
+
+def run_gemv(lib, x, lin, out, ws, m=1, entry="mh_gptq_gemv"):
+    lib.call(entry, None, x.data_ptr, lin.qweight.data_ptr, lin.qzeros.data_ptr, lin.scales.data_ptr, None,
+             out.data_ptr, m, lin.n, lin.k, GROUP, BITS, ws._pointer, ws._size)
+
+
+def bench_int8(lib, HIPTensor, memory, n, iters=20):
+    """W8A8 GEMM, M = 2048, K = 4096 (fp16 output + scale epilogue)."""
+    m, k = 2048, 4096
+    a = HIPTensor.allocate((m, k), "int8")
+    sa = HIPTensor.allocate((m,), "float32")
+    sw = HIPTensor.allocate((n,), "float32")
+    out = HIPTensor.allocate((m, n), "float16")
+    lib.call("mh_synth_i8", None, a.data_ptr, m * k, -127, 127, 11)
+    lib.call("mh_synth_normal", None, sa.data_ptr, m, 0.0, 0.01, 1, 0.0, 12, 2)
+    lib.call("mh_synth_normal", None, sw.data_ptr, n, 0.0, 0.005, 1, 0.0, 13, 2)
+    ws = []
+    for i in range(4):  # rotate weight buffers
+        w = HIPTensor.allocate((n, k), "int8")
+        lib.call("mh_synth_i8", None, w.data_ptr, n * k, -127, 127, 20 + i)
+        ws.append(w)
+
+    def go(i):
+        lib.call("mh_i8_gemm", None, a.data_ptr, ws[i % 4].data_ptr, sa.data_ptr, sw.data_ptr, out.data_ptr,
+                 None, m, n, k)
+    for i in range(3):
+        go(i)
+    memory.synchronize()
+    e0, e1 = memory.Event(), memory.Event()
+    e0.record()
+    for i in range(iters):
+        go(i)
+    e1.record()
+    e1.synchronize()
+    us = e0.elapsed_ms(e1) * 1e3 / iters
+    tops = 2.0 * m * n * k / us / 1e6
+    return {"M": m, "N": n, "K": k, "us": round(us, 2), "tops": round(tops, 1),
+            "frac_of_peak": round(tops / INT8_PEAK_TOPS, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=6, help="distinct weight sets cycled through")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+            "(no collectives or sharding in this path).")
+        sys.exit(2)
+
+    from minit_amd import lib
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+
+    lib.cdll()
+    if lib.device_count() < 1:
+        log("bench.py: no HIP device visible")
+        sys.exit(1)
+    info = lib.device_info()
+    log("device:", info)
+
+    # ---- inputs, resident in HBM before the timed region ------------------------------------
+    t0 = time.time()
+    layers = []
+    for layer in range(args.layers):
+        layers.append([DeviceLinear(lib, HIPTensor, k, n, 1000 * layer + j) for j, (_, k, n) in enumerate(LINEARS)])
+    xs, outs = {}, {}
+    for _, k, n in LINEARS:
+        if k not in xs:
+            xs[k] = HIPTensor.allocate((1, k), "float16")
+            lib.call("mh_synth_normal", None, xs[k].data_ptr, k, 0.0, 1.0, 0, 0.0, 7 + k, 0)
+        outs[n] = HIPTensor.allocate((1, n), "float16")
+    ws_bytes = max(lib.call("mh_gptq_workspace_bytes", 1, n, k, GROUP, BITS) for _, k, n in LINEARS)
+    ws = memory.workspace(max(ws_bytes, 256))
+    memory.synchronize()
+    weight_bytes = sum(linear_bytes(0, k, n) for _, k, n in LINEARS)
+    log(f"generated {args.layers} layers x {weight_bytes / 1e6:.1f} MB in {time.time() - t0:.1f} s")
+
+    def step(i):
+        for lin in layers[i % args.layers]:
+            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws)
+
+    for i in range(args.warmup):
+        step(i)
+    memory.synchronize()
+    e0, e1 = memory.Event(), memory.Event()
+    wall0 = time.perf_counter()
+    e0.record()                      # null stream: the stream the kernels run on
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    e1.synchronize()
+    memory.synchronize()
+    wall = time.perf_counter() - wall0
+    dev_ms = e0.elapsed_ms(e1)
+    ms_per_step = dev_ms / args.steps
+    step_bytes = sum(linear_bytes(1, k, n) for _, k, n in LINEARS)
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launches = args.steps * len(LINEARS)
+    log(f"{args.steps} steps: {dev_ms:.2f} ms on device ({wall * 1e3:.2f} ms wall), "
+        f"{ms_per_step * 1e3:.1f} us/step, {gbps:.0f} GB/s")
+
+    result = {
+        "metric": "w4a16_gemv_hbm_gbps",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "llama3-70b-shape GPTQ w4a16 decode GEMVs, M=1, group 128: qkv 8192x10240, "
+                        "o 8192x8192, gate_up 8192x57344, down 28672x8192; one step = one layer",
+            "layers_cycled": args.layers,
+            "bytes_per_step": step_bytes,
+            "device": info["name"].strip(),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gptq_gemv_kernel<4,1,8>",
+            "achieved": round(gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
+            "bytes_per_launch": step_bytes // len(LINEARS),
+            "traffic": None,
+        },
+    }
+
+    # ---- per-shape breakdown and the other metrics named by the baseline --------------------
+    if not args.no_extras:
+        per_shape = {}
+        for j, (name, k, n) in enumerate(LINEARS):
+            for i in range(3):
+                run_gemv(lib, xs[k], layers[i % args.layers][j], outs[n], ws)
+            memory.synchronize()
+            a, b = memory.Event(), memory.Event()
+            a.record()
+            for i in range(50):
+                run_gemv(lib, xs[k], layers[i % args.layers][j], outs[n], ws)
+            b.record()
+            b.synchronize()
+            us = a.elapsed_ms(b) * 1e3 / 50
+            per_shape[name] = {"us": round(us, 2), "gbps": round(linear_bytes(1, k, n) / us / 1e3, 1)}
+        result["extra"] = {"gemv_per_shape": per_shape}
+        try:
+            result["extra"]["int8_gemm"] = [bench_int8(lib, HIPTensor, memory, n) for n in (4096, 11008)]
+        except Exception as exc:  # report, do not hide
+            result["extra"]["int8_gemm_error"] = str(exc)
+        try:
+            from minit_amd import decode
+            result["extra"]["decode_70b"] = decode.bench_tokens_per_second(batches=(1,), tokens=16, log=log)
+        except Exception as exc:
+            result["extra"]["decode_70b_error"] = str(exc)
+
+    # ---- CPU baseline: the C restatement on this host's cores, same layer ---------------------
+    if not args.no_cpu_baseline:
+        from oracle import cport
+        cport.build()
+        threads = cport.threads()
+        host = []
+        for lin in layers[0]:
+            host.append((lin.qweight.numpy(), lin.qzeros.numpy(), lin.scales.numpy()))
+        hx = {k: t.numpy() for k, t in xs.items()}
+        # GPU results for layer 0, to check against what the CPU computes
+        gpu_out = []
+        for lin in layers[0]:
+            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws)
+            gpu_out.append(outs[lin.n].numpy().copy())
+        times, worst = [], 0.0
+        for rep in range(2):
+            t = time.perf_counter()
+            cpu_out = [cport.matmul(hx[lin.k], *h, None, BITS, GROUP) for lin, h in zip(layers[0], host)]
+            times.append(time.perf_counter() - t)
+        for g, c in zip(gpu_out, cpu_out):
+            d = np.abs(g.astype(np.float64) - c.astype(np.float64))
+            tol = np.maximum(1e-2, np.spacing(np.abs(c)).astype(np.float64))
+            worst = max(worst, float((d / tol).max()))
+        cpu_s = min(times)
+        result["cpu_baseline"] = {
+            "value": round(step_bytes / cpu_s / 1e9, 2),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"one layer (4 GEMVs, {step_bytes / 1e6:.0f} MB) x 2 runs, best of 2, "
+                      f"{cpu_s:.2f} s per run, OpenMP over output columns",
+            "gpu_vs_cpu_worst_err_over_tol": round(worst, 3),
+        }
+        log(f"cpu baseline: {cpu_s:.2f} s per layer on {threads} threads; "
+            f"GPU vs CPU worst error / tolerance = {worst:.3f}")
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

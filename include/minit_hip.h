@@ -188,6 +188,20 @@ int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, si
 int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
                 size_t n, int exact, int dtype);
 
+/* ---- synthetic inputs ------------------------------------------------------------------
+ * No counterpart in the reference (it loads checkpoints from disk,
+ * minit/module/checkpoint.py:11-44).  Counter-based generators that fill device
+ * buffers for benchmarks: uniform 32-bit words (= uniform 4-bit weights),
+ * sub-words uniform in [lo, hi] (zero points), N(mean, std) optionally folded
+ * and offset (scales, activations), uniform int8.
+ */
+int mh_synth_u32(mh_stream_t stream, uint32_t* out, size_t n, uint64_t seed);
+int mh_synth_subwords(mh_stream_t stream, uint32_t* out, size_t n, int bits, uint32_t lo, uint32_t hi,
+                      uint64_t seed);
+int mh_synth_normal(mh_stream_t stream, void* out, size_t n, float mean, float std, int take_abs,
+                    float offset, uint64_t seed, int dtype);
+int mh_synth_i8(mh_stream_t stream, int8_t* out, size_t n, int lo, int hi, uint64_t seed);
+
 #ifdef __cplusplus
 }
 #endif

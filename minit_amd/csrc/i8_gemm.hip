@@ -122,7 +122,12 @@ __global__ __launch_bounds__(256) void i8_gemm_kernel(
                 if (acc_out) acc_out[(size_t)m * N + n] = v;
                 if (out) {
                     const float s = (a_scale ? a_scale[m] : 1.f) * ws;
-                    out[(size_t)m * N + n] = (half_t)((float)v * s);
+                    // The product is rounded to fp32 and only then to fp16; the
+                    // empty asm keeps the compiler from fusing both into one
+                    // mixed-precision instruction that rounds once.
+                    float prod = (float)v * s;
+                    asm volatile("" : "+v"(prod));
+                    out[(size_t)m * N + n] = (half_t)prod;
                 }
             }
         }

@@ -8,7 +8,7 @@ There is no fallback: if the library is missing, loading raises.
 """
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_uint32, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libminit_hip.so")
@@ -58,6 +58,10 @@ PROTOTYPES = {
     "mh_sum": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_max": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
+    "mh_synth_u32": (c_int, [_P, _P, c_size_t, c_uint64]),
+    "mh_synth_subwords": (c_int, [_P, _P, c_size_t, c_int, c_uint32, c_uint32, c_uint64]),
+    "mh_synth_normal": (c_int, [_P, _P, c_size_t, c_float, c_float, c_int, c_float, c_uint64, c_int]),
+    "mh_synth_i8": (c_int, [_P, _P, c_size_t, c_int, c_int, c_uint64]),
 }
 
 # functions whose return value is not a status code

@@ -15,11 +15,22 @@ import numpy as np
 
 
 def gemm_i32(a_mk: np.ndarray, w_nk: np.ndarray) -> np.ndarray:
-    """Exact ``int32`` accumulators; |acc| <= 127^2 * K stays far below 2^31."""
+    """Exact ``int32`` accumulators; |acc| <= 128^2 * K stays far below 2^31.
+
+    Evaluated with a float64 library matmul: every product and partial sum is an
+    integer below 2^53, so float64 arithmetic is exact whatever the summation
+    order (numpy's integer matmul is not BLAS-backed and takes minutes at the
+    benchmark sizes).  Pinned against int64 and brute-force loops in the tests.
+    """
     assert a_mk.dtype == np.int8 and w_nk.dtype == np.int8
-    acc = a_mk.astype(np.int64) @ w_nk.astype(np.int64).T
-    assert np.abs(acc).max(initial=0) < 2 ** 31
-    return acc.astype(np.int32)
+    assert 128 * 128 * a_mk.shape[1] < 2 ** 31
+    acc = a_mk.astype(np.float64) @ w_nk.astype(np.float64).T
+    return acc.astype(np.int64).astype(np.int32)
+
+
+def gemm_i32_int64(a_mk: np.ndarray, w_nk: np.ndarray) -> np.ndarray:
+    """The same product in int64 integer arithmetic (slow; for pinning)."""
+    return (a_mk.astype(np.int64) @ w_nk.astype(np.int64).T).astype(np.int32)
 
 
 def gemm_i32_loops(a_mk: np.ndarray, w_nk: np.ndarray) -> np.ndarray:

@@ -51,7 +51,8 @@ def test_unpack_bit_exact(hip, bits, axis):
     per_word = 32 // bits
     shape = (37 * per_word, 53) if axis == 0 else (37, 53 * per_word)
     out = HIPTensor.allocate(shape, "uint8")
-    hip.call("mh_gptq_unpack", None, _dev(hip, packed).data_ptr, out.data_ptr, 37, 53, axis, bits)
+    dp = _dev(hip, packed)
+    hip.call("mh_gptq_unpack", None, dp.data_ptr, out.data_ptr, 37, 53, axis, bits)
     np.testing.assert_array_equal(out.numpy(), O.unpack(packed, axis, bits))
 
 
@@ -65,8 +66,9 @@ def test_dequant_bit_exact(hip, k, n, group_size, bits):
     from minit_amd.hip.tensor import HIPTensor
     qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=1, zero_range=(0, (1 << bits) - 1))
     out = HIPTensor.allocate((k, n), "float16")
-    hip.call("mh_gptq_dequant", None, _dev(hip, qweight).data_ptr, _dev(hip, qzeros).data_ptr,
-             _dev(hip, scales).data_ptr, None, out.data_ptr, n, k, group_size, bits)
+    dq, dz, ds = _dev(hip, qweight), _dev(hip, qzeros), _dev(hip, scales)
+    hip.call("mh_gptq_dequant", None, dq.data_ptr, dz.data_ptr, ds.data_ptr, None, out.data_ptr,
+             n, k, group_size, bits)
     ref = O.dequantize_packed(qweight, qzeros, scales, None, bits, group_size)
     np.testing.assert_array_equal(out.numpy().view(np.uint16), ref.view(np.uint16))
 
@@ -77,8 +79,9 @@ def test_dequant_act_order_bit_exact(hip):
     qweight, qzeros, scales = _weights(k, n, g, 4, seed=2)
     g_idx = np.random.default_rng(3).permutation(k).astype(np.int32) // g
     out = HIPTensor.allocate((k, n), "float16")
-    hip.call("mh_gptq_dequant", None, _dev(hip, qweight).data_ptr, _dev(hip, qzeros).data_ptr,
-             _dev(hip, scales).data_ptr, _dev(hip, g_idx).data_ptr, out.data_ptr, n, k, g, 4)
+    dq, dz, ds, dg = _dev(hip, qweight), _dev(hip, qzeros), _dev(hip, scales), _dev(hip, g_idx)
+    hip.call("mh_gptq_dequant", None, dq.data_ptr, dz.data_ptr, ds.data_ptr, dg.data_ptr, out.data_ptr,
+             n, k, g, 4)
     ref = O.dequantize_packed(qweight, qzeros, scales, g_idx, 4)
     np.testing.assert_array_equal(out.numpy().view(np.uint16), ref.view(np.uint16))
 

@@ -1,0 +1,121 @@
+"""Host-side logic that needs no GPU: the multimethod table, the C ABI surface
+and the loader."""
+import ctypes
+import os
+import re
+from typing import Union
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from minit_amd import lib
+    header = open(os.path.join(ROOT, "include", "minit_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(mh_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) > 30
+    cdll = lib.cdll()                      # loads without a GPU
+    for name in sorted(declared):
+        assert hasattr(cdll, name), f"{name} is declared in minit_hip.h but not exported"
+        assert name in lib.PROTOTYPES, f"{name} has no ctypes prototype"
+    assert set(lib.PROTOTYPES) <= declared, set(lib.PROTOTYPES) - declared
+    assert cdll.mh_abi_version() == 1
+
+
+def test_loader_raises_without_the_library(monkeypatch, tmp_path):
+    from minit_amd import lib
+    monkeypatch.setattr(lib, "_cdll", None)
+    monkeypatch.setattr(lib, "LIB_PATH", str(tmp_path / "missing.so"))
+    with pytest.raises(lib.HipError, match="no CPU fallback"):
+        lib.cdll()
+
+
+def test_status_codes_raise_with_message():
+    from minit_amd import lib
+    with pytest.raises(lib.HipError, match="bits must be 4 or 8"):
+        lib.call("mh_gptq_unpack", None, 256, 256, 4, 4, 0, 5)
+    with pytest.raises(lib.HipError, match="t=7 must equal"):
+        lib.call("mh_softmax_causal", None, 256, 256, 1, 2, 7, 3, 1.0, 0)
+    assert lib.call("mh_gptq_workspace_bytes", 1, 4096, 4096, 128, 4) > 0
+    assert lib.call("mh_gptq_workspace_bytes", 1, 4096, 4100, 128, 4) == 0   # contract violated
+
+
+def test_dispatch_rules():
+    from minit_amd.core.dispatch import DISPATCH_CACHE, DISPATCH_TABLE, dispatch, register_dispatch
+    from minit_amd.core.operator import Operator
+    from minit_amd.core.tensor import Tensor
+
+    class Op(Operator):
+        pass
+
+    class A(Tensor):
+        pass
+
+    class B(A):
+        pass
+
+    class C(Tensor):
+        pass
+
+    saved = list(DISPATCH_TABLE)
+    try:
+        @register_dispatch()
+        def generic(op: Op, x: Tensor):
+            return ("generic",)
+
+        @register_dispatch(priority=1)
+        def for_a(op: Op, x: A):
+            return ("a",)
+
+        @register_dispatch()
+        def union(op: Op, x: Union[A, C], y: Union[A, C]):
+            return ("union",)
+
+        @register_dispatch()
+        def variadic(op: Op, x: C, y: C, *rest: C):
+            return ("variadic", len(rest))
+
+        assert dispatch(Op(), C()) == ("generic",)
+        assert dispatch(Op(), A()) == ("a",)          # higher priority wins
+        assert dispatch(Op(), B()) == ("a",)          # subclasses match
+        assert dispatch(Op(), A(), C()) == ("union",)
+        assert dispatch(Op(), C(), C(), C(), C()) == ("variadic", 2)
+        with pytest.raises(AssertionError, match="more than one"):
+            dispatch(Op(), C(), C())                   # union and variadic tie
+        with pytest.raises(AssertionError, match="no matching"):
+            dispatch(Op(), A(), A(), A())
+
+        @register_dispatch(predicate=lambda *tys: False, priority=5)
+        def never(op: Op, x: Tensor):
+            return ("never",)
+
+        assert dispatch(Op(), C()) == ("generic",)
+    finally:
+        DISPATCH_TABLE[:] = saved
+        DISPATCH_CACHE.clear()
+
+
+def test_quantized_rule_outranks_the_generic_one():
+    """(MatrixMultiply, HIPTensor, QuantizedTensor) must resolve to the fused
+    rule, registered above priority 0."""
+    import minit_amd  # noqa: F401
+    from minit_amd.core.dispatch import lookup_implementation_from_types
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.operator import MatrixMultiply, RMSNorm, RoPE, Softmax, Sum
+    from minit_amd.quantize.tensor import QuantizedTensor
+    fn = lookup_implementation_from_types((MatrixMultiply, HIPTensor, QuantizedTensor))
+    assert fn.__name__ == "dispatch_quantized_matmul"
+    assert lookup_implementation_from_types((MatrixMultiply, HIPTensor, HIPTensor)).__name__ == "dispatch_matmul"
+    for tys in [(RMSNorm, HIPTensor, HIPTensor), (RoPE, HIPTensor, HIPTensor, HIPTensor),
+                (RoPE, HIPTensor, HIPTensor, HIPTensor, HIPTensor), (Softmax, HIPTensor), (Sum, HIPTensor)]:
+        assert lookup_implementation_from_types(tys) is not None
+
+
+def test_functional_argument_checks():
+    import minit_amd.functional as F
+    with pytest.raises(AssertionError):
+        F.rms_norm(None, None, 0, 1)         # eps must be a float, as in the reference
+    with pytest.raises(AssertionError):
+        F.rms_norm(None, None, 0, 0.75)
