@@ -284,6 +284,7 @@ GemmPlan plan_gemm(int M, int N, int K) {
     const long traffic_cap = K / (64L * M) > 1 ? K / (64L * M) : 1;
     if (max_split > traffic_cap) max_split = traffic_cap;
     if (split > max_split) split = max_split;
+    if ((long)p.col_tiles * p.m_blocks > kMaxCounters) split = 1;  // no counter for that many tiles
     if (split < 1) split = 1;
     long spb = (p.steps_total + split - 1) / split;
     spb = (spb + sc - 1) / sc * sc;
@@ -301,18 +302,16 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)group_size;
     (void)bits;
     const GemmPlan p = plan_gemm(M, N, K);
-    size_t counters = ((size_t)p.col_tiles * p.m_blocks * sizeof(unsigned) + 255) / 256 * 256;
     size_t partial = (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
-    return counters + partial;
+    return kCounterRegionBytes + partial;
 }
 
 template <int BITS, int MT>
 static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                         const int32_t* qzeros, const void* scales, void* out, void* workspace, int M, int N,
                         int K, int group_size) {
-    const size_t counters_bytes = ((size_t)p.col_tiles * p.m_blocks * sizeof(unsigned) + 255) / 256 * 256;
     unsigned* counters = reinterpret_cast<unsigned*>(workspace);
-    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters_bytes);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterRegionBytes);
     hipLaunchKernelGGL((gptq_gemm_kernel<BITS, MT>), dim3(p.col_tiles, p.split_k, p.m_blocks), dim3(256), 0,
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, counters, M, N, K, group_size / 32,

@@ -212,6 +212,7 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
     if (split > max_split) split = max_split;
     if (split < min_split) split = min_split;
     if (split < 1) split = 1;
+    if (p.col_tiles > kMaxCounters && min_split <= 1) split = 1;  // no counter for that many tiles
     p.steps_per_wave = (int)((p.steps_total + split * kGemvWaves - 1) / (split * kGemvWaves));
     p.split_k = (p.steps_total + p.steps_per_wave * kGemvWaves - 1) / (p.steps_per_wave * kGemvWaves);
     return p;
@@ -219,9 +220,8 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
 
 size_t gemv_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     const GemvPlan p = plan_gemv(N, K, group_size, bits);
-    size_t counters = ((size_t)p.col_tiles * sizeof(unsigned) + 255) / 256 * 256;
     size_t partial = (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
-    return counters + partial;
+    return kCounterRegionBytes + partial;
 }
 
 template <int BITS, int M, int ROWS>
@@ -229,9 +229,8 @@ static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, co
                         const int32_t* qzeros, const void* scales, void* out, void* workspace,
                         int N, int K, int group_size) {
     constexpr int P = Packing<BITS>::kPerWord;
-    const size_t counters_bytes = ((size_t)p.col_tiles * sizeof(unsigned) + 255) / 256 * 256;
     unsigned* counters = reinterpret_cast<unsigned*>(workspace);
-    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters_bytes);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterRegionBytes);
     const size_t lds = (size_t)M * kGemvWaves * p.steps_per_wave * ROWS * Packing<BITS>::kPairs * sizeof(uint32_t);
     hipLaunchKernelGGL((gptq_gemv_kernel<BITS, M, ROWS>), dim3(p.col_tiles, p.split_k), dim3(256), lds, stream,
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
@@ -275,6 +274,9 @@ int gptq_gemv_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     const GemvPlan p = plan_gemv(N, K, group_size, bits);
     const size_t need = gemv_workspace_bytes(M, N, K, group_size, bits);
     if (p.split_k > 1) {
+        if (p.col_tiles > kMaxCounters)
+            return fail(MH_ERR_INVALID, "mh_gptq_gemv: N=%d with K=%d needs more than %d tile counters", N, K,
+                        kMaxCounters);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemv: workspace of %zu bytes required, got %zu", need,
                         workspace ? workspace_bytes : (size_t)0);

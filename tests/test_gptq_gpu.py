@@ -158,6 +158,21 @@ def test_repeated_calls_are_deterministic(hip):
             np.testing.assert_array_equal(first.view(np.uint16), again.view(np.uint16))
 
 
+def test_shared_workspace_across_shapes(hip):
+    """One workspace serves calls of different shapes: the partial sums of a call
+    with few column tiles must not disturb the arrival counters of a later call
+    with many (counters live in a fixed region of the workspace)."""
+    from minit_amd import synthetic
+    shapes = [(1, 2048, 256), (16, 2048, 512), (1, 1024, 57344), (2, 4096, 1024), (24, 1024, 20480)]
+    for m, k, n in shapes:
+        qweight, qzeros, scales = _weights(k, n, 128, 4, seed=13)
+        x = synthetic.activations("test13", f"x{m}-{k}", (m, k))
+        entry = "mh_gptq_gemv" if m <= 4 else "mh_gptq_gemm"
+        got = _run_linear(hip, entry, x, qweight, qzeros, scales, 128, 4)
+        ref = O.matmul_f64(x, qweight, qzeros, scales, None, 4, 128)
+        assert_fp16_close(got, ref, what=f"shared workspace {m}x{k}x{n}")
+
+
 def test_act_order_through_matmul(hip):
     from minit_amd import synthetic
     m, k, n, g = 3, 512, 128, 128
