@@ -188,6 +188,49 @@ int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, si
 int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
                 size_t n, int exact, int dtype);
 
+/* ---- Llama-family GPTQ decode loop ------------------------------------------------------
+ * The callers around the quantized linears: one greedy decode step per token as
+ * the reference's models run it (examples/llama3_70b.py:77-162,215-249;
+ * sampling minit/chat/sample.py:11-14), enqueued from native code.  All
+ * pointers are device pointers owned by the caller.
+ *   qkv      fused q|k|v projection, GPTQ, [hidden] -> [(QH + 2 KVH) * D]
+ *   gate_up  fused gate|up projection, [hidden] -> [2 * ffn]
+ *   k_cache / v_cache  fp16 [batch_max, KVH, max_seq, D], appended in place
+ *   embed, lm_head     fp16 [vocab, hidden]; norms fp16 [hidden]
+ *   freqs_cos / sin    fp32 [max_seq, D / 2]
+ */
+typedef struct {
+    int n_layers, hidden, n_q_heads, n_kv_heads, head_dim, ffn, vocab;
+    int group_size, bits, max_seq;
+    float rms_eps;
+} mh_llama_config;
+typedef struct {
+    const int32_t* qweight;
+    const int32_t* qzeros;
+    const void* scales;
+} mh_qlinear;
+typedef struct {
+    mh_qlinear qkv, o, gate_up, down;
+    const void* input_norm;
+    const void* post_norm;
+    void* k_cache;
+    void* v_cache;
+} mh_llama_layer;
+int mh_llama_create(void** handle, const mh_llama_config* cfg);
+int mh_llama_destroy(void* handle);
+int mh_llama_set_layer(void* handle, int layer, const mh_llama_layer* l);
+int mh_llama_set_globals(void* handle, const void* embed, const void* lm_head, const void* final_norm,
+                         const float* freqs_cos, const float* freqs_sin);
+/* Scratch for activations, split-K partials and counters; zero-fill it once. */
+size_t mh_llama_scratch_bytes(void* handle, int batch);
+/* Runs n_steps greedy steps.  tokens [batch] int32 holds the input token of the
+ * first step and the last sampled token on return; positions [batch] int32 is
+ * where each row's next K/V entry goes and is advanced by one per step;
+ * out_tokens (optional) receives [n_steps, batch]; logits_out (optional)
+ * receives the last step's fp16 logits [batch, vocab]. */
+int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
+                    int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes);
+
 /* ---- synthetic inputs ------------------------------------------------------------------
  * No counterpart in the reference (it loads checkpoints from disk,
  * minit/module/checkpoint.py:11-44).  Counter-based generators that fill device

@@ -1,0 +1,553 @@
+// Llama-family GPTQ decode step: the callers on either side of the quantized
+// linears (examples/llama3_70b.py:77-162,215-249 of the reference), run as one
+// native loop that enqueues every kernel of a token step from C++.
+//
+// What differs from the reference's step, by design:
+//   * KV cache is preallocated [B, KVH, T, D] and appended in place; the
+//     reference re-allocates and concatenates it every token (llama3_70b.py:97-100)
+//     and stores it expanded to all query heads (:164-168).
+//   * attention for one new token is a split-KV streaming kernel that fuses the
+//     1/sqrt(d) scale, softmax and the P.V product; grouped-query heads that
+//     share a KV head are processed together so K and V are read once.
+//   * residual add + RMSNorm, RoPE + cache append, SiLU*up are fused kernels.
+//   * sampling is an on-device argmax (the reference copies the logits to the
+//     host, minit/chat/sample.py:11-14).
+#include "common.h"
+
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace mh {
+
+int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                         const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                         void* workspace, size_t workspace_bytes);
+
+// ---- small fused kernels --------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void embed_gather_kernel(const int32_t* __restrict__ tokens,
+                                                           const half_t* __restrict__ embed,
+                                                           half_t* __restrict__ out, int hidden, int vocab) {
+    const int b = blockIdx.x;
+    int tok = tokens[b];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const uint4* src = reinterpret_cast<const uint4*>(embed + (size_t)tok * hidden);
+    uint4* dst = reinterpret_cast<uint4*>(out + (size_t)b * hidden);
+    for (int i = threadIdx.x; i < hidden / 8; i += blockDim.x) dst[i] = src[i];
+}
+
+// h <- fp16(h + delta) (skipped when delta == nullptr); xn <- rmsnorm(h) * w.
+// The sum is rounded to fp16 before it is normalised, as the separate add and
+// norm kernels of the reference would (llama3_70b.py:159-162).
+__global__ __launch_bounds__(256) void add_rms_norm_kernel(half_t* __restrict__ h, const half_t* __restrict__ delta,
+                                                           const half_t* __restrict__ w, half_t* __restrict__ xn,
+                                                           int hidden, float eps) {
+    __shared__ float smem[16];
+    const size_t row = blockIdx.x;
+    uint4* hp = reinterpret_cast<uint4*>(h + row * hidden);
+    const uint4* dp = delta ? reinterpret_cast<const uint4*>(delta + row * hidden) : nullptr;
+    const uint4* wp = reinterpret_cast<const uint4*>(w);
+    uint4* op = reinterpret_cast<uint4*>(xn + row * hidden);
+    const int nvec = hidden / 8;
+    half8_t vals[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int v = c * 256 + threadIdx.x;
+        if (v < nvec) {
+            half8_t a = __builtin_bit_cast(half8_t, hp[v]);
+            if (dp) {
+                a = a + __builtin_bit_cast(half8_t, dp[v]);  // fp16 add, one rounding
+                hp[v] = __builtin_bit_cast(uint4, a);
+            }
+            vals[c] = a;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += (float)a[i] * (float)a[i];
+        }
+    }
+    ss = block_sum(ss, smem);
+    const float rms = sqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int v = c * 256 + threadIdx.x;
+        if (v < nvec) {
+            const half8_t wv = __builtin_bit_cast(half8_t, wp[v]);
+            half8_t o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = (half_t)((float)vals[c][i] / rms * (float)wv[i]);
+            op[v] = __builtin_bit_cast(uint4, o);
+        }
+    }
+}
+
+// h <- fp16(h + delta) only (after the last block).
+__global__ void add_kernel(half_t* __restrict__ h, const half_t* __restrict__ delta, size_t n8) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint4* hp = reinterpret_cast<uint4*>(h);
+    const uint4* dp = reinterpret_cast<const uint4*>(delta);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+        const half8_t a = __builtin_bit_cast(half8_t, hp[i]) + __builtin_bit_cast(half8_t, dp[i]);
+        hp[i] = __builtin_bit_cast(uint4, a);
+    }
+}
+
+// qkv [B, (QH + 2 KVH) * D]: rotate q heads into q_out [B, QH, D]; rotate k
+// heads and copy v heads into the caches at positions[b].  One 64-thread block
+// per (head, batch row); thread i owns the interleaved pair i
+// (minit/cuda/kernel/cuda/rope.py:58-73).
+__global__ __launch_bounds__(64) void rope_kv_append_kernel(
+    const half_t* __restrict__ qkv, const float* __restrict__ freqs_cos, const float* __restrict__ freqs_sin,
+    const int32_t* __restrict__ positions, half_t* __restrict__ q_out, half_t* __restrict__ k_cache,
+    half_t* __restrict__ v_cache, int qh, int kvh, int head_dim, int max_seq) {
+    const int head = blockIdx.x, b = blockIdx.y;
+    const int half_dim = head_dim / 2;
+    const int pos = positions[b];
+    const half_t* src = qkv + ((size_t)b * (qh + 2 * kvh) + head) * head_dim;
+    for (int i = threadIdx.x; i < half_dim; i += blockDim.x) {
+        const float re = (float)src[2 * i], im = (float)src[2 * i + 1];
+        if (head >= qh + kvh) {  // v: plain copy
+            half_t* dst = v_cache + (((size_t)b * kvh + (head - qh - kvh)) * max_seq + pos) * head_dim;
+            dst[2 * i] = src[2 * i];
+            dst[2 * i + 1] = src[2 * i + 1];
+            continue;
+        }
+        const float c = freqs_cos[(size_t)pos * half_dim + i], s = freqs_sin[(size_t)pos * half_dim + i];
+        const half_t o0 = (half_t)(re * c - im * s), o1 = (half_t)(im * c + re * s);
+        half_t* dst = head < qh ? q_out + ((size_t)b * qh + head) * head_dim
+                                : k_cache + (((size_t)b * kvh + (head - qh)) * max_seq + pos) * head_dim;
+        dst[2 * i] = o0;
+        dst[2 * i + 1] = o1;
+    }
+}
+
+// act[b, f] = silu(gu[b, f]) * gu[b, F + f]; fp32 until the store.
+__global__ void silu_mul_fused_kernel(const half_t* __restrict__ gu, half_t* __restrict__ act, int batch, int ffn) {
+    const size_t n8 = (size_t)batch * ffn / 8;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const int row8 = ffn / 8;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+        const size_t b = i / row8, c = i % row8;
+        const half8_t g = __builtin_bit_cast(half8_t, reinterpret_cast<const uint4*>(gu + b * 2 * ffn)[c]);
+        const half8_t u = __builtin_bit_cast(half8_t, reinterpret_cast<const uint4*>(gu + b * 2 * ffn + ffn)[c]);
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float gf = (float)g[e];
+            o[e] = (half_t)(gf / (1.f + expf(-gf)) * (float)u[e]);
+        }
+        reinterpret_cast<uint4*>(act)[i] = __builtin_bit_cast(uint4, o);
+    }
+}
+
+// token[b] = argmax_v logits[b, v] (first maximum); appended to the output
+// stream and fed back as the next input; positions[b] += 1.
+__global__ __launch_bounds__(256) void argmax_advance_kernel(const half_t* __restrict__ logits,
+                                                             int32_t* __restrict__ tokens,
+                                                             int32_t* __restrict__ out_tokens,
+                                                             int32_t* __restrict__ positions, int vocab) {
+    __shared__ float sval[256];
+    __shared__ int sidx[256];
+    const int b = blockIdx.x;
+    const half_t* row = logits + (size_t)b * vocab;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int v = threadIdx.x; v < vocab; v += blockDim.x) {
+        const float x = (float)row[v];
+        if (x > best || (x == best && v < best_i)) {
+            best = x;
+            best_i = v;
+        }
+    }
+    sval[threadIdx.x] = best;
+    sidx[threadIdx.x] = best_i;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            const float o = sval[threadIdx.x + off];
+            const int oi = sidx[threadIdx.x + off];
+            if (o > sval[threadIdx.x] || (o == sval[threadIdx.x] && oi < sidx[threadIdx.x])) {
+                sval[threadIdx.x] = o;
+                sidx[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const int tok = sidx[0] == 0x7fffffff ? 0 : sidx[0];
+        tokens[b] = tok;
+        if (out_tokens) out_tokens[b] = tok;
+        positions[b] += 1;
+    }
+}
+
+// ---- split-KV decode attention ---------------------------------------------------------------------
+// One block per (split, kv head, batch row); G query heads share the KV head.
+// Phase A (lane = one cached position): scores of a 64-position chunk for all G
+// heads, running max / sum per head.  Phase B (lane = 8 output dims x one of 4
+// position sub-streams): acc[h] += p[h, t] * V[t].  Waves own alternate chunks
+// and are merged through LDS; splits are merged by the last block to arrive.
+
+template <int G, int D>
+struct AttnPartial {  // per (b, q head, split): m, l, acc[D]
+    static constexpr int kFloats = D + 2;
+};
+
+template <int G, int D>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const half_t* __restrict__ q, const half_t* __restrict__ k_cache, const half_t* __restrict__ v_cache,
+    const int32_t* __restrict__ positions, half_t* __restrict__ out, float* partial, unsigned* counters,
+    int kvh, int max_seq, float scale, int splits) {
+    static_assert(D == 128, "head size 128");
+    constexpr int CH = D / 8;  // 16-byte chunks per row
+    const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int len = positions[b] + 1;  // the new token has been appended
+    const int span = (len + splits - 1) / splits;
+    const int t0 = split * span, t1 = min(len, t0 + span);
+
+    __shared__ uint4 q_s[G * CH];
+    __shared__ float p_s[4][G][64];
+    __shared__ float m_s[4][G], l_s[4][G];
+    __shared__ float acc_s[4][G][D];
+
+    const half_t* qp = q + ((size_t)b * kvh + g) * G * D;
+    for (int i = tid; i < G * CH; i += 256) q_s[i] = reinterpret_cast<const uint4*>(qp)[i];
+    __syncthreads();
+
+    const half_t* kbase = k_cache + ((size_t)b * kvh + g) * max_seq * D;
+    const half_t* vbase = v_cache + ((size_t)b * kvh + g) * max_seq * D;
+
+    float m_run[G], l_run[G];
+    float acc[G][8];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        m_run[h] = -INFINITY;
+        l_run[h] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
+    }
+    const int dl = lane & 15, tg = lane >> 4;
+
+    for (int c0 = t0 + wave * 64; c0 < t1; c0 += 256) {
+        // ---- phase A
+        const int t = c0 + lane;
+        const bool valid = t < t1;
+        float s[G];
+#pragma unroll
+        for (int h = 0; h < G; ++h) s[h] = 0.f;
+        const uint4* krow = reinterpret_cast<const uint4*>(kbase + (size_t)(valid ? t : t0) * D);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const uint4 kv = krow[c];
+            const half2_t k0 = __builtin_bit_cast(half2_t, kv.x), k1 = __builtin_bit_cast(half2_t, kv.y),
+                          k2 = __builtin_bit_cast(half2_t, kv.z), k3 = __builtin_bit_cast(half2_t, kv.w);
+#pragma unroll
+            for (int h = 0; h < G; ++h) {
+                const uint4 qv = q_s[h * CH + c];
+                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.x), k0, s[h], false);
+                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.y), k1, s[h], false);
+                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.z), k2, s[h], false);
+                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.w), k3, s[h], false);
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            const float sv = valid ? s[h] * scale : -INFINITY;
+            const float m_new = fmaxf(m_run[h], wave_max(sv));
+            const float p = valid ? expf(sv - m_new) : 0.f;
+            const float alpha = expf(m_run[h] - m_new);  // exp(-inf) = 0 on the first chunk
+            l_run[h] = l_run[h] * alpha + wave_sum(p);
+            m_run[h] = m_new;
+            p_s[wave][h][lane] = p;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e] *= alpha;
+        }
+        __builtin_amdgcn_wave_barrier();
+        // ---- phase B
+#pragma unroll 4
+        for (int tt = 0; tt < 16; ++tt) {
+            const int tl = tt * 4 + tg;
+            const int tv = c0 + tl;
+            if (tv < t1) {
+                const uint4 vv = reinterpret_cast<const uint4*>(vbase + (size_t)tv * D)[dl];
+                const half8_t vh = __builtin_bit_cast(half8_t, vv);
+#pragma unroll
+                for (int h = 0; h < G; ++h) {
+                    const float p = p_s[wave][h][tl];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[h][e] = __builtin_fmaf(p, (float)vh[e], acc[h][e]);
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // merge the four position sub-streams of the wave
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            acc[h][e] += __shfl_xor(acc[h][e], 16, 64);
+            acc[h][e] += __shfl_xor(acc[h][e], 32, 64);
+        }
+    if (tg == 0) {
+#pragma unroll
+        for (int h = 0; h < G; ++h)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc_s[wave][h][dl * 8 + e] = acc[h][e];
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            m_s[wave][h] = m_run[h];
+            l_s[wave][h] = l_run[h];
+        }
+    }
+    __syncthreads();
+
+    // merge the four waves: thread -> (head, dims)
+    constexpr int ITEMS = G * D;  // outputs per block
+    const size_t head0 = ((size_t)b * kvh + g) * G;
+    for (int i = tid; i < ITEMS; i += 256) {
+        const int h = i / D, d = i % D;
+        float mm = fmaxf(fmaxf(m_s[0][h], m_s[1][h]), fmaxf(m_s[2][h], m_s[3][h]));
+        float ll = 0.f, a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float f = (m_s[w][h] == -INFINITY) ? 0.f : expf(m_s[w][h] - mm);
+            ll += l_s[w][h] * f;
+            a += acc_s[w][h][d] * f;
+        }
+        if (splits == 1) {
+            out[(head0 + h) * D + d] = (half_t)(a / ll);
+        } else {
+            float* pp = partial + ((head0 + h) * splits + split) * (D + 2);
+            store_agent(pp + 2 + d, a);
+            if (d == 0) {
+                store_agent(pp, mm);
+                store_agent(pp + 1, ll);
+            }
+        }
+    }
+    if (splits == 1) return;
+
+    __shared__ int is_last;
+    if (!arrive_and_check_last(counters + (size_t)b * kvh + g, (unsigned)splits, &is_last)) return;
+    for (int i = tid; i < ITEMS; i += 256) {
+        const int h = i / D, d = i % D;
+        const float* pp = partial + (head0 + h) * splits * (D + 2);
+        float mm = -INFINITY;
+        for (int sp = 0; sp < splits; ++sp) mm = fmaxf(mm, load_agent(pp + (size_t)sp * (D + 2)));
+        float ll = 0.f, a = 0.f;
+        for (int sp = 0; sp < splits; ++sp) {
+            const float ms = load_agent(pp + (size_t)sp * (D + 2));
+            const float f = (ms == -INFINITY) ? 0.f : expf(ms - mm);
+            ll += load_agent(pp + (size_t)sp * (D + 2) + 1) * f;
+            a += load_agent(pp + (size_t)sp * (D + 2) + 2 + d) * f;
+        }
+        out[(head0 + h) * D + d] = (half_t)(a / ll);
+    }
+}
+
+// ---- model description and the decode loop ------------------------------------------------------------
+
+struct Llama {
+    mh_llama_config cfg;
+    std::vector<mh_llama_layer> layers;
+    const void* embed = nullptr;
+    const void* lm_head = nullptr;
+    const void* final_norm = nullptr;
+    const float* cos = nullptr;
+    const float* sin = nullptr;
+};
+
+struct Scratch {
+    half_t *h, *xn, *qkv, *q, *attn, *delta, *gu, *act, *logits;
+    float* attn_partial;
+    unsigned* attn_counters;
+    void* gptq_ws;
+    size_t gptq_ws_bytes;
+    size_t total;
+};
+
+static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
+
+static int attn_splits(const Llama& m, int batch) {
+    const int pairs = batch * m.cfg.n_kv_heads;
+    int splits = (2 * compute_units() + pairs - 1) / pairs;
+    const int max_splits = (m.cfg.max_seq + 255) / 256;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 64) splits = 64;
+    return splits < 1 ? 1 : splits;
+}
+
+static Scratch carve(const Llama& m, int batch, char* base) {
+    const mh_llama_config& c = m.cfg;
+    const size_t qkv_n = (size_t)(c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* p = base ? base + off : nullptr;
+        off += align_up(bytes);
+        return p;
+    };
+    Scratch s;
+    // counters first: they must start (and are left) zero
+    s.attn_counters = (unsigned*)take((size_t)batch * c.n_kv_heads * sizeof(unsigned));
+    size_t ws = 0;
+    const int shapes[4][2] = {{c.hidden, (int)qkv_n}, {c.n_q_heads * c.head_dim, c.hidden},
+                              {c.hidden, 2 * c.ffn}, {c.ffn, c.hidden}};
+    for (auto& sh : shapes) {
+        const size_t need = mh_gptq_workspace_bytes(batch, sh[1], sh[0], c.group_size, c.bits);
+        if (need > ws) ws = need;
+    }
+    s.gptq_ws_bytes = align_up(ws > 0 ? ws : 256);
+    s.gptq_ws = take(s.gptq_ws_bytes);
+    s.h = (half_t*)take((size_t)batch * c.hidden * 2);
+    s.xn = (half_t*)take((size_t)batch * c.hidden * 2);
+    s.qkv = (half_t*)take((size_t)batch * qkv_n * 2);
+    s.q = (half_t*)take((size_t)batch * c.n_q_heads * c.head_dim * 2);
+    s.attn = (half_t*)take((size_t)batch * c.n_q_heads * c.head_dim * 2);
+    s.delta = (half_t*)take((size_t)batch * c.hidden * 2);
+    s.gu = (half_t*)take((size_t)batch * 2 * c.ffn * 2);
+    s.act = (half_t*)take((size_t)batch * c.ffn * 2);
+    s.logits = (half_t*)take((size_t)batch * c.vocab * 2);
+    s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 2) * 4);
+    s.total = off;
+    return s;
+}
+
+template <int G>
+static void launch_attn(hipStream_t st, const Llama& m, const Scratch& s, const mh_llama_layer& L,
+                        const int32_t* positions, int batch, int splits) {
+    const mh_llama_config& c = m.cfg;
+    hipLaunchKernelGGL((attn_decode_kernel<G, 128>), dim3(splits, c.n_kv_heads, batch), dim3(256), 0, st,
+                       s.q, (const half_t*)L.k_cache, (const half_t*)L.v_cache, positions, s.attn,
+                       s.attn_partial, s.attn_counters, c.n_kv_heads, c.max_seq,
+                       1.0f / sqrtf((float)c.head_dim), splits);
+}
+
+}  // namespace mh
+
+using namespace mh;
+
+extern "C" {
+
+int mh_llama_create(void** handle, const mh_llama_config* cfg) {
+    MH_REQUIRE(handle && cfg, "mh_llama_create: null argument");
+    MH_REQUIRE(cfg->n_layers > 0 && cfg->hidden > 0 && cfg->ffn > 0 && cfg->vocab > 0, "mh_llama_create: bad sizes");
+    MH_REQUIRE(cfg->head_dim == 128, "mh_llama_create: head_dim must be 128, got %d", cfg->head_dim);
+    MH_REQUIRE(cfg->n_kv_heads > 0 && cfg->n_q_heads % cfg->n_kv_heads == 0, "mh_llama_create: bad head counts");
+    const int g = cfg->n_q_heads / cfg->n_kv_heads;
+    MH_REQUIRE(g == 1 || g == 2 || g == 4 || g == 8, "mh_llama_create: %d query heads per KV head unsupported", g);
+    MH_REQUIRE(cfg->hidden % 8 == 0 && cfg->hidden <= 8192, "mh_llama_create: hidden must be <= 8192 and a multiple of 8");
+    MH_REQUIRE(cfg->ffn % 8 == 0, "mh_llama_create: ffn must be a multiple of 8");
+    Llama* m = new (std::nothrow) Llama();
+    MH_REQUIRE(m != nullptr, "mh_llama_create: out of host memory");
+    m->cfg = *cfg;
+    m->layers.resize(cfg->n_layers);
+    memset(m->layers.data(), 0, sizeof(mh_llama_layer) * cfg->n_layers);
+    *handle = m;
+    return MH_OK;
+}
+
+int mh_llama_destroy(void* handle) {
+    delete reinterpret_cast<Llama*>(handle);
+    return MH_OK;
+}
+
+int mh_llama_set_layer(void* handle, int layer, const mh_llama_layer* l) {
+    Llama* m = reinterpret_cast<Llama*>(handle);
+    MH_REQUIRE(m && l, "mh_llama_set_layer: null argument");
+    MH_REQUIRE(layer >= 0 && layer < m->cfg.n_layers, "mh_llama_set_layer: layer %d out of range", layer);
+    m->layers[layer] = *l;
+    return MH_OK;
+}
+
+int mh_llama_set_globals(void* handle, const void* embed, const void* lm_head, const void* final_norm,
+                         const float* freqs_cos, const float* freqs_sin) {
+    Llama* m = reinterpret_cast<Llama*>(handle);
+    MH_REQUIRE(m && embed && lm_head && final_norm && freqs_cos && freqs_sin, "mh_llama_set_globals: null argument");
+    m->embed = embed;
+    m->lm_head = lm_head;
+    m->final_norm = final_norm;
+    m->cos = freqs_cos;
+    m->sin = freqs_sin;
+    return MH_OK;
+}
+
+size_t mh_llama_scratch_bytes(void* handle, int batch) {
+    Llama* m = reinterpret_cast<Llama*>(handle);
+    if (!m || batch <= 0) return 0;
+    return carve(*m, batch, nullptr).total;
+}
+
+int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
+                    int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes) {
+    Llama* m = reinterpret_cast<Llama*>(handle);
+    MH_REQUIRE(m != nullptr, "mh_llama_decode: null handle");
+    MH_REQUIRE(batch > 0 && n_steps >= 0, "mh_llama_decode: bad batch / steps");
+    MH_REQUIRE(tokens && positions && scratch, "mh_llama_decode: null argument");
+    MH_REQUIRE(m->embed != nullptr, "mh_llama_decode: globals not set");
+    MH_REQUIRE((uintptr_t)scratch % 256 == 0, "mh_llama_decode: scratch must be 256-byte aligned");
+    const Scratch s = carve(*m, batch, reinterpret_cast<char*>(scratch));
+    if (scratch_bytes < s.total)
+        return fail(MH_ERR_WORKSPACE, "mh_llama_decode: scratch of %zu bytes required, got %zu", s.total, scratch_bytes);
+    const mh_llama_config& c = m->cfg;
+    for (int l = 0; l < c.n_layers; ++l)
+        MH_REQUIRE(m->layers[l].qkv.qweight && m->layers[l].k_cache, "mh_llama_decode: layer %d not set", l);
+    hipStream_t st = as_stream(stream);
+    const int qkv_n = (c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim;
+    const int g = c.n_q_heads / c.n_kv_heads;
+    const int splits = attn_splits(*m, batch);
+    const unsigned ew_grid = (unsigned)compute_units() * 4;
+
+    auto linear = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k) -> int {
+        return gptq_matmul_dispatch(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
+                                    s.gptq_ws, s.gptq_ws_bytes);
+    };
+
+    for (int step = 0; step < n_steps; ++step) {
+        hipLaunchKernelGGL(embed_gather_kernel, dim3(batch), dim3(256), 0, st, tokens, (const half_t*)m->embed, s.h,
+                           c.hidden, c.vocab);
+        hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, (const half_t*)nullptr,
+                           (const half_t*)m->layers[0].input_norm, s.xn, c.hidden, c.rms_eps);
+        for (int l = 0; l < c.n_layers; ++l) {
+            const mh_llama_layer& L = m->layers[l];
+            int rc = linear(s.xn, L.qkv, s.qkv, qkv_n, c.hidden);
+            if (rc) return rc;
+            hipLaunchKernelGGL(rope_kv_append_kernel, dim3(c.n_q_heads + 2 * c.n_kv_heads, batch), dim3(64), 0, st,
+                               s.qkv, m->cos, m->sin, positions, s.q, (half_t*)L.k_cache, (half_t*)L.v_cache,
+                               c.n_q_heads, c.n_kv_heads, c.head_dim, c.max_seq);
+            switch (g) {
+                case 1: launch_attn<1>(st, *m, s, L, positions, batch, splits); break;
+                case 2: launch_attn<2>(st, *m, s, L, positions, batch, splits); break;
+                case 4: launch_attn<4>(st, *m, s, L, positions, batch, splits); break;
+                default: launch_attn<8>(st, *m, s, L, positions, batch, splits); break;
+            }
+            rc = linear(s.attn, L.o, s.delta, c.hidden, c.n_q_heads * c.head_dim);
+            if (rc) return rc;
+            hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, s.delta,
+                               (const half_t*)L.post_norm, s.xn, c.hidden, c.rms_eps);
+            rc = linear(s.xn, L.gate_up, s.gu, 2 * c.ffn, c.hidden);
+            if (rc) return rc;
+            hipLaunchKernelGGL(silu_mul_fused_kernel, dim3(ew_grid), dim3(256), 0, st, s.gu, s.act, batch, c.ffn);
+            rc = linear(s.act, L.down, s.delta, c.hidden, c.ffn);
+            if (rc) return rc;
+            const half_t* next_norm =
+                (const half_t*)(l + 1 < c.n_layers ? m->layers[l + 1].input_norm : m->final_norm);
+            hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, s.delta, next_norm, s.xn,
+                               c.hidden, c.rms_eps);
+        }
+        int rc = mh_f16_matmul_nk(stream, s.xn, m->lm_head, s.logits, batch, c.vocab, c.hidden);
+        if (rc) return rc;
+        hipLaunchKernelGGL(argmax_advance_kernel, dim3(batch), dim3(256), 0, st, s.logits, tokens,
+                           out_tokens ? out_tokens + (size_t)step * batch : nullptr, positions, c.vocab);
+        MH_CHECK_LAUNCH();
+    }
+    if (logits_out && n_steps > 0)
+        MH_CHECK_HIP(hipMemcpyAsync(logits_out, s.logits, (size_t)batch * c.vocab * 2, hipMemcpyDeviceToDevice, st));
+    return MH_OK;
+}
+
+}  // extern "C"

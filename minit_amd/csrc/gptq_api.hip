@@ -19,6 +19,21 @@ int gptq_generic_launch(hipStream_t stream, const void* x, const int32_t* qweigh
 int gemv_gemm_crossover();
 }  // namespace mh
 
+namespace mh {
+// Trusted-argument path for callers inside the library (the decode loop).
+int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                         const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                         void* workspace, size_t workspace_bytes) {
+    if (M <= gemv_gemm_crossover() && gemv_supported(M, N, K, group_size, bits))
+        return gptq_gemv_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
+                                workspace_bytes);
+    if (gemm_supported(M, N, K, group_size, bits))
+        return gptq_gemm_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
+                                workspace_bytes);
+    return gptq_generic_launch(stream, x, qweight, qzeros, scales, nullptr, out, M, N, K, group_size, bits);
+}
+}  // namespace mh
+
 using namespace mh;
 
 extern "C" {

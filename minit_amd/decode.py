@@ -1,0 +1,209 @@
+"""Greedy decode of a Llama-family GPTQ model on one GPU, driven through the
+native loop ``mh_llama_decode`` (one call enqueues every kernel of the requested
+steps).  Mirrors what the reference's cached server does per token
+(examples/llama3_70b.py:394-398 -> Llama3LM.forward -> Top1Sampler) with a
+preallocated KV cache, fused q|k|v and gate|up projections and on-device
+sampling.
+"""
+import ctypes
+import time
+from ctypes import c_float, c_int, c_void_p
+
+import numpy as np
+
+from . import lib, synthetic
+from .hip import memory
+from .hip.tensor import HIPTensor
+
+
+class LlamaConfig(ctypes.Structure):
+    _fields_ = [(n, c_int) for n in ("n_layers", "hidden", "n_q_heads", "n_kv_heads", "head_dim", "ffn",
+                                     "vocab", "group_size", "bits", "max_seq")] + [("rms_eps", c_float)]
+
+
+class QLinear(ctypes.Structure):
+    _fields_ = [("qweight", c_void_p), ("qzeros", c_void_p), ("scales", c_void_p)]
+
+
+class LlamaLayer(ctypes.Structure):
+    _fields_ = [("qkv", QLinear), ("o", QLinear), ("gate_up", QLinear), ("down", QLinear),
+                ("input_norm", c_void_p), ("post_norm", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p)]
+
+
+LLAMA3_70B = dict(n_layers=80, hidden=8192, n_q_heads=64, n_kv_heads=8, head_dim=128, ffn=28672,
+                  vocab=128256, group_size=128, bits=4, rope_theta=5e5, rms_eps=1e-5)
+
+
+class LlamaDecoder:
+    """Owns the device tensors of one model and its KV cache."""
+
+    def __init__(self, config: dict, batch_max: int, max_seq: int):
+        self.config = dict(config)
+        self.batch_max, self.max_seq = batch_max, max_seq
+        c = self.config
+        self._cfg = LlamaConfig(c["n_layers"], c["hidden"], c["n_q_heads"], c["n_kv_heads"], c["head_dim"],
+                                c["ffn"], c["vocab"], c["group_size"], c["bits"], max_seq, c["rms_eps"])
+        h = c_void_p()
+        lib.call("mh_llama_create", ctypes.byref(h), ctypes.byref(self._cfg))
+        self._handle = h.value
+        self._keep = []          # device tensors referenced by the native model
+        self.k_cache, self.v_cache = [], []
+        self._scratch = {}
+        cos, sin = synthetic.rope_tables(c["head_dim"], max_seq, c["rope_theta"])
+        self.cos, self.sin = HIPTensor.from_numpy(cos), HIPTensor.from_numpy(sin)
+
+    def __del__(self):
+        try:
+            lib.call("mh_llama_destroy", self._handle)
+        except Exception:
+            pass
+
+    # ---- weights ------------------------------------------------------------------------------
+    def _alloc_cache(self):
+        c = self.config
+        shape = (self.batch_max, c["n_kv_heads"], self.max_seq, c["head_dim"])
+        return HIPTensor.allocate(shape, "float16"), HIPTensor.allocate(shape, "float16")
+
+    def _set_layer(self, index, linears, input_norm, post_norm, k_cache, v_cache):
+        def ql(t):
+            return QLinear(t[0].data_ptr, t[1].data_ptr, t[2].data_ptr)
+        layer = LlamaLayer(ql(linears["qkv"]), ql(linears["o"]), ql(linears["gate_up"]), ql(linears["down"]),
+                           input_norm.data_ptr, post_norm.data_ptr, k_cache.data_ptr, v_cache.data_ptr)
+        lib.call("mh_llama_set_layer", self._handle, index, ctypes.byref(layer))
+        self._keep.append((linears, input_norm, post_norm))
+        self.k_cache.append(k_cache)
+        self.v_cache.append(v_cache)
+
+    def _set_globals(self, embed, lm_head, final_norm):
+        lib.call("mh_llama_set_globals", self._handle, embed.data_ptr, lm_head.data_ptr, final_norm.data_ptr,
+                 self.cos.data_ptr, self.sin.data_ptr)
+        self._keep.append((embed, lm_head, final_norm))
+        self.embed, self.lm_head, self.final_norm = embed, lm_head, final_norm
+
+    def linear_shapes(self):
+        c = self.config
+        d = c["head_dim"]
+        return {"qkv": (c["hidden"], (c["n_q_heads"] + 2 * c["n_kv_heads"]) * d),
+                "o": (c["n_q_heads"] * d, c["hidden"]),
+                "gate_up": (c["hidden"], 2 * c["ffn"]),
+                "down": (c["ffn"], c["hidden"])}
+
+    def load_synthetic(self, seed: int = 0, prefill: int = 0):
+        """Random-init weights generated on the device; KV cache prefilled with N(0, 1)."""
+        c = self.config
+        per = 32 // c["bits"]
+        g = c["group_size"]
+        for l in range(c["n_layers"]):
+            linears = {}
+            for j, (name, (k, n)) in enumerate(self.linear_shapes().items()):
+                s0 = (seed * 100003 + l) * 16 + j * 3
+                qw = HIPTensor.allocate((k // per, n), "int32")
+                qz = HIPTensor.allocate((k // g, n // per), "int32")
+                sc = HIPTensor.allocate((k // g, n), "float16")
+                lib.call("mh_synth_u32", None, qw.data_ptr, (k // per) * n, s0)
+                lib.call("mh_synth_subwords", None, qz.data_ptr, (k // g) * (n // per), c["bits"], 6, 9, s0 + 1)
+                lib.call("mh_synth_normal", None, sc.data_ptr, (k // g) * n, 0.0, 0.02, 1, 1e-3, s0 + 2, 0)
+                linears[name] = (qw, qz, sc)
+            norms = []
+            for j in range(2):
+                w = HIPTensor.allocate((c["hidden"],), "float16")
+                lib.call("mh_synth_normal", None, w.data_ptr, c["hidden"], 1.0, 0.1, 0, 0.0, s0 + 10 + j, 0)
+                norms.append(w)
+            kc, vc = self._alloc_cache()
+            if prefill:
+                for t, sd in ((kc, 13), (vc, 14)):
+                    lib.call("mh_synth_normal", None, t.data_ptr, int(np.prod(t._shape)), 0.0, 1.0, 0, 0.0,
+                             s0 + sd, 0)
+            self._set_layer(l, linears, norms[0], norms[1], kc, vc)
+        embed = HIPTensor.allocate((c["vocab"], c["hidden"]), "float16")
+        lm_head = HIPTensor.allocate((c["vocab"], c["hidden"]), "float16")
+        final_norm = HIPTensor.allocate((c["hidden"],), "float16")
+        n = c["vocab"] * c["hidden"]
+        lib.call("mh_synth_normal", None, embed.data_ptr, n, 0.0, 0.02, 0, 0.0, seed * 7 + 1, 0)
+        lib.call("mh_synth_normal", None, lm_head.data_ptr, n, 0.0, 0.02, 0, 0.0, seed * 7 + 2, 0)
+        lib.call("mh_synth_normal", None, final_norm.data_ptr, c["hidden"], 1.0, 0.1, 0, 0.0, seed * 7 + 3, 0)
+        self._set_globals(embed, lm_head, final_norm)
+        memory.synchronize()
+
+    def load_host(self, model: dict, k_cache=None, v_cache=None):
+        """Uploads a model given as numpy arrays (the layout of ``oracle.decode``)."""
+        for l, layer in enumerate(model["layers"]):
+            linears = {name: tuple(HIPTensor.from_numpy(np.ascontiguousarray(a)) for a in layer[name][:3])
+                       for name in ("qkv", "o", "gate_up", "down")}
+            kc, vc = self._alloc_cache()
+            if k_cache is not None:
+                kc.copy_from_numpy(k_cache[l])
+                vc.copy_from_numpy(v_cache[l])
+            self._set_layer(l, linears, HIPTensor.from_numpy(layer["input_norm"]),
+                            HIPTensor.from_numpy(layer["post_norm"]), kc, vc)
+        self._set_globals(HIPTensor.from_numpy(model["embed"]), HIPTensor.from_numpy(model["lm_head"]),
+                          HIPTensor.from_numpy(model["final_norm"]))
+
+    # ---- decode ---------------------------------------------------------------------------------
+    def _scratch_for(self, batch):
+        if batch not in self._scratch:
+            nbytes = lib.call("mh_llama_scratch_bytes", self._handle, batch)
+            mem = memory.HIPMemory(nbytes)
+            mem.reset()
+            memory.synchronize()
+            self._scratch[batch] = mem
+        return self._scratch[batch]
+
+    def decode(self, tokens, positions, n_steps: int, want_logits: bool = False, stream=None):
+        """Greedy-decodes ``n_steps`` tokens for ``len(tokens)`` rows.
+
+        Returns ``(out_tokens [n_steps, B] int32, logits of the last step or None)``.
+        """
+        batch = len(tokens)
+        assert batch <= self.batch_max
+        assert int(np.max(positions)) + n_steps <= self.max_seq, "KV cache too short"
+        tok = HIPTensor.from_numpy(np.asarray(tokens, np.int32))
+        pos = HIPTensor.from_numpy(np.asarray(positions, np.int32))
+        out = HIPTensor.allocate((n_steps, batch), "int32")
+        logits = HIPTensor.allocate((batch, self.config["vocab"]), "float16") if want_logits else None
+        scratch = self._scratch_for(batch)
+        lib.call("mh_llama_decode", self._handle, stream, batch, tok.data_ptr, pos.data_ptr, n_steps,
+                 out.data_ptr, logits.data_ptr if logits else None, scratch._pointer, scratch._size)
+        result = out.numpy()
+        return result, (logits.numpy() if logits else None)
+
+    def weight_bytes_per_token(self, batch: int, context: int) -> int:
+        """Algorithmic HBM bytes one decode step has to move."""
+        c = self.config
+        g, bits = c["group_size"], c["bits"]
+        total = 0
+        for k, n in self.linear_shapes().values():
+            total += k * n * bits // 8 + (k // g) * n * 2 + (k // g) * (n * bits // 32) * 4
+        total *= c["n_layers"]
+        total += c["vocab"] * c["hidden"] * 2                                   # lm_head
+        total += c["n_layers"] * batch * 2 * context * c["n_kv_heads"] * c["head_dim"] * 2   # KV read
+        return total
+
+
+def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=print, config=None):
+    """Config 4: 70B-shape GPTQ decode, prefilled KV cache, greedy decode."""
+    cfg = dict(config or LLAMA3_70B)
+    bmax = max(batches)
+    t0 = time.time()
+    dec = LlamaDecoder(cfg, bmax, context + tokens + 8)
+    dec.load_synthetic(seed=1, prefill=context)
+    log(f"decode: model + cache resident after {time.time() - t0:.1f} s")
+    results = []
+    for b in batches:
+        toks = np.arange(b, dtype=np.int32) * 17 + 5
+        pos = np.full(b, context, np.int32)
+        dec.decode(toks, pos, 2)                       # warm-up
+        memory.synchronize()
+        e0, e1 = memory.Event(), memory.Event()
+        e0.record()
+        out, _ = dec.decode(toks, pos, tokens)
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_ms(e1)
+        tps = b * tokens / (ms * 1e-3)
+        gb = dec.weight_bytes_per_token(b, context + tokens // 2) / 1e9
+        results.append({"batch": b, "context": context, "tokens": tokens, "ms_per_token": round(ms / tokens, 3),
+                        "tok_s": round(tps, 1), "algorithmic_gb_per_step": round(gb, 2),
+                        "hbm_gbps": round(gb / (ms / tokens * 1e-3), 1)})
+        log(f"decode batch {b}: {ms / tokens:.3f} ms/token, {tps:.1f} tok/s")
+    return results

@@ -58,6 +58,12 @@ PROTOTYPES = {
     "mh_sum": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_max": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
+    "mh_llama_create": (c_int, [POINTER(c_void_p), _P]),
+    "mh_llama_destroy": (c_int, [_P]),
+    "mh_llama_set_layer": (c_int, [_P, c_int, _P]),
+    "mh_llama_set_globals": (c_int, [_P, _P, _P, _P, _P, _P]),
+    "mh_llama_scratch_bytes": (c_size_t, [_P, c_int]),
+    "mh_llama_decode": (c_int, [_P, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t]),
     "mh_synth_u32": (c_int, [_P, _P, c_size_t, c_uint64]),
     "mh_synth_subwords": (c_int, [_P, _P, c_size_t, c_int, c_uint32, c_uint32, c_uint64]),
     "mh_synth_normal": (c_int, [_P, _P, c_size_t, c_float, c_float, c_int, c_float, c_uint64, c_int]),
@@ -65,7 +71,7 @@ PROTOTYPES = {
 }
 
 # functions whose return value is not a status code
-_NOT_STATUS = {"mh_abi_version", "mh_last_error", "mh_gptq_workspace_bytes"}
+_NOT_STATUS = {"mh_abi_version", "mh_last_error", "mh_gptq_workspace_bytes", "mh_llama_scratch_bytes"}
 
 DTYPE_CODES = {"float16": 0, "bfloat16": 1, "float32": 2}
 

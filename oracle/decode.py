@@ -1,0 +1,80 @@
+"""One greedy decode step of the reference's Llama-family models on the CPU.
+
+Test infrastructure only.  Follows examples/llama3_70b.py:77-162,215-249 op by
+op, rounding to fp16 wherever the reference materialises an fp16 tensor:
+RMSNorm (eps from the model), q/k/v projections, interleaved RoPE at the row's
+position, K/V appended to the cache, scores = q.k^T (fp32 accumulate, fp16
+store), ``/ sqrt(d)`` in fp16, the additive causal mask (identically zero for a
+single new token), softmax, P.V, output projection, residual adds in fp16,
+``silu(gate) * up`` with its three roundings, and the lm_head product against
+``[vocab, hidden]``; sampling is ``argmax`` (minit/chat/sample.py:11-14).
+
+Grouped-query attention: query head j uses KV head ``j // (QH / KVH)``
+(the reference repeats each KV head, llama3_70b.py:85-93).
+"""
+import numpy as np
+
+from . import gptq, special
+
+
+def _linear(x, w):
+    """``w`` is ``(qweight, qzeros, scales, group_size)``."""
+    qweight, qzeros, scales, group_size = w
+    return gptq.matmul(x, qweight, qzeros, scales, None, 4, group_size)
+
+
+def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache: list, v_cache: list):
+    """Returns fp16 logits ``[B, vocab]``; caches ``[B, KVH, T, D]`` are updated in place."""
+    cfg = model["config"]
+    qh, kvh, d = cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    rep = qh // kvh
+    eps = cfg["rms_eps"]
+    b = len(tokens)
+    h = model["embed"][tokens].astype(np.float16)                      # [B, H]
+    cos, sin = model["cos"], model["sin"]
+    inv_sqrt_d = np.float16(np.sqrt(np.float64(d)))
+    for l, layer in enumerate(model["layers"]):
+        xn = special.rms_norm(h, layer["input_norm"], 1, eps)
+        qkv = _linear(xn, layer["qkv"])
+        q = qkv[:, :qh * d].reshape(b, 1, qh, d)
+        k = qkv[:, qh * d:(qh + kvh) * d].reshape(b, 1, kvh, d)
+        v = qkv[:, (qh + kvh) * d:].reshape(b, kvh, d)
+        pos = positions.reshape(b, 1)
+        q = special.rope(q, cos, sin, pos)[:, 0]                       # [B, QH, D]
+        k = special.rope(k, cos, sin, pos)[:, 0]                       # [B, KVH, D]
+        attn = np.zeros((b, qh, d), np.float16)
+        for i in range(b):
+            p = int(positions[i])
+            k_cache[l][i, :, p] = k[i]
+            v_cache[l][i, :, p] = v[i]
+            kk = k_cache[l][i, :, :p + 1].astype(np.float64)           # [KVH, T, D]
+            vv = v_cache[l][i, :, :p + 1].astype(np.float64)
+            for j in range(qh):
+                g = j // rep
+                scores = (kk[g] @ q[i, j].astype(np.float64)).astype(np.float16)
+                scores = (scores / inv_sqrt_d).astype(np.float16)      # fp16 division
+                probs = special.softmax(scores[None, :], 1)[0]
+                attn[i, j] = (probs.astype(np.float64) @ vv[g]).astype(np.float16)
+        o = _linear(attn.reshape(b, qh * d), layer["o"])
+        h = h + o                                                      # fp16 add
+        xn = special.rms_norm(h, layer["post_norm"], 1, eps)
+        gu = _linear(xn, layer["gate_up"])
+        f = gu.shape[1] // 2
+        act = gptq.silu_mul(gu[:, :f], gu[:, f:])
+        h = h + _linear(act, layer["down"])
+    xn = special.rms_norm(h, model["final_norm"], 1, eps)
+    return gptq.dense_matmul(xn, model["lm_head"].T.astype(np.float16))
+
+
+def greedy(model, tokens, positions, k_cache, v_cache, n_steps):
+    """Returns ``(out_tokens [n_steps, B], logits of every step)``."""
+    tokens = np.array(tokens, np.int64)
+    positions = np.array(positions, np.int64)
+    out, all_logits = [], []
+    for _ in range(n_steps):
+        logits = decode_step(model, tokens, positions, k_cache, v_cache)
+        tokens = logits.astype(np.float32).argmax(axis=-1)
+        positions = positions + 1
+        out.append(tokens.copy())
+        all_logits.append(logits)
+    return np.stack(out), all_logits
