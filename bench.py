@@ -115,6 +115,9 @@ def main():
     ap.add_argument("--layers", type=int, default=6, help="distinct weight sets cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only the plain copy kernel (1 GiB read + 1 GiB write per launch) that the "
+                         "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         log(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
@@ -131,6 +134,23 @@ def main():
         sys.exit(1)
     info = lib.device_info()
     log("device:", info)
+
+    if args.calibrate_copy:
+        nbytes = 1 << 30
+        src, dst = memory.HIPMemory(nbytes), memory.HIPMemory(nbytes)
+        src.reset()
+        dst.reset()
+        memory.synchronize()
+        e0, e1 = memory.Event(), memory.Event()
+        e0.record()
+        for _ in range(5):
+            lib.call("mh_copy_kernel", None, src._pointer, dst._pointer, nbytes)
+        e1.record()
+        e1.synchronize()
+        us = e0.elapsed_ms(e1) * 1e3 / 5
+        print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
+                          "us": round(us, 1), "gbps_read_plus_write": round(2 * nbytes / us / 1e3, 1)}))
+        return
 
     # ---- inputs, resident in HBM before the timed region ------------------------------------
     t0 = time.time()

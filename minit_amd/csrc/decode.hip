@@ -142,39 +142,46 @@ __global__ void silu_mul_fused_kernel(const half_t* __restrict__ gu, half_t* __r
 
 // token[b] = argmax_v logits[b, v] (first maximum); appended to the output
 // stream and fed back as the next input; positions[b] += 1.
-__global__ __launch_bounds__(256) void argmax_advance_kernel(const half_t* __restrict__ logits,
-                                                             int32_t* __restrict__ tokens,
-                                                             int32_t* __restrict__ out_tokens,
-                                                             int32_t* __restrict__ positions, int vocab) {
-    __shared__ float sval[256];
-    __shared__ int sidx[256];
+__global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __restrict__ logits,
+                                                              int32_t* __restrict__ tokens,
+                                                              int32_t* __restrict__ out_tokens,
+                                                              int32_t* __restrict__ positions, int vocab) {
+    __shared__ float sval[16];
+    __shared__ int sidx[16];
     const int b = blockIdx.x;
     const half_t* row = logits + (size_t)b * vocab;
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    for (int v = threadIdx.x; v < vocab; v += blockDim.x) {
-        const float x = (float)row[v];
+    auto consider = [&](float x, int v) {
         if (x > best || (x == best && v < best_i)) {
             best = x;
             best_i = v;
         }
+    };
+    const bool aligned = ((uintptr_t)row % 16) == 0;
+    const int nvec = aligned ? vocab / 8 : 0;
+    for (int i = threadIdx.x; i < nvec; i += blockDim.x) {
+        const half8_t v = __builtin_bit_cast(half8_t, reinterpret_cast<const uint4*>(row)[i]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) consider((float)v[e], i * 8 + e);
     }
-    sval[threadIdx.x] = best;
-    sidx[threadIdx.x] = best_i;
+    for (int v = nvec * 8 + threadIdx.x; v < vocab; v += blockDim.x) consider((float)row[v], v);
+    // wave reduction, then across the 16 waves
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(best_i, off, 64);
+        consider(o, oi);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        sval[wave] = best;
+        sidx[wave] = best_i;
+    }
     __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if ((int)threadIdx.x < off) {
-            const float o = sval[threadIdx.x + off];
-            const int oi = sidx[threadIdx.x + off];
-            if (o > sval[threadIdx.x] || (o == sval[threadIdx.x] && oi < sidx[threadIdx.x])) {
-                sval[threadIdx.x] = o;
-                sidx[threadIdx.x] = oi;
-            }
-        }
-        __syncthreads();
-    }
     if (threadIdx.x == 0) {
-        const int tok = sidx[0] == 0x7fffffff ? 0 : sidx[0];
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w) consider(sval[w], sidx[w]);
+        const int tok = best_i == 0x7fffffff ? 0 : best_i;
         tokens[b] = tok;
         if (out_tokens) out_tokens[b] = tok;
         positions[b] += 1;
@@ -237,9 +244,18 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
         for (int h = 0; h < G; ++h) s[h] = 0.f;
         const uint4* krow = reinterpret_cast<const uint4*>(kbase + (size_t)(valid ? t : t0) * D);
+        uint4 kq[CH], vq[16];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) kq[c] = krow[c];
+        // the V rows of phase B are requested now so both streams are in flight together
+#pragma unroll
+        for (int tt = 0; tt < 16; ++tt) {
+            const int tv = min(c0 + tt * 4 + tg, t1 - 1);
+            vq[tt] = reinterpret_cast<const uint4*>(vbase + (size_t)tv * D)[dl];
+        }
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const uint4 kv = krow[c];
+            const uint4 kv = kq[c];
             const half2_t k0 = __builtin_bit_cast(half2_t, kv.x), k1 = __builtin_bit_cast(half2_t, kv.y),
                           k2 = __builtin_bit_cast(half2_t, kv.z), k3 = __builtin_bit_cast(half2_t, kv.w);
 #pragma unroll
@@ -265,13 +281,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         }
         __builtin_amdgcn_wave_barrier();
         // ---- phase B
-#pragma unroll 4
+#pragma unroll
         for (int tt = 0; tt < 16; ++tt) {
             const int tl = tt * 4 + tg;
-            const int tv = c0 + tl;
-            if (tv < t1) {
-                const uint4 vv = reinterpret_cast<const uint4*>(vbase + (size_t)tv * D)[dl];
-                const half8_t vh = __builtin_bit_cast(half8_t, vv);
+            if (c0 + tl < t1) {
+                const half8_t vh = __builtin_bit_cast(half8_t, vq[tt]);
 #pragma unroll
                 for (int h = 0; h < G; ++h) {
                     const float p = p_s[wave][h][tl];
@@ -334,19 +348,48 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
     __shared__ int is_last;
     if (!arrive_and_check_last(counters + (size_t)b * kvh + g, (unsigned)splits, &is_last)) return;
+    // Last block: merge the splits.  First the per-split maxima and sums of every
+    // head (independent loads, a few per thread) become weights in LDS, then each
+    // thread sums its output element over the splits.
+    constexpr int kMaxSplits = 64;
+    __shared__ float w_s[G][kMaxSplits];
+    __shared__ float l_tot[G];
+    float* ml = &acc_s[0][0][0];  // reuse: [G][splits][2]
+    for (int i = tid; i < G * splits; i += 256) {
+        const int h = i / splits, sp = i % splits;
+        const float* pp = partial + ((head0 + h) * splits + sp) * (D + 2);
+        ml[2 * i] = load_agent(pp);
+        ml[2 * i + 1] = load_agent(pp + 1);
+    }
+    __syncthreads();
+    if (tid < G) {
+        const int h = tid;
+        float mm = -INFINITY;
+        for (int sp = 0; sp < splits; ++sp) mm = fmaxf(mm, ml[2 * (h * splits + sp)]);
+        float ll = 0.f;
+        for (int sp = 0; sp < splits; ++sp) {
+            const float ms = ml[2 * (h * splits + sp)];
+            const float f = (ms == -INFINITY) ? 0.f : expf(ms - mm);
+            w_s[h][sp] = f;
+            ll += ml[2 * (h * splits + sp) + 1] * f;
+        }
+        l_tot[h] = ll;
+    }
+    __syncthreads();
     for (int i = tid; i < ITEMS; i += 256) {
         const int h = i / D, d = i % D;
-        const float* pp = partial + (head0 + h) * splits * (D + 2);
-        float mm = -INFINITY;
-        for (int sp = 0; sp < splits; ++sp) mm = fmaxf(mm, load_agent(pp + (size_t)sp * (D + 2)));
-        float ll = 0.f, a = 0.f;
-        for (int sp = 0; sp < splits; ++sp) {
-            const float ms = load_agent(pp + (size_t)sp * (D + 2));
-            const float f = (ms == -INFINITY) ? 0.f : expf(ms - mm);
-            ll += load_agent(pp + (size_t)sp * (D + 2) + 1) * f;
-            a += load_agent(pp + (size_t)sp * (D + 2) + 2 + d) * f;
+        const float* pp = partial + (head0 + h) * splits * (D + 2) + 2 + d;
+        float a = 0.f;
+        int sp = 0;
+        for (; sp + 8 <= splits; sp += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = load_agent(pp + (size_t)(sp + u) * (D + 2));
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a += v[u] * w_s[h][sp + u];
         }
-        out[(head0 + h) * D + d] = (half_t)(a / ll);
+        for (; sp < splits; ++sp) a += load_agent(pp + (size_t)sp * (D + 2)) * w_s[h][sp];
+        out[(head0 + h) * D + d] = (half_t)(a / l_tot[h]);
     }
 }
 
@@ -376,6 +419,7 @@ static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
 static int attn_splits(const Llama& m, int batch) {
     const int pairs = batch * m.cfg.n_kv_heads;
     int splits = (2 * compute_units() + pairs - 1) / pairs;
+    // a block walks 256 positions per pass of its four waves
     const int max_splits = (m.cfg.max_seq + 255) / 256;
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
@@ -541,7 +585,7 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
         }
         int rc = mh_f16_matmul_nk(stream, s.xn, m->lm_head, s.logits, batch, c.vocab, c.hidden);
         if (rc) return rc;
-        hipLaunchKernelGGL(argmax_advance_kernel, dim3(batch), dim3(256), 0, st, s.logits, tokens,
+        hipLaunchKernelGGL(argmax_advance_kernel, dim3(batch), dim3(1024), 0, st, s.logits, tokens,
                            out_tokens ? out_tokens + (size_t)step * batch : nullptr, positions, c.vocab);
         MH_CHECK_LAUNCH();
     }
