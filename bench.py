@@ -6,7 +6,8 @@
 One *step* is one pass of the decode hot path over one layer's worth of
 Llama-3-70B-shape GPTQ 4-bit weights at M = 1: the four quantized linears
 (qkv 8192x10240, o 8192x8192, gate|up 8192x57344, down 28672x8192, group 128)
-through ``mh_gptq_gemv``.  ``--layers`` distinct weight sets (default 6,
+through ``mh_gptq_matmul`` (the library's dispatch; ``--entry`` times the VALU
+GEMV or the MFMA kernel explicitly).  ``--layers`` distinct weight sets (default 6,
 2.6 GB -- ten times the 256 MB Infinity Cache) are generated on the device and
 cycled, so every step streams its weights from HBM.  The value reported is
 algorithmic bytes per second: packed weights + scales + zero points +
@@ -68,7 +69,7 @@ class DeviceLinear:
         lib.call("mh_synth_normal", None, self.scales.data_ptr, groups * n, 0.0, 0.02, 1, 1e-3, seed * 3 + 2, 0)
 
 
-def run_gemv(lib, x, lin, out, ws, m=1, entry="mh_gptq_gemv"):
+def run_gemv(lib, x, lin, out, ws, m=1, entry="mh_gptq_matmul"):
     lib.call(entry, None, x.data_ptr, lin.qweight.data_ptr, lin.qzeros.data_ptr, lin.scales.data_ptr, None,
              out.data_ptr, m, lin.n, lin.k, GROUP, BITS, ws._pointer, ws._size)
 
@@ -115,10 +116,16 @@ def main():
     ap.add_argument("--layers", type=int, default=6, help="distinct weight sets cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--shapes-only", action="store_true",
+                    help="of the extras, keep only the per-shape GEMV breakdown")
+    ap.add_argument("--entry", default="mh_gptq_matmul", choices=["mh_gptq_matmul", "mh_gptq_gemv", "mh_gptq_gemm"],
+                    help="C-ABI entry point timed: the library's own dispatch (default), the VALU GEMV, "
+                         "or the MFMA kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel (1 GiB read + 1 GiB write per launch) that the "
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
     args = ap.parse_args()
+    ENTRY = args.entry
     if args.gpus != 1:
         log(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
             "(no collectives or sharding in this path).")
@@ -171,7 +178,7 @@ def main():
 
     def step(i):
         for lin in layers[i % args.layers]:
-            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws)
+            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
 
     for i in range(args.warmup):
         step(i)
@@ -215,7 +222,8 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gptq_gemv_kernel<4,1,8>",
+            "kernel": "gptq_gemv_kernel<4,1,8>" if ENTRY == "mh_gptq_gemv" else "gptq_gemm_small_kernel<4,1,4>",
+            "entry": ENTRY,
             "achieved": round(gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -231,22 +239,25 @@ def main():
         per_shape = {}
         for j, (name, k, n) in enumerate(LINEARS):
             for i in range(3):
-                run_gemv(lib, xs[k], layers[i % args.layers][j], outs[n], ws)
+                run_gemv(lib, xs[k], layers[i % args.layers][j], outs[n], ws, entry=ENTRY)
             memory.synchronize()
             a, b = memory.Event(), memory.Event()
             a.record()
             for i in range(50):
-                run_gemv(lib, xs[k], layers[i % args.layers][j], outs[n], ws)
+                run_gemv(lib, xs[k], layers[i % args.layers][j], outs[n], ws, entry=ENTRY)
             b.record()
             b.synchronize()
             us = a.elapsed_ms(b) * 1e3 / 50
             per_shape[name] = {"us": round(us, 2), "gbps": round(linear_bytes(1, k, n) / us / 1e3, 1)}
         result["extra"] = {"gemv_per_shape": per_shape}
         try:
-            result["extra"]["int8_gemm"] = [bench_int8(lib, HIPTensor, memory, n) for n in (4096, 11008)]
+            if not args.shapes_only:
+                result["extra"]["int8_gemm"] = [bench_int8(lib, HIPTensor, memory, n) for n in (4096, 11008)]
         except Exception as exc:  # report, do not hide
             result["extra"]["int8_gemm_error"] = str(exc)
         try:
+            if args.shapes_only:
+                raise RuntimeError("skipped (--shapes-only)")
             from minit_amd import decode
             result["extra"]["decode_70b"] = decode.bench_tokens_per_second(batches=(1,), tokens=16, log=log)
         except Exception as exc:
@@ -264,7 +275,7 @@ def main():
         # GPU results for layer 0, to check against what the CPU computes
         gpu_out = []
         for lin in layers[0]:
-            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws)
+            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
             gpu_out.append(outs[lin.n].numpy().copy())
         times, worst = [], 0.0
         for rep in range(2):

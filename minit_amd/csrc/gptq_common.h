@@ -123,11 +123,4 @@ int check_gptq_args(const char* who, const void* x, const void* qweight, const v
                     const void* scales, const void* out, int M, int N, int K, int group_size,
                     int bits);
 
-// Workspace layout shared by the split-K kernels: a fixed region of arrival
-// counters first (one per output tile, zero between launches), fp32 partial
-// sums after it.  The counter region has one size for every shape so that the
-// partials of one call can never land where a later call keeps its counters.
-constexpr size_t kCounterRegionBytes = 64 * 1024;
-constexpr int kMaxCounters = (int)(kCounterRegionBytes / sizeof(unsigned));
-
 }  // namespace mh

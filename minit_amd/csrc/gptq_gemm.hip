@@ -12,8 +12,8 @@
 // the activations instead, when they are staged into LDS, so both operands
 // agree.  A block is four waves side by side along N (256 columns, 1 KiB
 // contiguous per packed row) sharing one activation tile [16*MT, KC] in LDS.
-// K is split over blockIdx.y with fp32 partials summed in split order by the
-// last block to arrive (deterministic).
+// K is split over blockIdx.y with fp32 partials summed in split order by a
+// second, tiny kernel (deterministic; see gptq_gemv.hip).
 #include "gptq_common.h"
 
 namespace mh {
@@ -29,7 +29,7 @@ template <int BITS, int MT>
 __global__ __launch_bounds__(256) void gptq_gemm_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
-    half_t* __restrict__ out, float* partial, unsigned* counters,
+    half_t* __restrict__ out, float* __restrict__ partial,
     int M, int N, int K, int steps_per_group, int steps_total, int steps_per_block, int split_k) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
@@ -202,6 +202,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_kernel(
         return;
     }
 
+    // split-K: fp32 partials, summed in split order by splitk_finalize_kernel
     if (active) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -210,43 +211,207 @@ __global__ __launch_bounds__(256) void gptq_gemm_kernel(
                 const int m = m0 + mt * 16 + kq * 4 + r;
                 if (m < M) {
                     float* p = partial + ((size_t)split * M + m) * N + col;
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) store_agent(p + t, acc[mt][t][r]);
+                    *reinterpret_cast<float4_t*>(p) =
+                        float4_t{acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
                 }
             }
     }
-    __shared__ int is_last;
-    if (!arrive_and_check_last(counters + (size_t)mblock * gridDim.x + tile, (unsigned)split_k, &is_last))
-        return;
-    if (active) {
+}
+
+void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, size_t mn, int split_k);
+
+// ---- small-M variant (M <= 32: decode batches) --------------------------------------------------
+// Same operand mapping, a schedule built around two facts measured on this part:
+// (1) the weight stream only stays pipelined if every vector-memory load sits at
+// a fixed place in a branch-free loop body -- then the compiler can wait with an
+// exact s_waitcnt vmcnt(n); a branch around a load makes it wait for everything,
+// and without a scheduling barrier it sinks the ring reloads to the end of the
+// body; (2) with 13 VALU ops per packed word the kernel is close to VALU-bound,
+// so nothing else may cost vector instructions (addresses are scalar base + a
+// fixed lane offset, per-group constants arrive precomputed from LDS).
+//
+// K is walked in stages of 8 steps (256 k).  While a stage is consumed, the
+// activations and per-group constants of the next one travel global -> registers
+// -> the other LDS buffer; one barrier per stage.  The ring keeps 8 KiB of
+// weights per wave in flight at all times.
+constexpr int kSmallDepth = 8;  // steps per stage = ring depth
+
+template <int BITS, int MT, int SPG>
+__global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
+    half_t* __restrict__ out, float* __restrict__ partial,
+    int M, int N, int K, int steps_total, int stages_per_block, int split_k) {
+    constexpr int P = Packing<BITS>::kPerWord;
+    constexpr int PAIRS = Packing<BITS>::kPairs;
+    constexpr uint32_t MASK = Packing<BITS>::kMask;
+    constexpr int ROWS_PER_STEP = 32 / P;
+    constexpr int LOADS = ROWS_PER_STEP / 4;
+    constexpr int D = kSmallDepth;
+    constexpr int GPS = D / SPG;            // groups per stage
+    constexpr int BM = 16 * MT;
+    constexpr int XCH = D * 4;              // 16-byte activation chunks per row per stage
+    constexpr int RS = XCH + 1;             // padded row stride
+    constexpr int XL = BM * XCH / 256;      // chunks each thread stages: 2 (MT=1) or 4 (MT=2)
+    static_assert(D % SPG == 0, "a stage must hold whole groups");
+
+    __shared__ uint4 xs[2][BM * RS];
+    __shared__ uint32_t cs[2][GPS][3][kGemmCols];  // scale pair, zero_lo pair, zero_hi pair
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nl = lane & 15, kq = lane >> 4;
+    const int tile = blockIdx.x, split = blockIdx.y;
+    const int lcol = wave * 64 + nl * 4;
+    const int col = tile * kGemmCols + lcol;
+    const bool active = col < N;
+    const int colc = active ? col : 0;
+
+    const int step_begin = split * stages_per_block * D;
+    const int last_step = steps_total - 1;
+    const int g_last = last_step / SPG;
+
+    // ---- weight ring
+    uint4_t qb[D][LOADS];
+    uint32_t lane_off[LOADS];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+    for (int j = 0; j < LOADS; ++j) lane_off[j] = (uint32_t)((kq * LOADS + j) * N + colc) * 4u;
+    auto load_q = [&](int step, uint4_t* dst) {
+        const int s = min(step, last_step);
+        const char* base = reinterpret_cast<const char*>(qweight) + (size_t)s * ROWS_PER_STEP * N * 4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int m = m0 + mt * 16 + kq * 4 + r;
-                if (m < M) {
-                    float s[4] = {0.f, 0.f, 0.f, 0.f};
-                    const float* p = partial + (size_t)m * N + col;
-                    int sp = 0;
-                    for (; sp + 4 <= split_k; sp += 4) {
-                        float v[4][4];
+        for (int j = 0; j < LOADS; ++j)
+            dst[j] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(base + lane_off[j]));
+    };
 #pragma unroll
-                        for (int u = 0; u < 4; ++u)
+    for (int d = 0; d < D; ++d) load_q(step_begin + d, qb[d]);
+
+    // ---- staging of activations and constants: global -> registers -> LDS
+    uint4 xr[XL];
+    uint4 sr;       // eight scales of one group
+    uint32_t zr[8 / P];
+    int x_row[XL], x_chunk[XL];
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) v[u][t] = load_agent(p + (size_t)(sp + u) * M * N + t);
+    for (int u = 0; u < XL; ++u) {
+        const int idx = u * 256 + tid;
+        x_row[u] = min(idx / XCH, M - 1);  // rows >= M only feed accumulator rows that are never stored
+        x_chunk[u] = idx % XCH;
+    }
+    const int c_group = (tid >> 5) % GPS, c_col8 = tid & 31;  // threads 0 .. 32*GPS-1 stage the constants
+    const int c_colg = min(tile * kGemmCols + c_col8 * 8, N - 8);
+    auto fetch_stage = [&](int stage_step) {
+        const int sclamp = min(stage_step, (last_step / D) * D);  // never read past K
 #pragma unroll
-                        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < XL; ++u)
+            xr[u] = *reinterpret_cast<const uint4*>(x + (size_t)x_row[u] * K + (size_t)sclamp * 32 + x_chunk[u] * 8);
+        const int g = min(sclamp / SPG + c_group, g_last);
+        sr = *reinterpret_cast<const uint4*>(scales + (size_t)g * N + c_colg);
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) s[t] += v[u][t];
-                    }
-                    for (; sp < split_k; ++sp)
+        for (int j = 0; j < 8 / P; ++j) zr[j] = qzeros[(size_t)g * (N / P) + c_colg / P + j];
+    };
+    auto store_stage = [&](int buf, int stage_step) {
 #pragma unroll
-                        for (int t = 0; t < 4; ++t) s[t] += load_agent(p + (size_t)sp * M * N + t);
-                    const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+        for (int u = 0; u < XL; ++u) {
+            const uint32_t in[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+            uint32_t o[4];
+            if constexpr (BITS == 4) {
+                pair_activations<4>(in, o);
+            } else {
+                pair_activations<8>(in, o);
+                pair_activations<8>(in + 2, o + 2);
+            }
+            // steps past the end of K contribute nothing
+            const bool live = stage_step + x_chunk[u] / 4 <= last_step;
+            xs[buf][(u * 256 + tid) / XCH * RS + x_chunk[u]] =
+                live ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
+        }
+        if (tid < 32 * GPS) {
+            const half_t* sh = reinterpret_cast<const half_t*>(&sr);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t z = (zr[j / P] >> ((j % P) * BITS)) & MASK;
+                const ColumnConst k = make_column_const(sh[j], z);
+                cs[buf][c_group][0][c_col8 * 8 + j] = as_u32(k.scale);
+                cs[buf][c_group][1][c_col8 * 8 + j] = as_u32(k.zero_lo);
+                cs[buf][c_group][2][c_col8 * 8 + j] = as_u32(k.zero_hi);
+            }
+        }
+    };
+
+    fetch_stage(step_begin);
+    store_stage(0, step_begin);
+    fetch_stage(step_begin + D);
+    __syncthreads();
+
+    DequantRegs regs;
+    regs.init(BITS);
+    float4_t acc[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[mt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    ColumnConst cc[4];
+
+    for (int stage = 0; stage < stages_per_block; ++stage) {
+        const int buf = stage & 1;
+        const int stage_step = step_begin + stage * D;
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (d % SPG == 0) {  // compile-time: a new group starts here
+                const uint4 sc4 = *reinterpret_cast<const uint4*>(&cs[buf][d / SPG][0][lcol]);
+                const uint4 lo4 = *reinterpret_cast<const uint4*>(&cs[buf][d / SPG][1][lcol]);
+                const uint4 hi4 = *reinterpret_cast<const uint4*>(&cs[buf][d / SPG][2][lcol]);
+                cc[0] = ColumnConst{as_half2(sc4.x), as_half2(lo4.x), as_half2(hi4.x)};
+                cc[1] = ColumnConst{as_half2(sc4.y), as_half2(lo4.y), as_half2(hi4.y)};
+                cc[2] = ColumnConst{as_half2(sc4.z), as_half2(lo4.z), as_half2(hi4.z)};
+                cc[3] = ColumnConst{as_half2(sc4.w), as_half2(lo4.w), as_half2(hi4.w)};
+            }
+            half8_t b[4];
+            uint4_t* q = qb[d];
+            const uint32_t qa[4] = {q[0].x, q[0].y, q[0].z, q[0].w};
+            const uint32_t qc[4] = {q[LOADS - 1].x, q[LOADS - 1].y, q[LOADS - 1].z, q[LOADS - 1].w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                half2_t w[4];
+                dequant_word<BITS>(qa[t], cc[t], regs, w);
+                if constexpr (BITS == 8) dequant_word<BITS>(qc[t], cc[t], regs, w + PAIRS);
+                const uint4_t packed = {as_u32(w[0]), as_u32(w[1]), as_u32(w[2]), as_u32(w[3])};
+                b[t] = __builtin_bit_cast(half8_t, packed);
+            }
+            load_q(stage_step + d + D, q);
+            __builtin_amdgcn_sched_barrier(0);  // keep the reload here (see above)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const half8_t a = __builtin_bit_cast(half8_t, xs[buf][(mt * 16 + nl) * RS + d * 4 + kq]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[mt][t], 0, 0, 0);
+            }
+        }
+        store_stage(buf ^ 1, stage_step + D);
+        fetch_stage(stage_step + 2 * D);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    }
+
+    if (!active) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = mt * 16 + kq * 4 + r;
+            if (m < M) {
+                if (split_k == 1) {
+                    const half4_t h = {(half_t)acc[mt][0][r], (half_t)acc[mt][1][r], (half_t)acc[mt][2][r],
+                                       (half_t)acc[mt][3][r]};
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
+                } else {
+                    *reinterpret_cast<float4_t*>(partial + ((size_t)split * M + m) * N + col) =
+                        float4_t{acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
                 }
             }
-    }
+        }
 }
 
 // ---- host side ---------------------------------------------------------------------------------------
@@ -266,7 +431,40 @@ static int env_int_gemm(const char* name, int fallback) {
     return atoi(v);
 }
 
-GemmPlan plan_gemm(int M, int N, int K) {
+constexpr int kSmallMaxM = 32;
+
+// Plan of the small-M kernel: column tiles x K splits sized so the GPU holds
+// about MH_GEMM_SMALL_WAVES_PER_CU waves per CU; a block walks whole stages.
+// GemmPlan::steps_per_block carries stages_per_block * kSmallDepth.
+GemmPlan plan_gemm_small(int M, int N, int K) {
+    GemmPlan p;
+    p.mt = M <= 16 ? 1 : 2;
+    p.col_tiles = (N + kGemmCols - 1) / kGemmCols;
+    p.m_blocks = 1;
+    p.steps_total = K / 32;
+    const long stages_total = (p.steps_total + kSmallDepth - 1) / kSmallDepth;
+    static const int waves_per_cu = env_int_gemm("MH_GEMM_SMALL_WAVES_PER_CU", 8);
+    const long target_blocks = (long)compute_units() * waves_per_cu / 4;
+    long split = target_blocks / p.col_tiles;
+    if (split > stages_total) split = stages_total;
+    // fp32 partials cost 8*M*N bytes per split against K*N/2 bytes of weights
+    const long traffic_cap = K / (32L * M) > 1 ? K / (32L * M) : 1;
+    if (split > traffic_cap) split = traffic_cap;
+    if (split < 1) split = 1;
+    const long spb = (stages_total + split - 1) / split;
+    p.steps_per_block = (int)(spb * kSmallDepth);
+    p.split_k = (int)((stages_total + spb - 1) / spb);
+    return p;
+}
+
+static bool use_small(int M, int group_size) {
+    static const int off = env_int_gemm("MH_GEMM_NO_SMALL", 0);
+    const int spg = group_size / 32;
+    return !off && M <= kSmallMaxM && (spg == 1 || spg == 2 || spg == 4 || spg == 8);
+}
+
+GemmPlan plan_gemm(int M, int N, int K, int group_size) {
+    if (use_small(M, group_size)) return plan_gemm_small(M, N, K);
     GemmPlan p;
     p.mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
     const int bm = 16 * p.mt;
@@ -284,7 +482,6 @@ GemmPlan plan_gemm(int M, int N, int K) {
     const long traffic_cap = K / (64L * M) > 1 ? K / (64L * M) : 1;
     if (max_split > traffic_cap) max_split = traffic_cap;
     if (split > max_split) split = max_split;
-    if ((long)p.col_tiles * p.m_blocks > kMaxCounters) split = 1;  // no counter for that many tiles
     if (split < 1) split = 1;
     long spb = (p.steps_total + split - 1) / split;
     spb = (spb + sc - 1) / sc * sc;
@@ -299,29 +496,54 @@ bool gemm_supported(int M, int N, int K, int group_size, int bits) {
 }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
-    (void)group_size;
     (void)bits;
-    const GemmPlan p = plan_gemm(M, N, K);
-    size_t partial = (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
-    return kCounterRegionBytes + partial;
+    const GemmPlan p = plan_gemm(M, N, K, group_size);
+    return (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
 }
 
 template <int BITS, int MT>
 static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                         const int32_t* qzeros, const void* scales, void* out, void* workspace, int M, int N,
                         int K, int group_size) {
-    unsigned* counters = reinterpret_cast<unsigned*>(workspace);
-    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterRegionBytes);
+    float* partial = reinterpret_cast<float*>(workspace);
     hipLaunchKernelGGL((gptq_gemm_kernel<BITS, MT>), dim3(p.col_tiles, p.split_k, p.m_blocks), dim3(256), 0,
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
-                       (const half_t*)scales, (half_t*)out, partial, counters, M, N, K, group_size / 32,
+                       (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size / 32,
                        p.steps_total, p.steps_per_block, p.split_k);
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
+}
+
+template <int BITS, int MT>
+static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
+                              const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
+                              int N, int K, int group_size) {
+    float* partial = reinterpret_cast<float*>(workspace);
+    const dim3 grid(p.col_tiles, p.split_k);
+#define MH_LAUNCH_SMALL(SPG)                                                                                  \
+    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG>), grid, dim3(256), 0, stream, (const half_t*)x,  \
+                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,  \
+                       partial, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k)
+    switch (group_size / 32) {
+        case 1: MH_LAUNCH_SMALL(1); break;
+        case 2: MH_LAUNCH_SMALL(2); break;
+        case 4: MH_LAUNCH_SMALL(4); break;
+        default: MH_LAUNCH_SMALL(8); break;
+    }
+#undef MH_LAUNCH_SMALL
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
 }
 
 template <int BITS>
 static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                            const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
                            int N, int K, int group_size) {
+    if (use_small(M, group_size)) {
+        if (p.mt == 1)
+            launch_gemm_small<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+        else
+            launch_gemm_small<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+        return;
+    }
     switch (p.mt) {
         case 1: launch_gemm<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size); break;
         case 2: launch_gemm<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size); break;
@@ -333,7 +555,7 @@ static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x,
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                      void* workspace, size_t workspace_bytes) {
-    const GemmPlan p = plan_gemm(M, N, K);
+    const GemmPlan p = plan_gemm(M, N, K, group_size);
     const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
     if (p.split_k > 1) {
         if (workspace == nullptr || workspace_bytes < need)
@@ -351,7 +573,8 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
 }
 
 int gemv_gemm_crossover() {
-    static const int m = env_int_gemm("MH_GEMV_MAX_M", MH_GPTQ_GEMV_MAX_M);
+    // measured on MI355X: the MFMA kernel is at least as fast from M = 1 on
+    static const int m = env_int_gemm("MH_GEMV_MAX_M", 0);
     return m < MH_GPTQ_GEMV_MAX_M ? m : MH_GPTQ_GEMV_MAX_M;
 }
 

@@ -1,20 +1,25 @@
 // GPTQ w4a16 / w8a16 dequant-GEMV for decode (M <= 4), wave64 VALU, no MFMA.
 //
 // Replaces the fused qmm kernel of the reference
-// (examples/qwen1_5_int8.py:156-216) for small M.  Bandwidth-bound design:
+// (examples/qwen1_5_int8.py:156-216) for small M without the matrix cores.
 //
 //   * qweight [K/P, N] is N-contiguous, so lanes walk N: a lane owns four
-//     adjacent columns and fetches them with one 16-byte load per packed row;
-//     a wave therefore streams 1 KiB-contiguous row segments.
-//   * the packed rows a wave walks are wave-uniform, so the activations it
-//     needs are uniform too and live in scalar registers; each dequantised
-//     fp16 pair is consumed by one v_dot2_f32_f16 per output row.
-//   * K is split three ways: over the four waves of a block (reduced through
-//     LDS), over blockIdx.y (fp32 partials in the workspace, summed in a fixed
-//     order by whichever block finishes last -- deterministic, no atomics on
-//     data), and within a lane (private fp32 accumulators).
+//     adjacent columns and fetches them with one 16-byte non-temporal load per
+//     packed row; a wave streams 1 KiB-contiguous row segments, eight rows in
+//     flight.
+//   * the activations of the block's K range are staged once in LDS in the
+//     k-order the extraction produces and read back as wave-uniform
+//     broadcasts; each dequantised fp16 pair feeds one v_dot2_f32_f16 per
+//     output row (17 VALU ops per packed word at M = 1).
+//   * K is split over the four waves of a block (LDS), over blockIdx.y (fp32
+//     partials summed in split order by a second tiny kernel: deterministic, no
+//     atomics, no fences) and within a lane (private fp32 accumulators).
 //   * zero points and scales are fetched once per (group, column) and folded
-//     into packed fp16 constants (see gptq_common.h).
+//     into packed fp16 constants (gptq_common.h).
+//
+// The MFMA kernel in gptq_gemm.hip needs 13 VALU ops per word and is what
+// mh_gptq_matmul dispatches to by default; this kernel stays callable as
+// mh_gptq_gemv and through MH_GEMV_MAX_M.
 #include "gptq_common.h"
 
 namespace mh {
@@ -28,7 +33,7 @@ template <int BITS, int M, int ROWS>
 __global__ __launch_bounds__(256) void gptq_gemv_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
-    half_t* __restrict__ out, float* partial, unsigned* counters,
+    half_t* __restrict__ out, float* __restrict__ partial,
     int N, int K, int rows_per_group, int steps_total, int steps_per_wave, int split_k) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
@@ -43,10 +48,26 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
     const int split = blockIdx.y;
     const int n = tile * kGemvCols + lane * 4;
     const bool active = n < N;
+    const int nc = active ? n : 0;
 
     const int rows_total = steps_total * ROWS;
     const int rows_blk = kGemvWaves * steps_per_wave * ROWS;
     const int row_base = split * rows_blk;
+    const int slot = split * kGemvWaves + wave;
+    const int step_begin = slot * steps_per_wave;
+    const int step_end = min(steps_total, step_begin + steps_per_wave);
+
+    // The first step's weight rows are requested before anything else, so that
+    // staging the activations overlaps their latency.
+    uint4_t q[ROWS];
+    auto load_rows = [&](int step) {
+        const uint32_t* wp = qweight + (size_t)step * ROWS * N + nc;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+            q[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wp + (size_t)i * N));
+    };
+    if (step_begin < step_end) load_rows(step_begin);
+
     for (int idx = threadIdx.x; idx < rows_blk * M; idx += 256) {
         const int m = idx / rows_blk, rl = idx % rows_blk;
         const int row = row_base + rl;
@@ -73,52 +94,40 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[m][c] = 0.f;
 
-    const int slot = split * kGemvWaves + wave;
-    const int step_begin = slot * steps_per_wave;
-    const int step_end = min(steps_total, step_begin + steps_per_wave);
-
-    if (active && step_begin < step_end) {
-        ColumnConst cc[4];
-        int g_cur = -1;
-        for (int step = step_begin; step < step_end; ++step) {
-            const int row = step * ROWS;
-            const uint32_t* wp = qweight + (size_t)row * N + n;
-            uint4_t q[ROWS];
+    ColumnConst cc[4];
+    int g_cur = -1;
+    for (int step = step_begin; step < step_end; ++step) {
+        const int row = step * ROWS;
+        if (step != step_begin) load_rows(step);
+        const int g = row / rows_per_group;
+        if (g != g_cur) {
+            g_cur = g;
+            const uint2 sraw = *reinterpret_cast<const uint2*>(scales + (size_t)g * N + nc);
+            const uint32_t zword = qzeros[(size_t)g * (N / P) + nc / P] >> ((nc % P) * BITS);
+            const half2_t s01 = as_half2(sraw.x), s23 = as_half2(sraw.y);
+            cc[0] = make_column_const(s01.x, zword & MASK);
+            cc[1] = make_column_const(s01.y, (zword >> BITS) & MASK);
+            cc[2] = make_column_const(s23.x, (zword >> (2 * BITS)) & MASK);
+            cc[3] = make_column_const(s23.y, (zword >> (3 * BITS)) & MASK);
+        }
+        const int rl0 = row - row_base;
 #pragma unroll
-            for (int i = 0; i < ROWS; ++i)
-                q[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wp + (size_t)i * N));
-
-            const int g = row / rows_per_group;
-            if (g != g_cur) {
-                g_cur = g;
-                const uint2 sraw = *reinterpret_cast<const uint2*>(scales + (size_t)g * N + n);
-                const uint32_t zword = qzeros[(size_t)g * (N / P) + n / P] >> ((n % P) * BITS);
-                const half2_t s01 = as_half2(sraw.x), s23 = as_half2(sraw.y);
-                cc[0] = make_column_const(s01.x, zword & MASK);
-                cc[1] = make_column_const(s01.y, (zword >> BITS) & MASK);
-                cc[2] = make_column_const(s23.x, (zword >> (2 * BITS)) & MASK);
-                cc[3] = make_column_const(s23.y, (zword >> (3 * BITS)) & MASK);
-            }
-
-            const int rl0 = row - row_base;
+        for (int i = 0; i < ROWS; ++i) {
+            uint32_t xp[M][PAIRS];
 #pragma unroll
-            for (int i = 0; i < ROWS; ++i) {
-                uint32_t xp[M][PAIRS];
+            for (int m = 0; m < M; ++m)
+#pragma unroll
+                for (int p = 0; p < PAIRS; ++p) xp[m][p] = xs[(m * rows_blk + rl0 + i) * PAIRS + p];
+            const uint32_t qs[4] = {q[i].x, q[i].y, q[i].z, q[i].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                half2_t w[PAIRS];
+                dequant_word<BITS>(qs[c], cc[c], regs, w);
 #pragma unroll
                 for (int m = 0; m < M; ++m)
 #pragma unroll
-                    for (int p = 0; p < PAIRS; ++p) xp[m][p] = xs[(m * rows_blk + rl0 + i) * PAIRS + p];
-                const uint32_t qs[4] = {q[i].x, q[i].y, q[i].z, q[i].w};
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    half2_t w[PAIRS];
-                    dequant_word<BITS>(qs[c], cc[c], regs, w);
-#pragma unroll
-                    for (int m = 0; m < M; ++m)
-#pragma unroll
-                        for (int p = 0; p < PAIRS; ++p)
-                            acc[m][c] = __builtin_amdgcn_fdot2(as_half2(xp[m][p]), w[p], acc[m][c], false);
-                }
+                    for (int p = 0; p < PAIRS; ++p)
+                        acc[m][c] = __builtin_amdgcn_fdot2(as_half2(xp[m][p]), w[p], acc[m][c], false);
             }
         }
     }
@@ -133,49 +142,44 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
 
     const int t = threadIdx.x;
     const int nt = tile * kGemvCols + t;
-    float total[M];
+    if (nt >= N) return;
 #pragma unroll
-    for (int m = 0; m < M; ++m) total[m] = (red[0][m][t] + red[1][m][t]) + (red[2][m][t] + red[3][m][t]);
+    for (int m = 0; m < M; ++m) {
+        const float total = (red[0][m][t] + red[1][m][t]) + (red[2][m][t] + red[3][m][t]);
+        if (split_k == 1)
+            out[(size_t)m * N + nt] = (half_t)total;
+        else
+            partial[((size_t)split * M + m) * N + nt] = total;  // summed by splitk_finalize_kernel
+    }
+}
 
-    if (split_k == 1) {
-        if (nt < N) {
+// Second stage of split-K: out[i] = fp16(sum over splits, in split order).
+// A separate launch instead of a "last block reduces" hand-off inside the main
+// kernel: the kernel boundary makes the partials visible without any
+// device-scope fence or atomic, the summation order is fixed, and the workspace
+// needs no initialisation.
+__global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __restrict__ partial,
+                                                              half_t* __restrict__ out, size_t mn, int split_k) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= mn) return;
+    float4_t s = {0.f, 0.f, 0.f, 0.f};
+    int sp = 0;
+    for (; sp + 8 <= split_k; sp += 8) {
+        float4_t v[8];
 #pragma unroll
-            for (int m = 0; m < M; ++m) out[(size_t)m * N + nt] = (half_t)total[m];
-        }
-        return;
+        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4_t*>(partial + (size_t)(sp + u) * mn + i);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
     }
+    for (; sp < split_k; ++sp) s += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
+    const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+    *reinterpret_cast<half4_t*>(out + i) = h;
+}
 
-    // K-reduction across blocks: publish the partial; the last block to arrive
-    // for this column tile sums all of them in split order (deterministic).
-    if (nt < N) {
-#pragma unroll
-        for (int m = 0; m < M; ++m) store_agent(&partial[((size_t)split * M + m) * N + nt], total[m]);
-    }
-    __shared__ int is_last;
-    if (!arrive_and_check_last(&counters[tile], (unsigned)split_k, &is_last)) return;
-    if (nt < N) {
-        float s[M];
-#pragma unroll
-        for (int m = 0; m < M; ++m) s[m] = 0.f;
-        const float* p = partial + nt;
-        int sp = 0;
-        for (; sp + 8 <= split_k; sp += 8) {
-            float v[8][M];
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-#pragma unroll
-                for (int m = 0; m < M; ++m) v[u][m] = load_agent(p + ((size_t)(sp + u) * M + m) * N);
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-#pragma unroll
-                for (int m = 0; m < M; ++m) s[m] += v[u][m];
-        }
-        for (; sp < split_k; ++sp)
-#pragma unroll
-            for (int m = 0; m < M; ++m) s[m] += load_agent(p + ((size_t)sp * M + m) * N);
-#pragma unroll
-        for (int m = 0; m < M; ++m) out[(size_t)m * N + nt] = (half_t)s[m];
-    }
+void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, size_t mn, int split_k) {
+    const size_t threads = (mn + 3) / 4;
+    hipLaunchKernelGGL(splitk_finalize_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                       partial, (half_t*)out, mn, split_k);
 }
 
 // ---- host side -----------------------------------------------------------------------
@@ -199,6 +203,8 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
     const int rows_per_group = group_size / P;
     GemvPlan p;
     p.rows = (rows_per_group % 8 == 0) ? 8 : (rows_per_group % 4 == 0) ? 4 : 1;
+    static const int rows_override = env_int("MH_GEMV_ROWS", 0);
+    if (rows_override == 4 && p.rows == 8) p.rows = 4;
     p.col_tiles = (N + kGemvCols - 1) / kGemvCols;
     p.steps_total = (K / P) / p.rows;
     // Enough waves to keep every SIMD busy with several loads in flight.
@@ -212,7 +218,6 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
     if (split > max_split) split = max_split;
     if (split < min_split) split = min_split;
     if (split < 1) split = 1;
-    if (p.col_tiles > kMaxCounters && min_split <= 1) split = 1;  // no counter for that many tiles
     p.steps_per_wave = (int)((p.steps_total + split * kGemvWaves - 1) / (split * kGemvWaves));
     p.split_k = (p.steps_total + p.steps_per_wave * kGemvWaves - 1) / (p.steps_per_wave * kGemvWaves);
     return p;
@@ -220,8 +225,7 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
 
 size_t gemv_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     const GemvPlan p = plan_gemv(N, K, group_size, bits);
-    size_t partial = (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
-    return kCounterRegionBytes + partial;
+    return (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
 }
 
 template <int BITS, int M, int ROWS>
@@ -229,13 +233,13 @@ static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, co
                         const int32_t* qzeros, const void* scales, void* out, void* workspace,
                         int N, int K, int group_size) {
     constexpr int P = Packing<BITS>::kPerWord;
-    unsigned* counters = reinterpret_cast<unsigned*>(workspace);
-    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterRegionBytes);
+    float* partial = reinterpret_cast<float*>(workspace);
     const size_t lds = (size_t)M * kGemvWaves * p.steps_per_wave * ROWS * Packing<BITS>::kPairs * sizeof(uint32_t);
     hipLaunchKernelGGL((gptq_gemv_kernel<BITS, M, ROWS>), dim3(p.col_tiles, p.split_k), dim3(256), lds, stream,
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
-                       (const half_t*)scales, (half_t*)out, partial, counters, N, K, group_size / P,
+                       (const half_t*)scales, (half_t*)out, partial, N, K, group_size / P,
                        p.steps_total, p.steps_per_wave, p.split_k);
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
 }
 
 template <int BITS, int M>
@@ -274,9 +278,6 @@ int gptq_gemv_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     const GemvPlan p = plan_gemv(N, K, group_size, bits);
     const size_t need = gemv_workspace_bytes(M, N, K, group_size, bits);
     if (p.split_k > 1) {
-        if (p.col_tiles > kMaxCounters)
-            return fail(MH_ERR_INVALID, "mh_gptq_gemv: N=%d with K=%d needs more than %d tile counters", N, K,
-                        kMaxCounters);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemv: workspace of %zu bytes required, got %zu", need,
                         workspace ? workspace_bytes : (size_t)0);
