@@ -7,28 +7,35 @@
 // operands are K-contiguous -- exactly what the MFMA operand layout wants
 // (16 consecutive k per lane).
 //
-// Tiling: block tile 128 x 256 x 64, four waves in a 2 x 2 arrangement, each
-// computing 64 x 128 as 2 x 4 MFMA tiles of 32 x 32.  Operand tiles are staged
-// through LDS with a 16-byte-chunk XOR swizzle (rows are 64 bytes, so unswizzled
-// ds_read_b128 of 8 consecutive rows would hit the same banks), double
-// buffered, with the next stage held in registers while the current one is
-// consumed: one barrier per 64-k step.  blockIdx -> tile mapping is XCD-aware:
+// Tiling: block tile 128 x 256 x 64, eight waves in a 2 x 4 arrangement (two
+// per SIMD, so one wave's MFMA issue gaps are filled by the other), each
+// computing 64 x 64 as 2 x 2 MFMA tiles of 32 x 32.  Operand tiles travel
+// global -> a register ring several k-steps deep -> LDS (double buffered, one
+// barrier per 64-k step) -> fragment registers (double buffered per half
+// k-step).  LDS rows are 64 bytes; the 16-byte chunk index is XOR-swizzled with
+// bits 2..3 of the row, which makes ds_read_b128 of 32 consecutive rows
+// conflict-free on the 64-bank LDS.  blockIdx -> tile mapping is XCD-aware:
 // consecutive block ids land on different XCDs, so each XCD is given a compact
 // rectangle of tiles and its L2 sees each operand row few times.
 #include "common.h"
 
 namespace mh {
 
-constexpr int kI8BM = 128, kI8BN = 256, kI8BK = 64;
+constexpr int kI8BM = 128, kI8BN = 256, kI8BK = 64, kI8Threads = 512;
+constexpr int kI8StagePitch = 144;  // bytes per staged output row: 64 fp16 + 16 bytes of padding
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * 64 + ((chunk ^ ((row >> 1) & 3)) << 4); }
+__device__ __forceinline__ int swz(int row, int chunk) { return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4); }
 
-__global__ __launch_bounds__(256) void i8_gemm_kernel(
+template <int R>  // k-steps a global load is issued ahead of its use; K / 64 is a multiple of R
+__global__ __launch_bounds__(kI8Threads) void i8_gemm_kernel(
     const int8_t* __restrict__ A, const int8_t* __restrict__ W, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, half_t* __restrict__ out, int32_t* __restrict__ acc_out,
     int M, int N, int K, int tiles_m, int tiles_n, int group_m, int xcd_chunk) {
-    __shared__ __attribute__((aligned(16))) int8_t As[2][kI8BM * kI8BK];
-    __shared__ __attribute__((aligned(16))) int8_t Bs[2][kI8BN * kI8BK];
+    // [2][A tile | W tile]; reused by the epilogue as eight 32-row output stages
+    __shared__ __attribute__((aligned(16))) int8_t smem[2 * (kI8BM + kI8BN) * kI8BK];
+    __shared__ float s_a[kI8BM], s_w[kI8BN];
+    auto As = [&](int buf) { return smem + buf * (kI8BM + kI8BN) * kI8BK; };
+    auto Bs = [&](int buf) { return smem + buf * (kI8BM + kI8BN) * kI8BK + kI8BM * kI8BK; };
 
     // XCD-aware tile order: block b runs on XCD b % 8; give every XCD a run of
     // xcd_chunk consecutive positions of a grouped (group_m rows at a time) order.
@@ -44,93 +51,195 @@ __global__ __launch_bounds__(256) void i8_gemm_kernel(
     const int m0 = tm * kI8BM, n0 = tn * kI8BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wy = wave >> 1, wx = wave & 1;
+    const int wy = wave >> 2, wx = wave & 3;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    int16_t_v acc[2][4];
+    if (out) {  // visible to the epilogue through the barriers of the main loop
+        if (tid < kI8BN) s_w[tid] = w_scale[min(n0 + tid, N - 1)];
+        if (tid < kI8BM) s_a[tid] = a_scale[min(m0 + tid, M - 1)];
+    }
+
+    // acc[i][j] is the 32 x 32 tile (rows m of A block i, columns n of W block j),
+    // computed transposed -- the W fragment is the MFMA's first operand -- so a
+    // lane ends up with runs of four consecutive n for one m (see the epilogue).
+    int16_t_v acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    // staging: A has 512 chunks (2 per thread), B has 1024 (4 per thread)
-    int4_t ra[2], rb[4];
-    const int crow = tid >> 2, cchunk = tid & 3;  // +64 rows per extra chunk
-    auto load_stage = [&](int k0) {
+    // Global -> register ring -> LDS.  A k-step of MFMAs (~0.2 us) is far shorter
+    // than a trip to L2/HBM: the operands of k-step kt + R are requested while kt
+    // is computed and only stored to LDS R steps later.  Per stage A has 512
+    // 16-byte chunks (one per thread) and W has 1024 (two per thread).
+    int4_t ra[R], rb[R][2];
+    const int crow = tid >> 2, cchunk = tid & 3;
+    const int8_t* a_src = A + (size_t)min(m0 + crow, M - 1) * K + cchunk * 16;
+    const int8_t* b_src[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int m = min(m0 + crow + 64 * j, M - 1);
-            ra[j] = *reinterpret_cast<const int4_t*>(A + (size_t)m * K + k0 + cchunk * 16);
-        }
+    for (int j = 0; j < 2; ++j) b_src[j] = W + (size_t)min(n0 + crow + 128 * j, N - 1) * K + cchunk * 16;
+    const int KT = K / kI8BK;
+    auto load_stage = [&](int slot, int kt) {
+        const int k0 = min(kt, KT - 1) * kI8BK;
+        ra[slot] = *reinterpret_cast<const int4_t*>(a_src + k0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = min(n0 + crow + 64 * j, N - 1);
-            rb[j] = *reinterpret_cast<const int4_t*>(W + (size_t)n * K + k0 + cchunk * 16);
+        for (int j = 0; j < 2; ++j) rb[slot][j] = *reinterpret_cast<const int4_t*>(b_src[j] + k0);
+    };
+    // A stage is written to LDS in two parts, one under each half k-step, so that
+    // neither half is heavy on LDS writes (which run at a third of the read rate).
+    auto store_part = [&](int part, int slot, int buf) {
+        if (part == 0) {
+            *reinterpret_cast<int4_t*>(As(buf) + swz(crow, cchunk)) = ra[slot];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                *reinterpret_cast<int4_t*>(Bs(buf) + swz(crow + 128 * j, cchunk)) = rb[slot][j];
         }
     };
-    auto store_stage = [&](int buf) {
+    // Fragment registers, two sets: the MFMAs of one half k-step (32 k) run
+    // while the ds_reads of the next half fill the other set.
+    int4_t fa[2][2], fb[2][2];
+    auto read_frag = [&](int set, int buf, int ks) {
+        const int chunk = ks * 2 + lh;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            fa[set][i] = *reinterpret_cast<const int4_t*>(As(buf) + swz(wy * 64 + i * 32 + l32, chunk));
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-            *reinterpret_cast<int4_t*>(&As[buf][swz(crow + 64 * j, cchunk)]) = ra[j];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<int4_t*>(&Bs[buf][swz(crow + 64 * j, cchunk)]) = rb[j];
+            fb[set][j] = *reinterpret_cast<const int4_t*>(Bs(buf) + swz(wx * 64 + j * 32 + l32, chunk));
+    };
+    auto mfma_one = [&](int set, int t) {
+        const int i = t >> 1, j = t & 1;
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
     };
 
-    const int KT = K / kI8BK;
-    load_stage(0);
-    store_stage(0);
+    // Stage s lives in ring slot s % R and LDS buffer s & 1.
+#pragma unroll
+    for (int r = 0; r < R; ++r) load_stage(r, r);
+    store_part(0, 0, 0);
+    store_part(1, 0, 0);
+    load_stage(0, R);
     __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < KT) load_stage((kt + 1) * kI8BK);
+    read_frag(0, 0, 0);
+    store_part(0, 1 % R, 1);
+    for (int kt0 = 0; kt0 < KT; kt0 += R) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const int chunk = ks * 2 + lh;
-            int4_t a[2], b[4];
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i] = *reinterpret_cast<const int4_t*>(&As[buf][swz(wy * 64 + i * 32 + l32, chunk)]);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                b[j] = *reinterpret_cast<const int4_t*>(&Bs[buf][swz(wx * 128 + j * 32 + l32, chunk)]);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int r = 0; r < R; ++r) {
+            const int kt = kt0 + r;
+            const int buf = kt & 1;
+            // first half: the rest of stage kt + 1 goes to the other buffer and the
+            // second-half fragments are fetched under the first-half MFMAs; the
+            // ring slot of stage kt + 1 is then requested again for kt + 1 + R.
+            // The first MFMA of each half is issued ahead of the half's LDS traffic
+            // so the matrix pipe is never waiting behind a full LDS queue.
+            mfma_one(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            store_part(1, (r + 1) % R, buf ^ 1);
+            read_frag(1, buf, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_one(0, 1);
+            mfma_one(0, 2);
+            mfma_one(0, 3);
+            load_stage((r + 1) % R, kt + 1 + R);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            // second half: first-half fragments of stage kt + 1 and the first part
+            // of stage kt + 2 (into this stage's buffer, which every wave has
+            // finished reading at the barrier) under the second-half MFMAs.
+            mfma_one(1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frag(0, buf ^ 1, 0);
+            store_part(0, (r + 2) % R, buf);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_one(1, 1);
+            mfma_one(1, 2);
+            mfma_one(1, 3);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (kt + 1 < KT) store_stage(buf ^ 1);
-        __syncthreads();
     }
+    __syncthreads();  // every wave is done with the operand buffers
 
-    // epilogue: acc[i][j][r] is row (r/4)*8 + lh*4 + r%4, column l32 of its 32x32 tile
+    // Epilogue.  acc[i][j][q * 4 + e] belongs to row m = l32 and column
+    // n = q * 8 + lh * 4 + e of its tile: four consecutive n per (lane, q).
+    const int wm = wy * 64, wn = wx * 64;  // wave tile origin inside the block tile
+    if (acc_out) {
+        const bool n_vec = (N % 4 == 0);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 2; ++i) {
+            const int m = m0 + wm + i * 32 + l32;
+            if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + wx * 128 + j * 32 + l32;
-            if (n >= N) continue;
-            const float ws = w_scale ? w_scale[n] : 1.f;
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wy * 64 + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (m >= M) continue;
-                const int v = acc[i][j][r];
-                if (acc_out) acc_out[(size_t)m * N + n] = v;
-                if (out) {
-                    const float s = (a_scale ? a_scale[m] : 1.f) * ws;
-                    // The product is rounded to fp32 and only then to fp16; the
-                    // empty asm keeps the compiler from fusing both into one
-                    // mixed-precision instruction that rounds once.
-                    float prod = (float)v * s;
-                    asm volatile("" : "+v"(prod));
-                    out[(size_t)m * N + n] = (half_t)prod;
+                for (int q = 0; q < 4; ++q) {
+                    const int n = n0 + wn + j * 32 + q * 8 + lh * 4;
+                    if (n >= N) continue;
+                    int32_t* dst = acc_out + (size_t)m * N + n;
+                    if (n_vec && n + 4 <= N) {
+                        int4_t v = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                        *reinterpret_cast<int4_t*>(dst) = v;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (n + e < N) dst[e] = acc[i][j][q * 4 + e];
+                    }
+                }
+        }
+    }
+    if (out) {
+        // Scaled fp16 values are staged per wave as 32 rows x 64 columns in LDS
+        // and leave as whole 128-byte row pieces, 16 bytes per lane.
+        int8_t* stage = smem + wave * (32 * kI8StagePitch);
+        const bool n_vec = (N % 8 == 0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float sa = s_a[wm + i * 32 + l32];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = j * 32 + q * 8 + lh * 4;
+                    const float4_t sw = *reinterpret_cast<const float4_t*>(s_w + wn + nl);
+                    half4_t h;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        // The scale product and its product with the sum are each
+                        // rounded to fp32 and only then to fp16; the empty asm keeps
+                        // the compiler from fusing the last two steps into one
+                        // mixed-precision instruction that rounds once.
+                        float prod = (float)acc[i][j][q * 4 + e] * (sa * sw[e]);
+                        asm volatile("" : "+v"(prod));
+                        h[e] = (half_t)prod;
+                    }
+                    *reinterpret_cast<half4_t*>(stage + l32 * kI8StagePitch + nl * 2) = h;
+                }
+            // wave-private region: only this wave's own LDS traffic has to land
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int row = rr * 8 + (lane >> 3), c8 = (lane & 7) * 8;
+                const int m = m0 + wm + i * 32 + row, n = n0 + wn + c8;
+                const int4_t v = *reinterpret_cast<const int4_t*>(stage + row * kI8StagePitch + c8 * 2);
+                if (m >= M || n >= N) continue;
+                half_t* dst = out + (size_t)m * N + n;
+                if (n_vec) {
+                    *reinterpret_cast<int4_t*>(dst) = v;
+                } else {
+                    const half_t* hv = reinterpret_cast<const half_t*>(&v);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (n + e < N) dst[e] = hv[e];
                 }
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
+    }
 }
 
 // out[c, r] = in[r, c] through a 64 x 64 LDS tile.
@@ -164,13 +273,24 @@ int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w, const float
     MH_REQUIRE(a && w, "mh_i8_gemm: null operand");
     MH_REQUIRE(out_f16 || acc_i32, "mh_i8_gemm: no output requested");
     MH_REQUIRE(!out_f16 || (a_scale && w_scale), "mh_i8_gemm: scales required for the fp16 output");
-    MH_REQUIRE(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "mh_i8_gemm: operands must be 16-byte aligned");
+    MH_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)acc_i32) % 16 == 0 && (uintptr_t)out_f16 % 16 == 0,
+               "mh_i8_gemm: operands and outputs must be 16-byte aligned");
     const int tiles_m = (M + kI8BM - 1) / kI8BM, tiles_n = (N + kI8BN - 1) / kI8BN;
     const int tiles = tiles_m * tiles_n;
     const int group_m = tiles_m < 8 ? tiles_m : 8;
     const int xcd_chunk = (tiles % 8 == 0) ? tiles / 8 : 0;
-    hipLaunchKernelGGL(i8_gemm_kernel, dim3(tiles), dim3(256), 0, as_stream(stream), a, w, a_scale, w_scale,
-                       (half_t*)out_f16, acc_i32, M, N, K, tiles_m, tiles_n, group_m, xcd_chunk);
+    const int kt = K / kI8BK;
+#define MH_I8_LAUNCH(R)                                                                                      \
+    hipLaunchKernelGGL(i8_gemm_kernel<R>, dim3(tiles), dim3(kI8Threads), 0, as_stream(stream), a, w, a_scale, w_scale, \
+                       (half_t*)out_f16, acc_i32, M, N, K, tiles_m, tiles_n, group_m, xcd_chunk)
+    if (kt % 4 == 0) {
+        MH_I8_LAUNCH(4);
+    } else if (kt % 2 == 0) {
+        MH_I8_LAUNCH(2);
+    } else {
+        MH_I8_LAUNCH(1);
+    }
+#undef MH_I8_LAUNCH
     MH_CHECK_LAUNCH();
     return MH_OK;
 }

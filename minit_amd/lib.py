@@ -11,7 +11,7 @@ import os
 from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_uint32, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libminit_hip.so")
+LIB_PATH = os.environ.get("MINIT_HIP_LIB") or os.path.join(_HERE, "libminit_hip.so")
 
 
 class HipError(RuntimeError):
