@@ -96,9 +96,11 @@ int mh_gptq_dequant(mh_stream_t stream, const int32_t* qweight, const int32_t* q
  * K % group_size == 0.
  *
  * workspace: device scratch of at least mh_gptq_workspace_bytes(M, N, K, ...)
- * bytes (fp32 split-K partial sums), 256-byte aligned, no initialisation
- * needed; may be NULL when the size query returns 0.  It may be shared by calls
- * that are ordered on one stream, never by concurrent calls.
+ * bytes (arrival counters followed by fp32 split-K partial sums), 256-byte
+ * aligned, zero-filled once by the caller after allocation: every call leaves
+ * the counters at zero again, so the buffer is never cleared between calls.
+ * May be NULL when the size query returns 0.  It may be shared by calls that
+ * are ordered on one stream, never by concurrent calls.
  *
  * mh_gptq_gemv   wave64 VALU path, no MFMA; M <= MH_GPTQ_GEMV_MAX_M.
  * mh_gptq_gemm   fp16 MFMA path; any M >= 1.

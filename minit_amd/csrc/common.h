@@ -101,6 +101,24 @@ __device__ __forceinline__ void store_agent(float* p, float v) {
 __device__ __forceinline__ float load_agent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// 16-byte forms of the two above (the compiler has no vector atomics; sc1 is the
+// agent-scope cache policy it gives the scalar ones).  The load is asynchronous:
+// wait_agent_loads() must come between it and the first use of its result.
+__device__ __forceinline__ void store_agent4(float* p, float4_t v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ float4_t load_agent4(const float* p) {
+    float4_t v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int COUNT>
+__device__ __forceinline__ void wait_agent_loads(float4_t (&v)[COUNT]) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < COUNT; ++i) asm volatile("" : "+v"(v[i]));  // uses of v[i] stay below the wait
+}
+
 // True, in every thread, for the workgroup that arrives last of `expected`; that
 // workgroup also resets the counter for the next launch.  All threads of the
 // workgroup must call it.

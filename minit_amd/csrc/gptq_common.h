@@ -118,6 +118,12 @@ __device__ __forceinline__ void pair_activations<8>(const uint32_t* x, uint32_t*
     xp[1] = (x[0] >> 16) | (x[1] & 0xFFFF0000u);
 }
 
+// The workspace of the split-K kernels starts with one arrival counter per
+// 256-column tile.  The caller zero-fills the workspace once; every launch
+// leaves the counters at zero again.
+constexpr int kMaxTileCounters = 16384;
+constexpr size_t kTileCounterBytes = kMaxTileCounters * sizeof(unsigned);
+
 // Host-side argument validation shared by the GPTQ entry points.
 int check_gptq_args(const char* who, const void* x, const void* qweight, const void* qzeros,
                     const void* scales, const void* out, int M, int N, int K, int group_size,

@@ -240,7 +240,7 @@ template <int BITS, int MT, int SPG>
 __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
-    half_t* __restrict__ out, float* __restrict__ partial,
+    half_t* __restrict__ out, float* partial, unsigned* counters,
     int M, int N, int K, int steps_total, int stages_per_block, int split_k) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
@@ -395,26 +395,58 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         __syncthreads();
     }
 
-    if (!active) return;
+    // ---- results.  With K split over several workgroups every one publishes
+    // its fp32 partial tile with agent-scope stores (they go through to memory,
+    // which is what workgroups on other XCDs see) and counts itself in; the one
+    // that arrives last adds the partials in split order -- a fixed order, so the
+    // result does not depend on which workgroup that is -- and puts the counter
+    // back to zero for the next launch.
+    if (active) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = mt * 16 + kq * 4 + r;
-            if (m < M) {
+            for (int r = 0; r < 4; ++r) {
+                const int m = mt * 16 + kq * 4 + r;
+                if (m >= M) continue;
                 if (split_k == 1) {
                     const half4_t h = {(half_t)acc[mt][0][r], (half_t)acc[mt][1][r], (half_t)acc[mt][2][r],
                                        (half_t)acc[mt][3][r]};
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
                 } else {
-                    *reinterpret_cast<float4_t*>(partial + ((size_t)split * M + m) * N + col) =
-                        float4_t{acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
+                    const float4_t v = {acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
+                    float* dst = partial + ((size_t)split * M + m) * N + col;
+                    if (counters)
+                        store_agent4(dst, v);
+                    else
+                        *reinterpret_cast<float4_t*>(dst) = v;
                 }
             }
-        }
-}
+    }
+    if (split_k == 1 || counters == nullptr) return;  // without counters a second kernel adds the partials
 
-// ---- host side ---------------------------------------------------------------------------------------
+    __shared__ int is_last;
+    if (!arrive_and_check_last(&counters[tile], (unsigned)split_k, &is_last)) return;
+    constexpr int BATCH = 8;  // partial loads in flight per thread
+    const size_t plane = (size_t)M * N;
+    for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
+        const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
+        if (c >= N) continue;
+        const float* p = partial + (size_t)m * N + c;
+        float4_t s = {0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < split_k; sp += BATCH) {
+            float4_t v[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+                v[u] = sp + u < split_k ? load_agent4(p + (size_t)(sp + u) * plane) : float4_t{0.f, 0.f, 0.f, 0.f};
+            wait_agent_loads(v);
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u)
+                if (sp + u < split_k) s += v[u];
+        }
+        const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+        *reinterpret_cast<half4_t*>(out + (size_t)m * N + c) = h;
+    }
+}
 
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
@@ -432,6 +464,7 @@ static int env_int_gemm(const char* name, int fallback) {
 }
 
 constexpr int kSmallMaxM = 32;
+constexpr int kFusedReduceMaxM = 8;
 
 // Plan of the small-M kernel: column tiles x K splits sized so the GPU holds
 // about MH_GEMM_SMALL_WAVES_PER_CU waves per CU; a block walks whole stages.
@@ -498,14 +531,16 @@ bool gemm_supported(int M, int N, int K, int group_size, int bits) {
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)bits;
     const GemmPlan p = plan_gemm(M, N, K, group_size);
-    return (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
+    if (p.split_k <= 1) return 0;
+    return kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float);
 }
 
 template <int BITS, int MT>
 static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                         const int32_t* qzeros, const void* scales, void* out, void* workspace, int M, int N,
                         int K, int group_size) {
-    float* partial = reinterpret_cast<float*>(workspace);
+    // the arrival counters at the head of the workspace belong to the small-M kernel
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     hipLaunchKernelGGL((gptq_gemm_kernel<BITS, MT>), dim3(p.col_tiles, p.split_k, p.m_blocks), dim3(256), 0,
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size / 32,
@@ -517,12 +552,16 @@ template <int BITS, int MT>
 static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                               const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
                               int N, int K, int group_size) {
-    float* partial = reinterpret_cast<float*>(workspace);
+    // workspace: [tile counters, zero between launches][fp32 partials]
+    // in-kernel reduction by the last workgroup of a tile pays for few rows only
+    unsigned* counters =
+        (M <= kFusedReduceMaxM && p.col_tiles <= kMaxTileCounters) ? reinterpret_cast<unsigned*>(workspace) : nullptr;
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     const dim3 grid(p.col_tiles, p.split_k);
 #define MH_LAUNCH_SMALL(SPG)                                                                                  \
     hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG>), grid, dim3(256), 0, stream, (const half_t*)x,  \
                        (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,  \
-                       partial, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k)
+                       partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k)
     switch (group_size / 32) {
         case 1: MH_LAUNCH_SMALL(1); break;
         case 2: MH_LAUNCH_SMALL(2); break;
@@ -530,7 +569,7 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
         default: MH_LAUNCH_SMALL(8); break;
     }
 #undef MH_LAUNCH_SMALL
-    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
+    if (p.split_k > 1 && counters == nullptr) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
 }
 
 template <int BITS>

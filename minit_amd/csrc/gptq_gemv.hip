@@ -153,11 +153,9 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
     }
 }
 
-// Second stage of split-K: out[i] = fp16(sum over splits, in split order).
-// A separate launch instead of a "last block reduces" hand-off inside the main
-// kernel: the kernel boundary makes the partials visible without any
-// device-scope fence or atomic, the summation order is fixed, and the workspace
-// needs no initialisation.
+// Second stage of split-K for the kernels that do not reduce in place:
+// out[i] = fp16(sum over splits, in split order).  The kernel boundary makes
+// the partials visible without any device-scope fence or atomic.
 __global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __restrict__ partial,
                                                               half_t* __restrict__ out, size_t mn, int split_k) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
@@ -225,7 +223,7 @@ GemvPlan plan_gemv(int N, int K, int group_size, int bits) {
 
 size_t gemv_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     const GemvPlan p = plan_gemv(N, K, group_size, bits);
-    return (p.split_k > 1) ? (size_t)p.split_k * M * N * sizeof(float) : 0;
+    return (p.split_k > 1) ? kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float) : 0;
 }
 
 template <int BITS, int M, int ROWS>
@@ -233,7 +231,8 @@ static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, co
                         const int32_t* qzeros, const void* scales, void* out, void* workspace,
                         int N, int K, int group_size) {
     constexpr int P = Packing<BITS>::kPerWord;
-    float* partial = reinterpret_cast<float*>(workspace);
+    // the head of the workspace holds the arrival counters of the MFMA kernel and stays zero
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     const size_t lds = (size_t)M * kGemvWaves * p.steps_per_wave * ROWS * Packing<BITS>::kPairs * sizeof(uint32_t);
     hipLaunchKernelGGL((gptq_gemv_kernel<BITS, M, ROWS>), dim3(p.col_tiles, p.split_k), dim3(256), lds, stream,
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
