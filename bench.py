@@ -124,6 +124,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel (1 GiB read + 1 GiB write per launch) that the "
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
+    ap.add_argument("--int8-only", action="store_true",
+                    help="run only the W8A8 GEMM lines (M=2048, K=4096, N in {4096, 11008}), then exit")
     args = ap.parse_args()
     ENTRY = args.entry
     if args.gpus != 1:
@@ -157,6 +159,10 @@ def main():
         us = e0.elapsed_ms(e1) * 1e3 / 5
         print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
                           "us": round(us, 1), "gbps_read_plus_write": round(2 * nbytes / us / 1e3, 1)}))
+        return
+
+    if args.int8_only:
+        print(json.dumps({"int8_gemm": [bench_int8(lib, HIPTensor, memory, n, iters=50) for n in (4096, 11008)]}))
         return
 
     # ---- inputs, resident in HBM before the timed region ------------------------------------

@@ -207,3 +207,15 @@ def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=pr
                         "hbm_gbps": round(gb / (ms / tokens * 1e-3), 1)})
         log(f"decode batch {b}: {ms / tokens:.3f} ms/token, {tps:.1f} tok/s")
     return results
+
+
+if __name__ == "__main__":
+    import argparse
+    import json
+
+    ap = argparse.ArgumentParser(description="Llama-3-70B-shape GPTQ decode on one GPU: tokens per second")
+    ap.add_argument("--batches", default="1,8,32")
+    ap.add_argument("--tokens", type=int, default=64)
+    cli = ap.parse_args()
+    print(json.dumps(bench_tokens_per_second(batches=tuple(int(b) for b in cli.batches.split(",")),
+                                             tokens=cli.tokens, log=lambda *a: print(*a, flush=True))))
