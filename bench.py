@@ -30,6 +30,13 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the dominant kernel on this workload, measured with two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, in KiB per
+# dispatch, scaled by what the same counters read for the 1 GiB copy kernel of
+# --calibrate-copy: x2.000 and x1.000); the summary with the commands is kept
+# under profiles/.  A counter cannot be read from inside this process, so the
+# figure is carried here and is only reported for the entry point it was taken on.
+MEASURED_TRAFFIC = {"mh_gptq_matmul": 115_688_243}
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0
 
@@ -236,7 +243,7 @@ def main():
             "frac": round(gbps / HBM_PEAK_GBPS, 4),
             "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
             "bytes_per_launch": step_bytes // len(LINEARS),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get(ENTRY),
         },
     }
 
