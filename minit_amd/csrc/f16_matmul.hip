@@ -13,8 +13,14 @@
 
 namespace mh {
 
-constexpr int kDenseDepth = 4;
+constexpr int kDenseDepth = 8;
 
+// Both operands travel through a ring of kDenseDepth steps of registers that is
+// refilled one slot per step at a fixed place of a branch-free loop body, so the
+// compiler can wait with an exact vmcnt and the stream of b never drains.  (With
+// the a fragment fetched at its point of use, every step waited for the load it
+// had just issued.)  Steps past the end of K re-read the last step and multiply
+// it by a zeroed a fragment.
 template <int MT>
 __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __restrict__ a,
                                                             const half_t* __restrict__ b,
@@ -35,26 +41,31 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
     for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int steps = K / 32;
+    const int last = steps - 1;
     constexpr int D = kDenseDepth;
-    uint4_t bq[D];
+    uint4_t bq[D], aq[D][MT];
+    auto load = [&](int slot, int s) {
+        const size_t off = (size_t)min(s, last) * 32;
+        bq[slot] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow + off));
 #pragma unroll
-    for (int d = 0; d < D; ++d)
-        bq[d] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow + (size_t)min(d, steps - 1) * 32));
+        for (int mt = 0; mt < MT; ++mt) aq[slot][mt] = *reinterpret_cast<const uint4_t*>(arow[mt] + off);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load(d, d);
     for (int s0 = 0; s0 < steps; s0 += D) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            const int s = s0 + d;
-            if (s < steps) {
-                const half8_t bf = __builtin_bit_cast(half8_t, bq[d]);
-                bq[d] = __builtin_nontemporal_load(
-                    reinterpret_cast<const uint4_t*>(brow + (size_t)min(s + D, steps - 1) * 32));
+            const bool live = s0 + d <= last;
+            const half8_t bf = __builtin_bit_cast(half8_t, bq[d]);
+            half8_t af[MT];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    const half8_t af = *reinterpret_cast<const half8_t*>(arow[mt] + (size_t)s * 32);
-                    // rows of the result are m (operand A), columns are n (operand B)
-                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf, acc[mt], 0, 0, 0);
-                }
-            }
+            for (int mt = 0; mt < MT; ++mt)
+                af[mt] = __builtin_bit_cast(half8_t, live ? aq[d][mt] : uint4_t{0u, 0u, 0u, 0u});
+            load(d, s0 + d + D);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)  // rows of the result are m (operand A), columns are n (operand B)
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt], bf, acc[mt], 0, 0, 0);
         }
     }
     // acc[mt][r] is row m0 + mt*16 + kq*4 + r, column n0 + i16
