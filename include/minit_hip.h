@@ -197,7 +197,9 @@ int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
  * pointers are device pointers owned by the caller.
  *   qkv      fused q|k|v projection, GPTQ, [hidden] -> [(QH + 2 KVH) * D]
  *   gate_up  fused gate|up projection, [hidden] -> [2 * ffn]
- *   k_cache / v_cache  fp16 [batch_max, KVH, max_seq, D], appended in place
+ *   k_cache  fp16 [batch_max, KVH, max_seq, D], v_cache fp16 [batch_max, KVH, D, max_seq]
+ *            (V is kept transposed for the P.V matrix product); both appended in place;
+ *            max_seq is a multiple of 8
  *   embed, lm_head     fp16 [vocab, hidden]; norms fp16 [hidden]
  *   freqs_cos / sin    fp32 [max_seq, D / 2]
  */

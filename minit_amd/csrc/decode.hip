@@ -93,7 +93,7 @@ __global__ void add_kernel(half_t* __restrict__ h, const half_t* __restrict__ de
 }
 
 // qkv [B, (QH + 2 KVH) * D]: rotate q heads into q_out [B, QH, D]; rotate k
-// heads and copy v heads into the caches at positions[b].  One 64-thread block
+// heads and copy v heads into the caches at positions[b] (V transposed).  One 64-thread block
 // per (head, batch row); thread i owns the interleaved pair i
 // (minit/cuda/kernel/cuda/rope.py:58-73).
 __global__ __launch_bounds__(64) void rope_kv_append_kernel(
@@ -107,9 +107,10 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(
     for (int i = threadIdx.x; i < half_dim; i += blockDim.x) {
         const float re = (float)src[2 * i], im = (float)src[2 * i + 1];
         if (head >= qh + kvh) {  // v: plain copy
-            half_t* dst = v_cache + (((size_t)b * kvh + (head - qh - kvh)) * max_seq + pos) * head_dim;
-            dst[2 * i] = src[2 * i];
-            dst[2 * i + 1] = src[2 * i + 1];
+            // the V cache is dim-major, [B, KVH, D, T]: see attn_decode_kernel
+            half_t* dst = v_cache + ((size_t)b * kvh + (head - qh - kvh)) * head_dim * max_seq + pos;
+            dst[(size_t)(2 * i) * max_seq] = src[2 * i];
+            dst[(size_t)(2 * i + 1) * max_seq] = src[2 * i + 1];
             continue;
         }
         const float c = freqs_cos[(size_t)pos * half_dim + i], s = freqs_sin[(size_t)pos * half_dim + i];
@@ -189,207 +190,230 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
 }
 
 // ---- split-KV decode attention ---------------------------------------------------------------------
-// One block per (split, kv head, batch row); G query heads share the KV head.
-// Phase A (lane = one cached position): scores of a 64-position chunk for all G
-// heads, running max / sum per head.  Phase B (lane = 8 output dims x one of 4
-// position sub-streams): acc[h] += p[h, t] * V[t].  Waves own alternate chunks
-// and are merged through LDS; splits are merged by the last block to arrive.
-
-template <int G, int D>
-struct AttnPartial {  // per (b, q head, split): m, l, acc[D]
-    static constexpr int kFloats = D + 2;
-};
+// One block per (split, kv head, batch row); the G query heads that share the KV
+// head are the (padded to 16) rows of fp16 MFMA tiles.  Per 64-position chunk a
+// wave computes S = Q K^T with 16 v_mfma_f32_16x16x32_f16 (K rows are
+// d-contiguous, which is the B-operand layout as loaded), does the running
+// max / sum softmax on the accumulator layout, passes P through LDS to turn it
+// into an A operand, and accumulates O += P V with 16 more MFMAs.  For that
+// product the B operand needs eight consecutive positions of one dim per lane,
+// so V is cached transposed, [B, KVH, D, T] (positions contiguous).  Waves own
+// alternate chunks and are merged through LDS; splits are merged by the last
+// block to arrive.
 
 template <int G, int D>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
-    const half_t* __restrict__ q, const half_t* __restrict__ k_cache, const half_t* __restrict__ v_cache,
+    const half_t* __restrict__ q, const half_t* __restrict__ k_cache, const half_t* __restrict__ vt_cache,
     const int32_t* __restrict__ positions, half_t* __restrict__ out, float* partial, unsigned* counters,
     int kvh, int max_seq, float scale, int splits) {
-    static_assert(D == 128, "head size 128");
-    constexpr int CH = D / 8;  // 16-byte chunks per row
+    static_assert(D == 128 && G <= 16, "head size 128, at most 16 query heads per KV head");
+    constexpr int PP = 72;  // halfs per row of the P tile in LDS (64 + padding)
     const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i16 = lane & 15, kq = lane >> 4;
     const int len = positions[b] + 1;  // the new token has been appended
-    const int span = (len + splits - 1) / splits;
+    // chunk starts stay multiples of 64 so that the transposed V reads are 16-byte aligned
+    const int span = ((len + splits - 1) / splits + 63) / 64 * 64;
     const int t0 = split * span, t1 = min(len, t0 + span);
 
-    __shared__ uint4 q_s[G * CH];
-    __shared__ float p_s[4][G][64];
-    __shared__ float m_s[4][G], l_s[4][G];
+    __shared__ __attribute__((aligned(16))) half_t p_s[4][16 * PP];
+    __shared__ float m_s[4][16], l_s[4][16];
     __shared__ float acc_s[4][G][D];
 
-    const half_t* qp = q + ((size_t)b * kvh + g) * G * D;
-    for (int i = tid; i < G * CH; i += 256) q_s[i] = reinterpret_cast<const uint4*>(qp)[i];
-    __syncthreads();
-
-    const half_t* kbase = k_cache + ((size_t)b * kvh + g) * max_seq * D;
-    const half_t* vbase = v_cache + ((size_t)b * kvh + g) * max_seq * D;
-
-    float m_run[G], l_run[G];
-    float acc[G][8];
+    // A operand of S = Q K^T: row = head i16, k = dims s*32 + kq*8 .. +8
+    uint4 qf[4];
+    {
+        const half_t* qp = q + (((size_t)b * kvh + g) * G + min(i16, G - 1)) * D + kq * 8;
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-        m_run[h] = -INFINITY;
-        l_run[h] = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
+        for (int s = 0; s < 4; ++s) {
+            qf[s] = *reinterpret_cast<const uint4*>(qp + s * 32);
+            if (i16 >= G) qf[s] = make_uint4(0, 0, 0, 0);
+        }
     }
-    const int dl = lane & 15, tg = lane >> 4;
+    const half_t* kbase = k_cache + ((size_t)b * kvh + g) * max_seq * D;
+    const half_t* vbase = vt_cache + ((size_t)b * kvh + g) * D * max_seq;
+
+    // rows of every accumulator tile held by this lane: heads kq*4 + r
+    float m_run[4], l_run[4];
+    float4_t acc[8];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        m_run[r] = -INFINITY;
+        l_run[r] = 0.f;
+    }
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int c0 = t0 + wave * 64; c0 < t1; c0 += 256) {
-        // ---- phase A
-        const int t = c0 + lane;
-        const bool valid = t < t1;
-        float s[G];
+        // all loads of the chunk are issued before the first use
+        uint4 kf[4][4], vf[8][2];
 #pragma unroll
-        for (int h = 0; h < G; ++h) s[h] = 0.f;
-        const uint4* krow = reinterpret_cast<const uint4*>(kbase + (size_t)(valid ? t : t0) * D);
-        uint4 kq[CH], vq[16];
+        for (int pt = 0; pt < 4; ++pt) {
+            const int row = min(c0 + pt * 16 + i16, t1 - 1);
+            const half_t* kp = kbase + (size_t)row * D + kq * 8;
 #pragma unroll
-        for (int c = 0; c < CH; ++c) kq[c] = krow[c];
-        // the V rows of phase B are requested now so both streams are in flight together
-#pragma unroll
-        for (int tt = 0; tt < 16; ++tt) {
-            const int tv = min(c0 + tt * 4 + tg, t1 - 1);
-            vq[tt] = reinterpret_cast<const uint4*>(vbase + (size_t)tv * D)[dl];
+            for (int s = 0; s < 4; ++s) kf[pt][s] = *reinterpret_cast<const uint4*>(kp + s * 32);
         }
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const uint4 kv = kq[c];
-            const half2_t k0 = __builtin_bit_cast(half2_t, kv.x), k1 = __builtin_bit_cast(half2_t, kv.y),
-                          k2 = __builtin_bit_cast(half2_t, kv.z), k3 = __builtin_bit_cast(half2_t, kv.w);
+        for (int ks = 0; ks < 2; ++ks) {
+            const int p0 = min(c0 + ks * 32 + kq * 8, max_seq - 8);
 #pragma unroll
-            for (int h = 0; h < G; ++h) {
-                const uint4 qv = q_s[h * CH + c];
-                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.x), k0, s[h], false);
-                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.y), k1, s[h], false);
-                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.z), k2, s[h], false);
-                s[h] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qv.w), k3, s[h], false);
+            for (int dt = 0; dt < 8; ++dt)
+                vf[dt][ks] = *reinterpret_cast<const uint4*>(vbase + (size_t)(dt * 16 + i16) * max_seq + p0);
+        }
+
+        // S tile pt: rows = heads kq*4 + r, column = position c0 + pt*16 + i16
+        float4_t sc[4];
+#pragma unroll
+        for (int pt = 0; pt < 4; ++pt) {
+            sc[pt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                sc[pt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, qf[s]),
+                                                                __builtin_bit_cast(half8_t, kf[pt][s]), sc[pt], 0, 0, 0);
+        }
+        float alpha[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int pt = 0; pt < 4; ++pt) {
+                const bool valid = c0 + pt * 16 + i16 < t1;
+                sc[pt][r] = valid ? sc[pt][r] * scale : -INFINITY;
+                mx = fmaxf(mx, sc[pt][r]);
             }
-        }
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            const float sv = valid ? s[h] * scale : -INFINITY;
-            const float m_new = fmaxf(m_run[h], wave_max(sv));
-            const float p = valid ? expf(sv - m_new) : 0.f;
-            const float alpha = expf(m_run[h] - m_new);  // exp(-inf) = 0 on the first chunk
-            l_run[h] = l_run[h] * alpha + wave_sum(p);
-            m_run[h] = m_new;
-            p_s[wave][h][lane] = p;
+            for (int off = 1; off < 16; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+            const float m_new = fmaxf(m_run[r], mx);  // finite: every chunk holds a valid position
+            alpha[r] = expf(m_run[r] - m_new);         // exp(-inf) = 0 on the first chunk
+            float sum = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[h][e] *= alpha;
+            for (int pt = 0; pt < 4; ++pt) {
+                const float pv = expf(sc[pt][r] - m_new);  // exp(-inf) = 0 for masked positions
+                sum += pv;
+                p_s[wave][(kq * 4 + r) * PP + pt * 16 + i16] = (half_t)pv;
+            }
+#pragma unroll
+            for (int off = 1; off < 16; off <<= 1) sum += __shfl_xor(sum, off, 64);
+            l_run[r] = l_run[r] * alpha[r] + sum;
+            m_run[r] = m_new;
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        // ---- phase B
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // A operand of O += P V: row = head i16, k = positions ks*32 + kq*8 .. +8 of the chunk
+        uint4 pa[2];
 #pragma unroll
-        for (int tt = 0; tt < 16; ++tt) {
-            const int tl = tt * 4 + tg;
-            if (c0 + tl < t1) {
-                const half8_t vh = __builtin_bit_cast(half8_t, vq[tt]);
+        for (int ks = 0; ks < 2; ++ks)
+            pa[ks] = *reinterpret_cast<const uint4*>(&p_s[wave][i16 * PP + ks * 32 + kq * 8]);
+        if (c0 + 64 > t1) {
+            // positions past the end carry weight 0 but whatever the cache holds there
+            // (possibly not finite): clear them
 #pragma unroll
-                for (int h = 0; h < G; ++h) {
-                    const float p = p_s[wave][h][tl];
+            for (int ks = 0; ks < 2; ++ks) {
+                const int p0 = c0 + ks * 32 + kq * 8;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[h][e] = __builtin_fmaf(p, (float)vh[e], acc[h][e]);
+                for (int dt = 0; dt < 8; ++dt) {
+                    half8_t v = __builtin_bit_cast(half8_t, vf[dt][ks]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (p0 + e >= t1) v[e] = (half_t)0.f;
+                    vf[dt][ks] = __builtin_bit_cast(uint4, v);
                 }
             }
         }
-        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha[r];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, pa[ks]),
+                                                                 __builtin_bit_cast(half8_t, vf[dt][ks]), acc[dt], 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();  // p_s is rewritten by the next chunk
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 
-    // merge the four position sub-streams of the wave
+    // acc[dt][r] is head kq*4 + r, dim dt*16 + i16
 #pragma unroll
-    for (int h = 0; h < G; ++h)
+    for (int r = 0; r < 4; ++r) {
+        const int h = kq * 4 + r;
+        if (h < G) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            acc[h][e] += __shfl_xor(acc[h][e], 16, 64);
-            acc[h][e] += __shfl_xor(acc[h][e], 32, 64);
-        }
-    if (tg == 0) {
-#pragma unroll
-        for (int h = 0; h < G; ++h)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc_s[wave][h][dl * 8 + e] = acc[h][e];
-    }
-    if (lane == 0) {
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-            m_s[wave][h] = m_run[h];
-            l_s[wave][h] = l_run[h];
+            for (int dt = 0; dt < 8; ++dt) acc_s[wave][h][dt * 16 + i16] = acc[dt][r];
+            if (i16 == 0) {
+                m_s[wave][h] = m_run[r];
+                l_s[wave][h] = l_run[r];
+            }
         }
     }
     __syncthreads();
 
-    // merge the four waves: thread -> (head, dims)
-    constexpr int ITEMS = G * D;  // outputs per block
+    // merge the four waves: thread -> (head, four dims)
+    constexpr int REC = D + 4;        // floats per (head, split) record: acc[D], m, l, two unused
+    constexpr int ITEMS = G * D / 4;  // <= 256
     const size_t head0 = ((size_t)b * kvh + g) * G;
-    for (int i = tid; i < ITEMS; i += 256) {
-        const int h = i / D, d = i % D;
-        float mm = fmaxf(fmaxf(m_s[0][h], m_s[1][h]), fmaxf(m_s[2][h], m_s[3][h]));
-        float ll = 0.f, a = 0.f;
+    const int h = tid / (D / 4), d = tid % (D / 4) * 4;
+    if (tid < ITEMS) {
+        const float mm = fmaxf(fmaxf(m_s[0][h], m_s[1][h]), fmaxf(m_s[2][h], m_s[3][h]));
+        float ll = 0.f;
+        float4_t a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const float f = (m_s[w][h] == -INFINITY) ? 0.f : expf(m_s[w][h] - mm);
             ll += l_s[w][h] * f;
-            a += acc_s[w][h][d] * f;
+            a += *reinterpret_cast<const float4_t*>(&acc_s[w][h][d]) * f;
         }
         if (splits == 1) {
-            out[(head0 + h) * D + d] = (half_t)(a / ll);
+            const half4_t o = {(half_t)(a[0] / ll), (half_t)(a[1] / ll), (half_t)(a[2] / ll), (half_t)(a[3] / ll)};
+            *reinterpret_cast<half4_t*>(out + (head0 + h) * D + d) = o;
         } else {
-            float* pp = partial + ((head0 + h) * splits + split) * (D + 2);
-            store_agent(pp + 2 + d, a);
-            if (d == 0) {
-                store_agent(pp, mm);
-                store_agent(pp + 1, ll);
-            }
+            float* pp = partial + ((head0 + h) * splits + split) * REC;
+            store_agent4(pp + d, a);
+            if (d == 0) store_agent4(pp + D, float4_t{mm, ll, 0.f, 0.f});
         }
     }
     if (splits == 1) return;
 
     __shared__ int is_last;
     if (!arrive_and_check_last(counters + (size_t)b * kvh + g, (unsigned)splits, &is_last)) return;
-    // Last block: merge the splits.  First the per-split maxima and sums of every
-    // head (independent loads, a few per thread) become weights in LDS, then each
-    // thread sums its output element over the splits.
-    constexpr int kMaxSplits = 64;
-    __shared__ float w_s[G][kMaxSplits];
-    __shared__ float l_tot[G];
-    float* ml = &acc_s[0][0][0];  // reuse: [G][splits][2]
-    for (int i = tid; i < G * splits; i += 256) {
-        const int h = i / splits, sp = i % splits;
-        const float* pp = partial + ((head0 + h) * splits + sp) * (D + 2);
-        ml[2 * i] = load_agent(pp);
-        ml[2 * i + 1] = load_agent(pp + 1);
-    }
-    __syncthreads();
-    if (tid < G) {
-        const int h = tid;
-        float mm = -INFINITY;
-        for (int sp = 0; sp < splits; ++sp) mm = fmaxf(mm, ml[2 * (h * splits + sp)]);
-        float ll = 0.f;
-        for (int sp = 0; sp < splits; ++sp) {
-            const float ms = ml[2 * (h * splits + sp)];
-            const float f = (ms == -INFINITY) ? 0.f : expf(ms - mm);
-            w_s[h][sp] = f;
-            ll += ml[2 * (h * splits + sp) + 1] * f;
-        }
-        l_tot[h] = ll;
-    }
-    __syncthreads();
-    for (int i = tid; i < ITEMS; i += 256) {
-        const int h = i / D, d = i % D;
-        const float* pp = partial + (head0 + h) * splits * (D + 2) + 2 + d;
-        float a = 0.f;
-        int sp = 0;
-        for (; sp + 8 <= splits; sp += 8) {
-            float v[8];
+    // Last block: merge the splits.  Every thread folds the splits of its four
+    // output elements with the running-maximum recurrence, reading each split's
+    // maximum, sum and partial values itself: the loads of up to 16 splits are
+    // independent and in flight together, so the merge costs one memory round
+    // trip.
+    constexpr int BATCH = 16;
+    if (tid < ITEMS) {
+        const float* pp = partial + (head0 + h) * splits * REC;
+        float mm = -INFINITY, ll = 0.f;
+        float4_t a = {0.f, 0.f, 0.f, 0.f};
+        for (int sp0 = 0; sp0 < splits; sp0 += BATCH) {
+            float ms[BATCH], ls[BATCH];
+            float4_t as[BATCH];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = load_agent(pp + (size_t)(sp + u) * (D + 2));
+            for (int u = 0; u < BATCH; ++u) {
+                const float* ps = pp + (size_t)min(sp0 + u, splits - 1) * REC;
+                as[u] = load_agent4(ps + d);
+                ms[u] = load_agent(ps + D);
+                ls[u] = load_agent(ps + D + 1);
+            }
+            wait_agent_loads(as);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) a += v[u] * w_s[h][sp + u];
+            for (int u = 0; u < BATCH; ++u) {
+                if (sp0 + u < splits && ms[u] != -INFINITY) {
+                    const float m_new = fmaxf(mm, ms[u]);
+                    const float f_old = expf(mm - m_new);  // exp(-inf) = 0 for the first split folded in
+                    const float f = expf(ms[u] - m_new);
+                    ll = ll * f_old + ls[u] * f;
+                    a = a * f_old + as[u] * f;
+                    mm = m_new;
+                }
+            }
         }
-        for (; sp < splits; ++sp) a += load_agent(pp + (size_t)sp * (D + 2)) * w_s[h][sp];
-        out[(head0 + h) * D + d] = (half_t)(a / l_tot[h]);
+        const half4_t o = {(half_t)(a[0] / ll), (half_t)(a[1] / ll), (half_t)(a[2] / ll), (half_t)(a[3] / ll)};
+        *reinterpret_cast<half4_t*>(out + (head0 + h) * D + d) = o;
     }
 }
 
@@ -456,7 +480,7 @@ static Scratch carve(const Llama& m, int batch, char* base) {
     s.gu = (half_t*)take((size_t)batch * 2 * c.ffn * 2);
     s.act = (half_t*)take((size_t)batch * c.ffn * 2);
     s.logits = (half_t*)take((size_t)batch * c.vocab * 2);
-    s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 2) * 4);
+    s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 4) * 4);
     s.total = off;
     return s;
 }
@@ -484,6 +508,7 @@ int mh_llama_create(void** handle, const mh_llama_config* cfg) {
     MH_REQUIRE(cfg->n_kv_heads > 0 && cfg->n_q_heads % cfg->n_kv_heads == 0, "mh_llama_create: bad head counts");
     const int g = cfg->n_q_heads / cfg->n_kv_heads;
     MH_REQUIRE(g == 1 || g == 2 || g == 4 || g == 8, "mh_llama_create: %d query heads per KV head unsupported", g);
+    MH_REQUIRE(cfg->max_seq >= 8 && cfg->max_seq % 8 == 0, "mh_llama_create: max_seq must be a multiple of 8, got %d", cfg->max_seq);
     MH_REQUIRE(cfg->hidden % 8 == 0 && cfg->hidden <= 8192, "mh_llama_create: hidden must be <= 8192 and a multiple of 8");
     MH_REQUIRE(cfg->ffn % 8 == 0, "mh_llama_create: ffn must be a multiple of 8");
     Llama* m = new (std::nothrow) Llama();

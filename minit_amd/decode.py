@@ -39,6 +39,7 @@ class LlamaDecoder:
 
     def __init__(self, config: dict, batch_max: int, max_seq: int):
         self.config = dict(config)
+        max_seq = (max_seq + 7) // 8 * 8   # the transposed V cache is read 8 positions (16 bytes) at a time
         self.batch_max, self.max_seq = batch_max, max_seq
         c = self.config
         self._cfg = LlamaConfig(c["n_layers"], c["hidden"], c["n_q_heads"], c["n_kv_heads"], c["head_dim"],
@@ -61,8 +62,13 @@ class LlamaDecoder:
     # ---- weights ------------------------------------------------------------------------------
     def _alloc_cache(self):
         c = self.config
-        shape = (self.batch_max, c["n_kv_heads"], self.max_seq, c["head_dim"])
-        return HIPTensor.allocate(shape, "float16"), HIPTensor.allocate(shape, "float16")
+        # K is [B, KVH, T, D]; V is kept transposed, [B, KVH, D, T], for the P.V matrix product
+        k_shape = (self.batch_max, c["n_kv_heads"], self.max_seq, c["head_dim"])
+        v_shape = (self.batch_max, c["n_kv_heads"], c["head_dim"], self.max_seq)
+        kc, vc = HIPTensor.allocate(k_shape, "float16"), HIPTensor.allocate(v_shape, "float16")
+        kc._memory.reset()
+        vc._memory.reset()
+        return kc, vc
 
     def _set_layer(self, index, linears, input_norm, post_norm, k_cache, v_cache):
         def ql(t):
@@ -131,9 +137,14 @@ class LlamaDecoder:
             linears = {name: tuple(HIPTensor.from_numpy(np.ascontiguousarray(a)) for a in layer[name][:3])
                        for name in ("qkv", "o", "gate_up", "down")}
             kc, vc = self._alloc_cache()
-            if k_cache is not None:
-                kc.copy_from_numpy(k_cache[l])
-                vc.copy_from_numpy(v_cache[l])
+            if k_cache is not None:   # host caches are [B, KVH, T, D] with T <= max_seq
+                t = k_cache[l].shape[2]
+                kpad = np.zeros(kc._shape, np.float16)
+                kpad[:, :, :t] = k_cache[l]
+                vpad = np.zeros(vc._shape, np.float16)
+                vpad[:, :, :, :t] = np.transpose(v_cache[l], (0, 1, 3, 2))
+                kc.copy_from_numpy(kpad)
+                vc.copy_from_numpy(vpad)
             self._set_layer(l, linears, HIPTensor.from_numpy(layer["input_norm"]),
                             HIPTensor.from_numpy(layer["post_norm"]), kc, vc)
         self._set_globals(HIPTensor.from_numpy(model["embed"]), HIPTensor.from_numpy(model["lm_head"]),
