@@ -122,6 +122,22 @@ int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight,
                    void* out, int M, int N, int K, int group_size, int bits,
                    void* workspace, size_t workspace_bytes);
 
+/* The gate|up projection of a gated MLP with SiLU*up fused into the reduction of
+ * the product (examples/llama3_70b.py:126-130 runs the product, sigmoid,
+ * multiply, multiply as four launches).  The N = 2 * ffn columns are laid out
+ * in blocks of 256: 128 gate columns followed by the 128 up columns of the same
+ * positions (column t*256 + c is gate column t*128 + c, column t*256 + 128 + c
+ * is up column t*128 + c; qzeros and scales permuted alike -- a load-time
+ * permutation of whole 8-column words).  out is [M, N / 2]:
+ *   out[m, t*128 + c] = fp16( silu(y[m, t*256 + c]) * y[m, t*256 + 128 + c] ),
+ * y the fp16-rounded product, silu and the multiply in fp32.  M <= 32,
+ * N % 256 == 0, group_size in {32, 64, 128, 256}; workspace as above and always
+ * required. */
+int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* qweight,
+                              const int32_t* qzeros, const void* scales, void* out,
+                              int M, int N, int K, int group_size, int bits,
+                              void* workspace, size_t workspace_bytes);
+
 /* ---- dense fp16 product --------------------------------------------------------
  * Replaces dispatch_matmul + minit_gemm (minit/cuda/dispatch.py:59-78,
  * minit/cuda/kernel/cublas.py:68-111) for batch == 1:
@@ -196,7 +212,8 @@ int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
  * sampling minit/chat/sample.py:11-14), enqueued from native code.  All
  * pointers are device pointers owned by the caller.
  *   qkv      fused q|k|v projection, GPTQ, [hidden] -> [(QH + 2 KVH) * D]
- *   gate_up  fused gate|up projection, [hidden] -> [2 * ffn]
+ *   gate_up  fused gate|up projection, [hidden] -> [2 * ffn], columns interleaved in
+ *            blocks of 128 gate / 128 up as for mh_gptq_matmul_silu_pairs (ffn % 128 == 0)
  *   k_cache  fp16 [batch_max, KVH, max_seq, D], v_cache fp16 [batch_max, KVH, D, max_seq]
  *            (V is kept transposed for the P.V matrix product); both appended in place;
  *            max_seq is a multiple of 8

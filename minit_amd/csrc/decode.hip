@@ -23,6 +23,10 @@ namespace mh {
 int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                          const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                          void* workspace, size_t workspace_bytes);
+bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
+int gptq_matmul_silu_pairs(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                           const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                           void* workspace, size_t workspace_bytes);
 
 // ---- small fused kernels --------------------------------------------------------------------------
 
@@ -122,15 +126,18 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(
     }
 }
 
-// act[b, f] = silu(gu[b, f]) * gu[b, F + f]; fp32 until the store.
+// act[b, t*128 + c] = silu(gu[b, t*256 + c]) * gu[b, t*256 + 128 + c] (gate and up
+// interleaved in blocks of 128 columns); fp32 until the store.  Only used when the
+// product kernel cannot apply this epilogue itself.
 __global__ void silu_mul_fused_kernel(const half_t* __restrict__ gu, half_t* __restrict__ act, int batch, int ffn) {
     const size_t n8 = (size_t)batch * ffn / 8;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     const int row8 = ffn / 8;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
-        const size_t b = i / row8, c = i % row8;
-        const half8_t g = __builtin_bit_cast(half8_t, reinterpret_cast<const uint4*>(gu + b * 2 * ffn)[c]);
-        const half8_t u = __builtin_bit_cast(half8_t, reinterpret_cast<const uint4*>(gu + b * 2 * ffn + ffn)[c]);
+        const size_t b = i / row8, c = i % row8;   // c: 8-column chunk of the output row
+        const half_t* gp = gu + b * 2 * ffn + c / 16 * 256 + c % 16 * 8;
+        const half8_t g = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(gp));
+        const half8_t u = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(gp + 128));
         half8_t o;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -510,7 +517,7 @@ int mh_llama_create(void** handle, const mh_llama_config* cfg) {
     MH_REQUIRE(g == 1 || g == 2 || g == 4 || g == 8, "mh_llama_create: %d query heads per KV head unsupported", g);
     MH_REQUIRE(cfg->max_seq >= 8 && cfg->max_seq % 8 == 0, "mh_llama_create: max_seq must be a multiple of 8, got %d", cfg->max_seq);
     MH_REQUIRE(cfg->hidden % 8 == 0 && cfg->hidden <= 8192, "mh_llama_create: hidden must be <= 8192 and a multiple of 8");
-    MH_REQUIRE(cfg->ffn % 8 == 0, "mh_llama_create: ffn must be a multiple of 8");
+    MH_REQUIRE(cfg->ffn % 128 == 0, "mh_llama_create: ffn must be a multiple of 128 (gate/up interleave)");
     Llama* m = new (std::nothrow) Llama();
     MH_REQUIRE(m != nullptr, "mh_llama_create: out of host memory");
     m->cfg = *cfg;
@@ -570,6 +577,7 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
     const int g = c.n_q_heads / c.n_kv_heads;
     const int splits = attn_splits(*m, batch);
     const unsigned ew_grid = (unsigned)compute_units() * 4;
+    const bool fused_silu = gemm_silu_pairs_supported(batch, 2 * c.ffn, c.hidden, c.group_size, c.bits);
 
     auto linear = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k) -> int {
         return gptq_matmul_dispatch(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
@@ -598,9 +606,16 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
             if (rc) return rc;
             hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, s.delta,
                                (const half_t*)L.post_norm, s.xn, c.hidden, c.rms_eps);
-            rc = linear(s.xn, L.gate_up, s.gu, 2 * c.ffn, c.hidden);
-            if (rc) return rc;
-            hipLaunchKernelGGL(silu_mul_fused_kernel, dim3(ew_grid), dim3(256), 0, st, s.gu, s.act, batch, c.ffn);
+            if (fused_silu) {
+                rc = gptq_matmul_silu_pairs(st, s.xn, L.gate_up.qweight, L.gate_up.qzeros, L.gate_up.scales, s.act,
+                                            batch, 2 * c.ffn, c.hidden, c.group_size, c.bits, s.gptq_ws,
+                                            s.gptq_ws_bytes);
+                if (rc) return rc;
+            } else {
+                rc = linear(s.xn, L.gate_up, s.gu, 2 * c.ffn, c.hidden);
+                if (rc) return rc;
+                hipLaunchKernelGGL(silu_mul_fused_kernel, dim3(ew_grid), dim3(256), 0, st, s.gu, s.act, batch, c.ffn);
+            }
             rc = linear(s.act, L.down, s.delta, c.hidden, c.ffn);
             if (rc) return rc;
             const half_t* next_norm =

@@ -10,9 +10,10 @@ int gptq_gemv_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
                      void* workspace, size_t workspace_bytes);
 bool gemm_supported(int M, int N, int K, int group_size, int bits);
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits);
+bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
-                     void* workspace, size_t workspace_bytes);
+                     void* workspace, size_t workspace_bytes, int epilogue);
 int gptq_generic_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                         const void* scales, const int32_t* g_idx, void* out, int M, int N, int K,
                         int group_size, int bits);
@@ -29,8 +30,18 @@ int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweig
                                 workspace_bytes);
     if (gemm_supported(M, N, K, group_size, bits))
         return gptq_gemm_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
-                                workspace_bytes);
+                                workspace_bytes, kEpilogueNone);
     return gptq_generic_launch(stream, x, qweight, qzeros, scales, nullptr, out, M, N, K, group_size, bits);
+}
+
+// out [M, N / 2] = silu(gate) * up of the product, for weights whose column tiles
+// interleave gate and up (kEpilogueSiluPairs); the caller has checked
+// gemm_silu_pairs_supported().
+int gptq_matmul_silu_pairs(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                           const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                           void* workspace, size_t workspace_bytes) {
+    return gptq_gemm_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
+                            workspace_bytes, kEpilogueSiluPairs);
 }
 }  // namespace mh
 
@@ -72,7 +83,7 @@ int mh_gptq_gemm(mh_stream_t stream, const void* x, const int32_t* qweight, cons
                "mh_gptq_gemm: needs N %% 8 == 0, K %% 32 == 0, group_size %% 32 == 0 (M=%d N=%d K=%d g=%d)",
                M, N, K, group_size);
     return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
-                            workspace, workspace_bytes);
+                            workspace, workspace_bytes, kEpilogueNone);
 }
 
 int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
@@ -87,10 +98,20 @@ int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight, co
                                     bits, workspace, workspace_bytes);
         if (gemm_supported(M, N, K, group_size, bits))
             return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size,
-                                    bits, workspace, workspace_bytes);
+                                    bits, workspace, workspace_bytes, kEpilogueNone);
     }
     return gptq_generic_launch(as_stream(stream), x, qweight, qzeros, scales, g_idx, out, M, N, K,
                                group_size, bits);
+}
+
+int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                              const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                              void* workspace, size_t workspace_bytes) {
+    int rc = check_gptq_args("mh_gptq_matmul_silu_pairs", x, qweight, qzeros, scales, out, M, N, K, group_size, bits);
+    if (rc) return rc;
+    if (M == 0) return MH_OK;
+    return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
+                            workspace, workspace_bytes, kEpilogueSiluPairs);
 }
 
 }  // extern "C"

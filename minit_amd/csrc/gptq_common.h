@@ -118,6 +118,19 @@ __device__ __forceinline__ void pair_activations<8>(const uint32_t* x, uint32_t*
     xp[1] = (x[0] >> 16) | (x[1] & 0xFFFF0000u);
 }
 
+// Epilogues of the quantized product.  kEpilogueSiluPairs: every 256-column
+// tile holds 128 "gate" columns followed by the 128 matching "up" columns and
+// the result has N / 2 columns, out[m, t*128 + c] = silu(y[m, t*256 + c]) *
+// y[m, t*256 + 128 + c] with y rounded to fp16 first (what a separate
+// SiLU*up pass over the fp16 product would read) and fp32 until the store.
+constexpr int kEpilogueNone = 0;
+constexpr int kEpilogueSiluPairs = 1;
+
+__device__ __forceinline__ half_t silu_pair(half_t gate, half_t up) {
+    const float g = (float)gate;
+    return (half_t)(g / (1.f + expf(-g)) * (float)up);
+}
+
 // The workspace of the split-K kernels starts with one arrival counter per
 // 256-column tile.  The caller zero-fills the workspace once; every launch
 // leaves the counters at zero again.

@@ -218,7 +218,8 @@ __global__ __launch_bounds__(256) void gptq_gemm_kernel(
     }
 }
 
-void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, size_t mn, int split_k);
+void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
+                            int epilogue);
 
 // ---- small-M variant (M <= 32: decode batches) --------------------------------------------------
 // Same operand mapping, a schedule built around two facts measured on this part:
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
     half_t* __restrict__ out, float* partial, unsigned* counters,
-    int M, int N, int K, int steps_total, int stages_per_block, int split_k) {
+    int M, int N, int K, int steps_total, int stages_per_block, int split_k, int epilogue) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
     constexpr uint32_t MASK = Packing<BITS>::kMask;
@@ -400,7 +401,9 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     // which is what workgroups on other XCDs see) and counts itself in; the one
     // that arrives last adds the partials in split order -- a fixed order, so the
     // result does not depend on which workgroup that is -- and puts the counter
-    // back to zero for the next launch.
+    // back to zero for the next launch.  The SiLU-pair epilogue always takes this
+    // route (its two operands sit in different waves' accumulators).
+    const bool direct = split_k == 1 && epilogue == kEpilogueNone;
     if (active) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -408,7 +411,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             for (int r = 0; r < 4; ++r) {
                 const int m = mt * 16 + kq * 4 + r;
                 if (m >= M) continue;
-                if (split_k == 1) {
+                if (direct) {
                     const half4_t h = {(half_t)acc[mt][0][r], (half_t)acc[mt][1][r], (half_t)acc[mt][2][r],
                                        (half_t)acc[mt][3][r]};
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
@@ -422,16 +425,13 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 }
             }
     }
-    if (split_k == 1 || counters == nullptr) return;  // without counters a second kernel adds the partials
+    if (direct || counters == nullptr) return;  // without counters a second kernel adds the partials
 
     __shared__ int is_last;
     if (!arrive_and_check_last(&counters[tile], (unsigned)split_k, &is_last)) return;
     constexpr int BATCH = 8;  // partial loads in flight per thread
     const size_t plane = (size_t)M * N;
-    for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
-        const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
-        if (c >= N) continue;
-        const float* p = partial + (size_t)m * N + c;
+    auto sum_splits = [&](const float* p) {
         float4_t s = {0.f, 0.f, 0.f, 0.f};
         for (int sp = 0; sp < split_k; sp += BATCH) {
             float4_t v[BATCH];
@@ -443,6 +443,25 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             for (int u = 0; u < BATCH; ++u)
                 if (sp + u < split_k) s += v[u];
         }
+        return s;
+    };
+    if (epilogue == kEpilogueSiluPairs) {
+        // columns [0, 128) of the tile are gate, [128, 256) the matching up columns
+        for (int item = tid; item < M * (kGemmCols / 8); item += 256) {
+            const int m = item / (kGemmCols / 8), c4 = item % (kGemmCols / 8) * 4;
+            const float* p = partial + (size_t)m * N + tile * kGemmCols + c4;
+            const float4_t g = sum_splits(p), u = sum_splits(p + kGemmCols / 2);
+            half4_t h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
+            *reinterpret_cast<half4_t*>(out + (size_t)m * (N / 2) + tile * (kGemmCols / 2) + c4) = h;
+        }
+        return;
+    }
+    for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
+        const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
+        if (c >= N) continue;
+        const float4_t s = sum_splits(partial + (size_t)m * N + c);
         const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
         *reinterpret_cast<half4_t*>(out + (size_t)m * N + c) = h;
     }
@@ -528,10 +547,17 @@ bool gemm_supported(int M, int N, int K, int group_size, int bits) {
            K % group_size == 0;
 }
 
+// The epilogue out[m, j] = silu(y[m, gate(j)]) * y[m, up(j)] on column tiles laid out as
+// 128 gate columns followed by their 128 up columns; served by the small-M kernel only.
+bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits) {
+    return gemm_supported(M, N, K, group_size, bits) && use_small(M, group_size) && N % kGemmCols == 0;
+}
+
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)bits;
     const GemmPlan p = plan_gemm(M, N, K, group_size);
-    if (p.split_k <= 1) return 0;
+    // the small-M kernel may be asked for an epilogue that goes through the partials even unsplit
+    if (p.split_k <= 1 && !use_small(M, group_size)) return 0;
     return kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float);
 }
 
@@ -545,13 +571,13 @@ static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, co
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size / 32,
                        p.steps_total, p.steps_per_block, p.split_k);
-    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone);
 }
 
 template <int BITS, int MT>
 static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                               const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
-                              int N, int K, int group_size) {
+                              int N, int K, int group_size, int epilogue) {
     // workspace: [tile counters, zero between launches][fp32 partials]
     // in-kernel reduction by the last workgroup of a tile pays for few rows only
     unsigned* counters =
@@ -561,7 +587,8 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
 #define MH_LAUNCH_SMALL(SPG)                                                                                  \
     hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG>), grid, dim3(256), 0, stream, (const half_t*)x,  \
                        (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,  \
-                       partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k)
+                       partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k,  \
+                       epilogue)
     switch (group_size / 32) {
         case 1: MH_LAUNCH_SMALL(1); break;
         case 2: MH_LAUNCH_SMALL(2); break;
@@ -569,18 +596,21 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
         default: MH_LAUNCH_SMALL(8); break;
     }
 #undef MH_LAUNCH_SMALL
-    if (p.split_k > 1 && counters == nullptr) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
+    if (counters == nullptr && (p.split_k > 1 || epilogue != kEpilogueNone))
+        launch_splitk_finalize(stream, partial, out, M, N, p.split_k, epilogue);
 }
 
 template <int BITS>
 static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                            const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
-                           int N, int K, int group_size) {
+                           int N, int K, int group_size, int epilogue) {
     if (use_small(M, group_size)) {
         if (p.mt == 1)
-            launch_gemm_small<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+            launch_gemm_small<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size,
+                                       epilogue);
         else
-            launch_gemm_small<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+            launch_gemm_small<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size,
+                                       epilogue);
         return;
     }
     switch (p.mt) {
@@ -593,10 +623,13 @@ static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x,
 
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
-                     void* workspace, size_t workspace_bytes) {
+                     void* workspace, size_t workspace_bytes, int epilogue) {
     const GemmPlan p = plan_gemm(M, N, K, group_size);
     const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
-    if (p.split_k > 1) {
+    if (epilogue != kEpilogueNone && !gemm_silu_pairs_supported(M, N, K, group_size, bits))
+        return fail(MH_ERR_INVALID, "gptq gemm: the SiLU-pair epilogue needs M <= %d, N %% 256 == 0 and a group of 32..256",
+                    kSmallMaxM);
+    if (p.split_k > 1 || epilogue != kEpilogueNone) {
         if (workspace == nullptr || workspace_bytes < need)
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
                         workspace ? workspace_bytes : (size_t)0);
@@ -604,9 +637,9 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace must be 256-byte aligned");
     }
     if (bits == 4)
-        launch_gemm_mt<4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+        launch_gemm_mt<4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size, epilogue);
     else
-        launch_gemm_mt<8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size);
+        launch_gemm_mt<8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size, epilogue);
     MH_CHECK_LAUNCH();
     return MH_OK;
 }

@@ -174,7 +174,36 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __res
     *reinterpret_cast<half4_t*>(out + i) = h;
 }
 
-void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, size_t mn, int split_k) {
+// The same with the SiLU-pair epilogue: out is [M, N / 2].
+__global__ __launch_bounds__(256) void splitk_finalize_silu_kernel(const float* __restrict__ partial,
+                                                                   half_t* __restrict__ out, int M, int N,
+                                                                   int split_k) {
+    const size_t half_n = (size_t)N / 2;
+    const size_t o = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (o >= (size_t)M * half_n) return;
+    const size_t m = o / half_n, j = o % half_n;
+    const size_t gate = m * N + j / 128 * 256 + j % 128;
+    const size_t mn = (size_t)M * N;
+    float4_t g = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < split_k; ++sp) {
+        g += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + gate);
+        u += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + gate + 128);
+    }
+    half4_t h;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
+    *reinterpret_cast<half4_t*>(out + o) = h;
+}
+
+void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
+                            int epilogue) {
+    if (epilogue == kEpilogueSiluPairs) {
+        const size_t threads = ((size_t)M * (N / 2) + 3) / 4;
+        hipLaunchKernelGGL(splitk_finalize_silu_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                           stream, partial, (half_t*)out, M, N, split_k);
+        return;
+    }
+    const size_t mn = (size_t)M * N;
     const size_t threads = (mn + 3) / 4;
     hipLaunchKernelGGL(splitk_finalize_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
                        partial, (half_t*)out, mn, split_k);
@@ -238,7 +267,7 @@ static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, co
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, N, K, group_size / P,
                        p.steps_total, p.steps_per_wave, p.split_k);
-    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, (size_t)M * N, p.split_k);
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone);
 }
 
 template <int BITS, int M>

@@ -34,6 +34,27 @@ LLAMA3_70B = dict(n_layers=80, hidden=8192, n_q_heads=64, n_kv_heads=8, head_dim
                   vocab=128256, group_size=128, bits=4, rope_theta=5e5, rms_eps=1e-5)
 
 
+def interleave_gate_up(qweight, qzeros, scales, bits=4):
+    """Column order of the fused gate|up projection that the device path expects.
+
+    ``[gate (ffn) | up (ffn)]`` becomes blocks of 256 columns holding 128 gate
+    columns followed by the 128 up columns of the same positions, so one column
+    tile of the product kernel sees both operands of ``silu(gate) * up``.  128 is
+    a multiple of the 8 (or 4) columns packed into a ``qzeros`` word, so whole
+    words move and nothing is repacked.
+    """
+    n = qweight.shape[1]
+    ffn = n // 2
+    assert ffn % 128 == 0, "ffn must be a multiple of 128"
+    t = np.arange(ffn // 128)[:, None, None]
+    c = np.arange(128)[None, None, :]
+    part = np.arange(2)[None, :, None]            # 0 = gate, 1 = up
+    cols = (part * ffn + t * 128 + c).reshape(-1)  # new column j takes old column cols[j]
+    per = 32 // bits
+    words = cols.reshape(-1, per)[:, 0] // per
+    return qweight[:, cols], qzeros[:, words], scales[:, cols]
+
+
 class LlamaDecoder:
     """Owns the device tensors of one model and its KV cache."""
 
@@ -134,7 +155,9 @@ class LlamaDecoder:
     def load_host(self, model: dict, k_cache=None, v_cache=None):
         """Uploads a model given as numpy arrays (the layout of ``oracle.decode``)."""
         for l, layer in enumerate(model["layers"]):
-            linears = {name: tuple(HIPTensor.from_numpy(np.ascontiguousarray(a)) for a in layer[name][:3])
+            host = {name: layer[name][:3] for name in ("qkv", "o", "gate_up", "down")}
+            host["gate_up"] = interleave_gate_up(*host["gate_up"], bits=self.config["bits"])
+            linears = {name: tuple(HIPTensor.from_numpy(np.ascontiguousarray(a)) for a in host[name])
                        for name in ("qkv", "o", "gate_up", "down")}
             kc, vc = self._alloc_cache()
             if k_cache is not None:   # host caches are [B, KVH, T, D] with T <= max_seq

@@ -48,6 +48,7 @@ PROTOTYPES = {
     "mh_gptq_gemv": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_gptq_gemm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_gptq_matmul": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
+    "mh_gptq_matmul_silu_pairs": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_f16_matmul_nk": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
     "mh_i8_gemm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int]),
     "mh_i8_transpose": (c_int, [_P, _P, _P, c_int, c_int]),

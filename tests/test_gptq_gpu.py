@@ -214,3 +214,29 @@ def test_operator_api_drop_in(hip):
     wd = w.dequantize().numpy()
     np.testing.assert_array_equal(wd.view(np.uint16),
                                   O.dequantize_packed(qweight, qzeros, scales, None, 4, g).view(np.uint16))
+
+
+@pytest.mark.parametrize("m,k,ffn", [(1, 512, 256), (3, 1024, 384), (8, 256, 128), (16, 512, 256), (32, 768, 512)])
+def test_silu_pairs_epilogue(hip, m, k, ffn):
+    """gate|up product with SiLU*up applied in the reduction: equals the plain
+    product followed by silu(gate) * up on the interleaved column blocks."""
+    from minit_amd import synthetic
+    from minit_amd.decode import interleave_gate_up
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    g = 128
+    qweight, qzeros, scales = interleave_gate_up(*_weights(k, 2 * ffn, g, 4, seed=21))
+    x = synthetic.activations("test21", f"x{m}", (m, k))
+    dx, dq, dz, ds = _dev(hip, x), _dev(hip, qweight), _dev(hip, qzeros), _dev(hip, scales)
+    out = HIPTensor.allocate((m, ffn), "float16")
+    ws = memory.workspace(max(hip.call("mh_gptq_workspace_bytes", m, 2 * ffn, k, g, 4), 256))
+    hip.call("mh_gptq_matmul_silu_pairs", None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, out.data_ptr,
+             m, 2 * ffn, k, g, 4, ws._pointer, ws._size)
+    y = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, 4)      # the same device product
+    y = y.reshape(m, ffn // 128, 2, 128)
+    ref = O.silu_mul_f64(y[:, :, 0], y[:, :, 1]).reshape(m, ffn)
+    got = out.numpy()
+    ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64)
+    assert (np.abs(got.astype(np.float64) - ref) <= 1.0 * ulp + 1e-7).all()
+    # and the product itself is the oracle's
+    assert_fp16_close(y.reshape(m, 2 * ffn), O.matmul_f64(x, qweight, qzeros, scales, None, 4, g), what="gate|up")
