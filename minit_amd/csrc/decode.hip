@@ -12,7 +12,7 @@
 //   * residual add + RMSNorm, RoPE + cache append, SiLU*up are fused kernels.
 //   * sampling is an on-device argmax (the reference copies the logits to the
 //     host, minit/chat/sample.py:11-14).
-#include "common.h"
+#include "gptq_common.h"
 
 #include <cstring>
 #include <new>
@@ -24,6 +24,10 @@ int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweig
                          const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                          void* workspace, size_t workspace_bytes);
 bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
+bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits);
+int gptq_matmul_fused(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse);
 int gptq_matmul_silu_pairs(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                            const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                            void* workspace, size_t workspace_bytes);
@@ -439,6 +443,7 @@ struct Llama {
 struct Scratch {
     half_t *h, *xn, *qkv, *q, *attn, *delta, *gu, *act, *logits;
     float* attn_partial;
+    float *ssq_a, *ssq_b;  // per-tile sums of squares of the residual stream, [batch, hidden / 256]
     unsigned* attn_counters;
     void* gptq_ws;
     size_t gptq_ws_bytes;
@@ -488,6 +493,8 @@ static Scratch carve(const Llama& m, int batch, char* base) {
     s.act = (half_t*)take((size_t)batch * c.ffn * 2);
     s.logits = (half_t*)take((size_t)batch * c.vocab * 2);
     s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 4) * 4);
+    s.ssq_a = (float*)take((size_t)batch * ((c.hidden + 255) / 256) * 4);
+    s.ssq_b = (float*)take((size_t)batch * ((c.hidden + 255) / 256) * 4);
     s.total = off;
     return s;
 }
@@ -584,6 +591,20 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                                     s.gptq_ws, s.gptq_ws_bytes);
     };
 
+    // With few rows the residual add and RMSNorm around the linears are folded into
+    // them: o and down add their result to the residual stream and leave per-tile
+    // sums of squares, qkv and gate|up normalise that stream while staging it.
+    const bool fused_norm = gemm_norm_fusion_supported(batch, c.hidden, c.n_q_heads * c.head_dim, c.group_size, c.bits) &&
+                            gemm_norm_fusion_supported(batch, c.hidden, c.ffn, c.group_size, c.bits) &&
+                            gemm_norm_fusion_supported(batch, qkv_n, c.hidden, c.group_size, c.bits) &&
+                            gemm_norm_fusion_supported(batch, 2 * c.ffn, c.hidden, c.group_size, c.bits) && fused_silu;
+    const int res_tiles = c.hidden / 256;
+    auto fused = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k, int epilogue,
+                     const SmallFuse& fuse) -> int {
+        return gptq_matmul_fused(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
+                                 s.gptq_ws, s.gptq_ws_bytes, epilogue, fuse);
+    };
+
     for (int step = 0; step < n_steps; ++step) {
         hipLaunchKernelGGL(embed_gather_kernel, dim3(batch), dim3(256), 0, st, tokens, (const half_t*)m->embed, s.h,
                            c.hidden, c.vocab);
@@ -591,7 +612,17 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                            (const half_t*)m->layers[0].input_norm, s.xn, c.hidden, c.rms_eps);
         for (int l = 0; l < c.n_layers; ++l) {
             const mh_llama_layer& L = m->layers[l];
-            int rc = linear(s.xn, L.qkv, s.qkv, qkv_n, c.hidden);
+            int rc;
+            if (fused_norm && l > 0) {  // normalise the residual stream left by the previous down projection
+                SmallFuse f;
+                f.ssq_in = s.ssq_a;
+                f.ssq_tiles = res_tiles;
+                f.norm_w = (const half_t*)L.input_norm;
+                f.eps = c.rms_eps;
+                rc = fused(s.h, L.qkv, s.qkv, qkv_n, c.hidden, kEpilogueNone, f);
+            } else {
+                rc = linear(s.xn, L.qkv, s.qkv, qkv_n, c.hidden);
+            }
             if (rc) return rc;
             hipLaunchKernelGGL(rope_kv_append_kernel, dim3(c.n_q_heads + 2 * c.n_kv_heads, batch), dim3(64), 0, st,
                                s.qkv, m->cos, m->sin, positions, s.q, (half_t*)L.k_cache, (half_t*)L.v_cache,
@@ -601,6 +632,23 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                 case 2: launch_attn<2>(st, *m, s, L, positions, batch, splits); break;
                 case 4: launch_attn<4>(st, *m, s, L, positions, batch, splits); break;
                 default: launch_attn<8>(st, *m, s, L, positions, batch, splits); break;
+            }
+            if (fused_norm) {
+                SmallFuse res;
+                res.ssq_out = s.ssq_b;
+                rc = fused(s.attn, L.o, s.h, c.hidden, c.n_q_heads * c.head_dim, kEpilogueResidual, res);
+                if (rc) return rc;
+                SmallFuse f;
+                f.ssq_in = s.ssq_b;
+                f.ssq_tiles = res_tiles;
+                f.norm_w = (const half_t*)L.post_norm;
+                f.eps = c.rms_eps;
+                rc = fused(s.h, L.gate_up, s.act, 2 * c.ffn, c.hidden, kEpilogueSiluPairs, f);
+                if (rc) return rc;
+                res.ssq_out = s.ssq_a;
+                rc = fused(s.act, L.down, s.h, c.hidden, c.ffn, kEpilogueResidual, res);
+                if (rc) return rc;
+                continue;
             }
             rc = linear(s.attn, L.o, s.delta, c.hidden, c.n_q_heads * c.head_dim);
             if (rc) return rc;
@@ -623,6 +671,9 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
             hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, s.delta, next_norm, s.xn,
                                c.hidden, c.rms_eps);
         }
+        if (fused_norm)  // the last residual stream still wants its norm
+            hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, (const half_t*)nullptr,
+                               (const half_t*)m->final_norm, s.xn, c.hidden, c.rms_eps);
         int rc = mh_f16_matmul_nk(stream, s.xn, m->lm_head, s.logits, batch, c.vocab, c.hidden);
         if (rc) return rc;
         hipLaunchKernelGGL(argmax_advance_kernel, dim3(batch), dim3(1024), 0, st, s.logits, tokens,

@@ -13,7 +13,7 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits);
 bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
-                     void* workspace, size_t workspace_bytes, int epilogue);
+                     void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse);
 int gptq_generic_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                         const void* scales, const int32_t* g_idx, void* out, int M, int N, int K,
                         int group_size, int bits);
@@ -30,7 +30,7 @@ int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweig
                                 workspace_bytes);
     if (gemm_supported(M, N, K, group_size, bits))
         return gptq_gemm_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
-                                workspace_bytes, kEpilogueNone);
+                                workspace_bytes, kEpilogueNone, SmallFuse{});
     return gptq_generic_launch(stream, x, qweight, qzeros, scales, nullptr, out, M, N, K, group_size, bits);
 }
 
@@ -41,7 +41,16 @@ int gptq_matmul_silu_pairs(hipStream_t stream, const void* x, const int32_t* qwe
                            const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                            void* workspace, size_t workspace_bytes) {
     return gptq_gemm_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
-                            workspace_bytes, kEpilogueSiluPairs);
+                            workspace_bytes, kEpilogueSiluPairs, SmallFuse{});
+}
+
+// The product with the fusions of SmallFuse / an epilogue chosen by the caller
+// (the decode loop); the caller has checked the *_supported() predicate.
+int gptq_matmul_fused(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
+                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
+    return gptq_gemm_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, workspace,
+                            workspace_bytes, epilogue, fuse);
 }
 }  // namespace mh
 
@@ -83,7 +92,7 @@ int mh_gptq_gemm(mh_stream_t stream, const void* x, const int32_t* qweight, cons
                "mh_gptq_gemm: needs N %% 8 == 0, K %% 32 == 0, group_size %% 32 == 0 (M=%d N=%d K=%d g=%d)",
                M, N, K, group_size);
     return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
-                            workspace, workspace_bytes, kEpilogueNone);
+                            workspace, workspace_bytes, kEpilogueNone, SmallFuse{});
 }
 
 int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
@@ -98,7 +107,7 @@ int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight, co
                                     bits, workspace, workspace_bytes);
         if (gemm_supported(M, N, K, group_size, bits))
             return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size,
-                                    bits, workspace, workspace_bytes, kEpilogueNone);
+                                    bits, workspace, workspace_bytes, kEpilogueNone, SmallFuse{});
     }
     return gptq_generic_launch(as_stream(stream), x, qweight, qzeros, scales, g_idx, out, M, N, K,
                                group_size, bits);
@@ -111,7 +120,7 @@ int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* 
     if (rc) return rc;
     if (M == 0) return MH_OK;
     return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
-                            workspace, workspace_bytes, kEpilogueSiluPairs);
+                            workspace, workspace_bytes, kEpilogueSiluPairs, SmallFuse{});
 }
 
 }  // extern "C"

@@ -123,8 +123,25 @@ __device__ __forceinline__ void pair_activations<8>(const uint32_t* x, uint32_t*
 // the result has N / 2 columns, out[m, t*128 + c] = silu(y[m, t*256 + c]) *
 // y[m, t*256 + 128 + c] with y rounded to fp16 first (what a separate
 // SiLU*up pass over the fp16 product would read) and fp32 until the store.
+// kEpilogueResidual: out is the residual stream itself, out[m, n] = fp16(out[m, n] +
+// fp16(y[m, n])) (the fp16 add of the models, examples/llama3_70b.py:159-162), and
+// the sum of squares of the new values over each 256-column tile is left in
+// ssq_out[m, tile] for the consumer that normalises the row (SmallFuse).
 constexpr int kEpilogueNone = 0;
 constexpr int kEpilogueSiluPairs = 1;
+constexpr int kEpilogueResidual = 2;
+
+// Optional fusions of the small-M product kernel around RMSNorm
+// (minit/cuda/kernel/cuda/rms_norm.py:69-89): a producer with kEpilogueResidual
+// fills ssq_out; a consumer given ssq_in / norm_w normalises its activations while
+// staging them.
+struct SmallFuse {
+    const float* ssq_in = nullptr;   // [M, ssq_tiles]
+    int ssq_tiles = 0;
+    const half_t* norm_w = nullptr;  // [K]
+    float eps = 0.f;
+    float* ssq_out = nullptr;        // [M, N / 256]
+};
 
 __device__ __forceinline__ half_t silu_pair(half_t gate, half_t up) {
     const float g = (float)gate;

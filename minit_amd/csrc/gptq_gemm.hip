@@ -237,12 +237,19 @@ void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out,
 // weights per wave in flight at all times.
 constexpr int kSmallDepth = 8;  // steps per stage = ring depth
 
-template <int BITS, int MT, int SPG>
+// NORM: the product is taken of the RMS-normalised activations without a pass
+// over the row: while staging, x'[m, k] = fp16(x[m, k] * norm_w[k]) (one packed
+// fp16 multiply per two elements); the row factor 1 / sqrt(ssq[m] / K + eps), with
+// ssq[m] the sum of the fuse.ssq_tiles per-tile sums of squares that the producer
+// of x left behind (kEpilogueResidual), scales the fp32 accumulators at the end.
+// Against normalise-then-round the one fp16 rounding per activation moves from
+// after both factors to after the first.
+template <int BITS, int MT, int SPG, bool NORM>
 __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
-    half_t* __restrict__ out, float* partial, unsigned* counters,
-    int M, int N, int K, int steps_total, int stages_per_block, int split_k, int epilogue) {
+    half_t* out, float* partial, unsigned* counters,
+    int M, int N, int K, int steps_total, int stages_per_block, int split_k, int epilogue, SmallFuse fuse) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
     constexpr uint32_t MASK = Packing<BITS>::kMask;
@@ -258,6 +265,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 
     __shared__ uint4 xs[2][BM * RS];
     __shared__ uint32_t cs[2][GPS][3][kGemmCols];  // scale pair, zero_lo pair, zero_hi pair
+    __shared__ float inv_rms_s[NORM ? BM : 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -290,6 +298,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 
     // ---- staging of activations and constants: global -> registers -> LDS
     uint4 xr[XL];
+    uint4 wr[NORM ? XL : 1];  // norm weights of the same k
     uint4 sr;       // eight scales of one group
     uint32_t zr[8 / P];
     int x_row[XL], x_chunk[XL];
@@ -306,6 +315,11 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 #pragma unroll
         for (int u = 0; u < XL; ++u)
             xr[u] = *reinterpret_cast<const uint4*>(x + (size_t)x_row[u] * K + (size_t)sclamp * 32 + x_chunk[u] * 8);
+        if constexpr (NORM) {
+#pragma unroll
+            for (int u = 0; u < XL; ++u)
+                wr[u] = *reinterpret_cast<const uint4*>(fuse.norm_w + (size_t)sclamp * 32 + x_chunk[u] * 8);
+        }
         const int g = min(sclamp / SPG + c_group, g_last);
         sr = *reinterpret_cast<const uint4*>(scales + (size_t)g * N + c_colg);
 #pragma unroll
@@ -314,7 +328,12 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     auto store_stage = [&](int buf, int stage_step) {
 #pragma unroll
         for (int u = 0; u < XL; ++u) {
-            const uint32_t in[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+            uint32_t in[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+            if constexpr (NORM) {  // x * w in fp16; the row's 1 / rms scales the accumulators at the end
+                const uint32_t wv[4] = {wr[u].x, wr[u].y, wr[u].z, wr[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) in[e] = as_u32(as_half2(in[e]) * as_half2(wv[e]));
+            }
             uint32_t o[4];
             if constexpr (BITS == 4) {
                 pair_activations<4>(in, o);
@@ -341,6 +360,23 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     };
 
     fetch_stage(step_begin);
+    if constexpr (NORM) {
+        // 1 / rms of every row from the producer's per-tile sums of squares: 32
+        // lanes per row read the tiles in parallel (the loads travel with those of
+        // the first stage) and are folded by shuffles, a fixed order; read back
+        // after the K loop
+        static_assert(BM * 32 <= 512, "two passes of the 256 threads cover every row");
+#pragma unroll
+        for (int pass = 0; pass < (BM * 32 + 255) / 256; ++pass) {
+            const int row = pass * 8 + (tid >> 5), t0 = tid & 31;
+            float ss = 0.f;
+            if (row < M)
+                for (int t = t0; t < fuse.ssq_tiles; t += 32) ss += fuse.ssq_in[(size_t)row * fuse.ssq_tiles + t];
+#pragma unroll
+            for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
+            if (t0 == 0 && row < BM) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+        }
+    }
     store_stage(0, step_begin);
     fetch_stage(step_begin + D);
     __syncthreads();
@@ -403,7 +439,17 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     // result does not depend on which workgroup that is -- and puts the counter
     // back to zero for the next launch.  The SiLU-pair epilogue always takes this
     // route (its two operands sit in different waves' accumulators).
-    const bool direct = split_k == 1 && epilogue == kEpilogueNone;
+    if constexpr (NORM) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float inv = inv_rms_s[mt * 16 + kq * 4 + r];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[mt][t][r] *= inv;
+            }
+    }
+    const bool direct = split_k == 1 && epilogue == kEpilogueNone;  // the other epilogues need the whole tile
     if (active) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -455,6 +501,26 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 #pragma unroll
             for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
             *reinterpret_cast<half4_t*>(out + (size_t)m * (N / 2) + tile * (kGemmCols / 2) + c4) = h;
+        }
+        return;
+    }
+    if (epilogue == kEpilogueResidual) {
+        // a wave owns one row of the tile per pass (64 lanes x 4 columns), so the
+        // row's sum of squares is one wave reduction; N is a multiple of 256
+        for (int base = 0; base < M * (kGemmCols / 4); base += 256) {
+            const int m = base / (kGemmCols / 4) + wave, c = tile * kGemmCols + lane * 4;
+            float ss = 0.f;
+            if (m < M) {
+                const float4_t s = sum_splits(partial + (size_t)m * N + c);
+                half_t* hp = out + (size_t)m * N + c;
+                const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+                const half4_t h = *reinterpret_cast<const half4_t*>(hp) + y;  // fp16 add, one rounding
+                *reinterpret_cast<half4_t*>(hp) = h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
+            }
+            ss = wave_sum(ss);
+            if (lane == 0 && m < M) fuse.ssq_out[(size_t)m * gridDim.x + tile] = ss;
         }
         return;
     }
@@ -553,6 +619,14 @@ bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits) {
     return gemm_supported(M, N, K, group_size, bits) && use_small(M, group_size) && N % kGemmCols == 0;
 }
 
+// Residual-add epilogue and normalise-while-staging prologue: the in-kernel
+// reduction of the small-M kernel only (a second kernel could not see whole tiles
+// per wave), i.e. M <= kFusedReduceMaxM.
+bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits) {
+    return gemm_supported(M, N, K, group_size, bits) && use_small(M, group_size) && M <= kFusedReduceMaxM &&
+           N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
+}
+
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)bits;
     const GemmPlan p = plan_gemm(M, N, K, group_size);
@@ -577,18 +651,29 @@ static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, co
 template <int BITS, int MT>
 static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                               const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
-                              int N, int K, int group_size, int epilogue) {
+                              int N, int K, int group_size, int epilogue, const SmallFuse& fuse) {
     // workspace: [tile counters, zero between launches][fp32 partials]
     // in-kernel reduction by the last workgroup of a tile pays for few rows only
     unsigned* counters =
         (M <= kFusedReduceMaxM && p.col_tiles <= kMaxTileCounters) ? reinterpret_cast<unsigned*>(workspace) : nullptr;
     float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     const dim3 grid(p.col_tiles, p.split_k);
-#define MH_LAUNCH_SMALL(SPG)                                                                                  \
-    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG>), grid, dim3(256), 0, stream, (const half_t*)x,  \
-                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,  \
-                       partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k,  \
-                       epilogue)
+    const bool norm = fuse.ssq_in != nullptr;
+#define MH_LAUNCH_SMALL_N(SPG, NORM)                                                                                \
+    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG, NORM>), grid, dim3(256), 0, stream, (const half_t*)x, \
+                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,      \
+                       partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k,      \
+                       epilogue, fuse)
+#define MH_LAUNCH_SMALL(SPG)                              \
+    do {                                                  \
+        if constexpr (MT == 1) {                          \
+            if (norm) {                                   \
+                MH_LAUNCH_SMALL_N(SPG, true);             \
+                break;                                    \
+            }                                             \
+        }                                                 \
+        MH_LAUNCH_SMALL_N(SPG, false);                    \
+    } while (0)
     switch (group_size / 32) {
         case 1: MH_LAUNCH_SMALL(1); break;
         case 2: MH_LAUNCH_SMALL(2); break;
@@ -596,6 +681,7 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
         default: MH_LAUNCH_SMALL(8); break;
     }
 #undef MH_LAUNCH_SMALL
+#undef MH_LAUNCH_SMALL_N
     if (counters == nullptr && (p.split_k > 1 || epilogue != kEpilogueNone))
         launch_splitk_finalize(stream, partial, out, M, N, p.split_k, epilogue);
 }
@@ -603,14 +689,14 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
 template <int BITS>
 static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
                            const int32_t* qzeros, const void* scales, void* out, void* workspace, int M,
-                           int N, int K, int group_size, int epilogue) {
+                           int N, int K, int group_size, int epilogue, const SmallFuse& fuse) {
     if (use_small(M, group_size)) {
         if (p.mt == 1)
             launch_gemm_small<BITS, 1>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size,
-                                       epilogue);
+                                       epilogue, fuse);
         else
             launch_gemm_small<BITS, 2>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size,
-                                       epilogue);
+                                       epilogue, fuse);
         return;
     }
     switch (p.mt) {
@@ -623,8 +709,11 @@ static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x,
 
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
-                     void* workspace, size_t workspace_bytes, int epilogue) {
+                     void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
     const GemmPlan p = plan_gemm(M, N, K, group_size);
+    if ((fuse.ssq_in != nullptr || epilogue == kEpilogueResidual) && !gemm_norm_fusion_supported(M, N, K, group_size, bits))
+        return fail(MH_ERR_INVALID, "gptq gemm: RMSNorm fusion needs M <= %d, N %% 256 == 0 and a group of 32..256",
+                    kFusedReduceMaxM);
     const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
     if (epilogue != kEpilogueNone && !gemm_silu_pairs_supported(M, N, K, group_size, bits))
         return fail(MH_ERR_INVALID, "gptq gemm: the SiLU-pair epilogue needs M <= %d, N %% 256 == 0 and a group of 32..256",
@@ -637,9 +726,9 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace must be 256-byte aligned");
     }
     if (bits == 4)
-        launch_gemm_mt<4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size, epilogue);
+        launch_gemm_mt<4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size, epilogue, fuse);
     else
-        launch_gemm_mt<8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size, epilogue);
+        launch_gemm_mt<8>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size, epilogue, fuse);
     MH_CHECK_LAUNCH();
     return MH_OK;
 }
