@@ -613,20 +613,35 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
         for (int l = 0; l < c.n_layers; ++l) {
             const mh_llama_layer& L = m->layers[l];
             int rc;
-            if (fused_norm && l > 0) {  // normalise the residual stream left by the previous down projection
+            if (fused_norm) {
+                // RoPE and the cache append ride on the reduction of the q|k|v product
                 SmallFuse f;
-                f.ssq_in = s.ssq_a;
-                f.ssq_tiles = res_tiles;
-                f.norm_w = (const half_t*)L.input_norm;
-                f.eps = c.rms_eps;
-                rc = fused(s.h, L.qkv, s.qkv, qkv_n, c.hidden, kEpilogueNone, f);
+                f.rope_cos = m->cos;
+                f.rope_sin = m->sin;
+                f.positions = positions;
+                f.q_out = s.q;
+                f.k_cache = (half_t*)L.k_cache;
+                f.vt_cache = (half_t*)L.v_cache;
+                f.q_heads = c.n_q_heads;
+                f.kv_heads = c.n_kv_heads;
+                f.max_seq = c.max_seq;
+                const half_t* x = s.xn;
+                if (l > 0) {  // normalise the residual stream left by the previous down projection
+                    f.ssq_in = s.ssq_a;
+                    f.ssq_tiles = res_tiles;
+                    f.norm_w = (const half_t*)L.input_norm;
+                    f.eps = c.rms_eps;
+                    x = s.h;
+                }
+                rc = fused(x, L.qkv, s.qkv, qkv_n, c.hidden, kEpilogueRopeAppend, f);
+                if (rc) return rc;
             } else {
                 rc = linear(s.xn, L.qkv, s.qkv, qkv_n, c.hidden);
+                if (rc) return rc;
+                hipLaunchKernelGGL(rope_kv_append_kernel, dim3(c.n_q_heads + 2 * c.n_kv_heads, batch), dim3(64), 0, st,
+                                   s.qkv, m->cos, m->sin, positions, s.q, (half_t*)L.k_cache, (half_t*)L.v_cache,
+                                   c.n_q_heads, c.n_kv_heads, c.head_dim, c.max_seq);
             }
-            if (rc) return rc;
-            hipLaunchKernelGGL(rope_kv_append_kernel, dim3(c.n_q_heads + 2 * c.n_kv_heads, batch), dim3(64), 0, st,
-                               s.qkv, m->cos, m->sin, positions, s.q, (half_t*)L.k_cache, (half_t*)L.v_cache,
-                               c.n_q_heads, c.n_kv_heads, c.head_dim, c.max_seq);
             switch (g) {
                 case 1: launch_attn<1>(st, *m, s, L, positions, batch, splits); break;
                 case 2: launch_attn<2>(st, *m, s, L, positions, batch, splits); break;

@@ -130,6 +130,14 @@ __device__ __forceinline__ void pair_activations<8>(const uint32_t* x, uint32_t*
 constexpr int kEpilogueNone = 0;
 constexpr int kEpilogueSiluPairs = 1;
 constexpr int kEpilogueResidual = 2;
+// kEpilogueRopeAppend: the product is the fused q|k|v projection of one new
+// token per row, heads of 128 dims.  Query heads are rotated (interleaved pairs,
+// minit/cuda/kernel/cuda/rope.py:58-73, at positions[m]) into q_out [M, QH, 128];
+// key heads are rotated and value heads copied into the caches at that position
+// (examples/llama3_70b.py:93-100): k_cache [M, KVH, T, 128], vt_cache
+// [M, KVH, 128, T].  Values are rounded to fp16 before the rotation, as when the
+// projection is stored first.
+constexpr int kEpilogueRopeAppend = 3;
 
 // Optional fusions of the small-M product kernel around RMSNorm
 // (minit/cuda/kernel/cuda/rms_norm.py:69-89): a producer with kEpilogueResidual
@@ -141,6 +149,14 @@ struct SmallFuse {
     const half_t* norm_w = nullptr;  // [K]
     float eps = 0.f;
     float* ssq_out = nullptr;        // [M, N / 256]
+    // kEpilogueRopeAppend
+    const float* rope_cos = nullptr;  // [T, 64]
+    const float* rope_sin = nullptr;
+    const int32_t* positions = nullptr;  // [M]
+    half_t* q_out = nullptr;
+    half_t* k_cache = nullptr;
+    half_t* vt_cache = nullptr;
+    int q_heads = 0, kv_heads = 0, max_seq = 0;
 };
 
 __device__ __forceinline__ half_t silu_pair(half_t gate, half_t up) {

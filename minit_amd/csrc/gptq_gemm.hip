@@ -504,6 +504,37 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         }
         return;
     }
+    if (epilogue == kEpilogueRopeAppend) {
+        // four consecutive columns = two interleaved pairs of one head
+        for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
+            const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
+            const float4_t sum = sum_splits(partial + (size_t)m * N + c);
+            const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+            const int head = c / 128, d = c % 128;
+            const int pos = fuse.positions[m];
+            if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
+                half_t* dst = fuse.vt_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) *
+                                                  fuse.max_seq + pos;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
+                continue;
+            }
+            const float* cr = fuse.rope_cos + (size_t)pos * 64 + d / 2;
+            const float* sr = fuse.rope_sin + (size_t)pos * 64 + d / 2;
+            half4_t o;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const float re = (float)y[2 * j], im = (float)y[2 * j + 1];
+                o[2 * j] = (half_t)(re * cr[j] - im * sr[j]);
+                o[2 * j + 1] = (half_t)(im * cr[j] + re * sr[j]);
+            }
+            half_t* dst = head < fuse.q_heads
+                              ? fuse.q_out + ((size_t)m * fuse.q_heads + head) * 128 + d
+                              : fuse.k_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads)) * fuse.max_seq + pos) * 128 + d;
+            *reinterpret_cast<half4_t*>(dst) = o;
+        }
+        return;
+    }
     if (epilogue == kEpilogueResidual) {
         // a wave owns one row of the tile per pass (64 lanes x 4 columns), so the
         // row's sum of squares is one wave reduction; N is a multiple of 256
@@ -711,7 +742,8 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
     const GemmPlan p = plan_gemm(M, N, K, group_size);
-    if ((fuse.ssq_in != nullptr || epilogue == kEpilogueResidual) && !gemm_norm_fusion_supported(M, N, K, group_size, bits))
+    if ((fuse.ssq_in != nullptr || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
+        !gemm_norm_fusion_supported(M, N, K, group_size, bits))
         return fail(MH_ERR_INVALID, "gptq gemm: RMSNorm fusion needs M <= %d, N %% 256 == 0 and a group of 32..256",
                     kFusedReduceMaxM);
     const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
