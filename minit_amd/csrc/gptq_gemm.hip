@@ -475,7 +475,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 
     __shared__ int is_last;
     if (!arrive_and_check_last(&counters[tile], (unsigned)split_k, &is_last)) return;
-    constexpr int BATCH = 8;  // partial loads in flight per thread
+    constexpr int BATCH = 16;  // partial loads in flight per thread
     const size_t plane = (size_t)M * N;
     auto sum_splits = [&](const float* p) {
         float4_t s = {0.f, 0.f, 0.f, 0.f};

@@ -119,3 +119,20 @@ def test_functional_argument_checks():
         F.rms_norm(None, None, 0, 1)         # eps must be a float, as in the reference
     with pytest.raises(AssertionError):
         F.rms_norm(None, None, 0, 0.75)
+
+
+def test_interleave_gate_up_moves_whole_columns():
+    """The load-time column order of the fused gate|up projection: blocks of 128
+    gate columns followed by their 128 up columns; dequantizing after the
+    permutation equals permuting the dequantized matrix."""
+    import numpy as np
+    from minit_amd import synthetic
+    from minit_amd.decode import interleave_gate_up
+    from oracle import gptq as O
+    k, ffn, g = 256, 384, 128
+    qweight, qzeros, scales = synthetic.gptq_weights("host", "gu", k, 2 * ffn, g, 4, (0, 15))
+    w = O.dequantize_packed(qweight, qzeros, scales, None, 4, g)
+    wi = O.dequantize_packed(*interleave_gate_up(qweight, qzeros, scales), None, 4, g)
+    for t in range(ffn // 128):
+        np.testing.assert_array_equal(wi[:, t * 256:t * 256 + 128], w[:, t * 128:(t + 1) * 128])
+        np.testing.assert_array_equal(wi[:, t * 256 + 128:(t + 1) * 256], w[:, ffn + t * 128:ffn + (t + 1) * 128])
