@@ -131,6 +131,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel (1 GiB read + 1 GiB write per launch) that the "
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
+    ap.add_argument("--calibrate-mfma", action="store_true",
+                    help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the W8A8 GEMM lines (M=2048, K=4096, N in {4096, 11008}), then exit")
     args = ap.parse_args()
@@ -166,6 +168,32 @@ def main():
         us = e0.elapsed_ms(e1) * 1e3 / 5
         print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
                           "us": round(us, 1), "gbps_read_plus_write": round(2 * nbytes / us / 1e3, 1)}))
+        return
+
+    if args.calibrate_mfma:
+        # what the int8 matrix pipes sustain from registers alone, all-zero vs random operands
+        blocks, iters = 256 * 2, 40000          # two waves per SIMD
+        nbytes = blocks * 512 * 96
+        res = []
+        for label in ("zero", "random"):
+            ops_buf = HIPTensor.allocate((nbytes,), "int8")
+            if label == "zero":
+                ops_buf._memory.reset()
+            else:
+                lib.call("mh_synth_i8", None, ops_buf.data_ptr, nbytes, -127, 127, 99)
+            sink = HIPTensor.allocate((blocks * 512,), "int32")
+            lib.call("mh_i8_mfma_probe", None, ops_buf.data_ptr, sink.data_ptr, blocks, 1000)
+            memory.synchronize()
+            e0, e1 = memory.Event(), memory.Event()
+            e0.record()
+            lib.call("mh_i8_mfma_probe", None, ops_buf.data_ptr, sink.data_ptr, blocks, iters)
+            e1.record()
+            e1.synchronize()
+            ms = e0.elapsed_ms(e1)
+            tops = iters * 8 * 65536.0 * (blocks * 512 / 64) / (ms * 1e9)
+            res.append({"operands": label, "ms": round(ms, 2), "tops": round(tops, 1),
+                        "frac_of_datasheet": round(tops / INT8_PEAK_TOPS, 4)})
+        print(json.dumps({"kernel": "i8_mfma_probe_kernel", "waves_per_simd": 2, "results": res}))
         return
 
     if args.int8_only:

@@ -158,6 +158,12 @@ int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out
 int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w,
                const float* a_scale, const float* w_scale, void* out_f16,
                int32_t* acc_i32, int M, int N, int K);
+/* Calibration, no counterpart in the reference: blocks x 512 threads each run
+ * iters x 8 register-resident v_mfma_i32_32x32x32_i8 (2 * 32*32*32 operations
+ * per wave each) on operands read once from `operands` (blocks * 512 * 96 bytes);
+ * out receives blocks * 512 int32.  Used by bench.py --calibrate-mfma to find the
+ * int8 rate the matrix pipes sustain on this box for given operand values. */
+int mh_i8_mfma_probe(mh_stream_t stream, const int8_t* operands, int32_t* out, int blocks, int iters);
 /* out[n, k] = in[k, n]: one-time layout conversion for weights stored [K, N]. */
 int mh_i8_transpose(mh_stream_t stream, const int8_t* in, int8_t* out, int rows, int cols);
 

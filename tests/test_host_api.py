@@ -136,3 +136,24 @@ def test_interleave_gate_up_moves_whole_columns():
     for t in range(ffn // 128):
         np.testing.assert_array_equal(wi[:, t * 256:t * 256 + 128], w[:, t * 128:(t + 1) * 128])
         np.testing.assert_array_equal(wi[:, t * 256 + 128:(t + 1) * 256], w[:, ffn + t * 128:ffn + (t + 1) * 128])
+
+
+def test_prototypes_match_header_argument_counts():
+    """ctypes converts surplus arguments by default rules (a pointer becomes a
+    truncated int), so a prototype that is one entry short corrupts a call
+    silently: every prototype must list exactly the header's parameters."""
+    import os
+    import re
+    from minit_amd import lib
+    header = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include",
+                               "minit_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    decls = dict(re.findall(r"\b(mh_\w+)\s*\(([^;{]*?)\)\s*;", header))
+    assert decls, "no declarations parsed"
+    for name, (_, argtypes) in lib.PROTOTYPES.items():
+        assert name in decls, f"{name} is not declared in the header"
+        params = decls[name].strip()
+        n = 0 if params in ("", "void") else len([p for p in params.split(",") if p.strip()])
+        assert n == len(argtypes), f"{name}: header has {n} parameters, prototype lists {len(argtypes)}"
+    for name in decls:
+        assert name in lib.PROTOTYPES, f"{name} has no ctypes prototype"
