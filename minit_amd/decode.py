@@ -60,7 +60,8 @@ class LlamaDecoder:
 
     def __init__(self, config: dict, batch_max: int, max_seq: int):
         self.config = dict(config)
-        max_seq = (max_seq + 7) // 8 * 8   # the transposed V cache is read 8 positions (16 bytes) at a time
+        # the transposed V cache is read 8 positions (16 bytes) at a time; rows of whole 128-byte lines keep those reads inside one line
+        max_seq = (max_seq + 63) // 64 * 64
         self.batch_max, self.max_seq = batch_max, max_seq
         c = self.config
         self._cfg = LlamaConfig(c["n_layers"], c["hidden"], c["n_q_heads"], c["n_kv_heads"], c["head_dim"],
