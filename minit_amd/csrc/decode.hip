@@ -24,7 +24,8 @@ int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweig
                          const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                          void* workspace, size_t workspace_bytes);
 bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
-bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits);
+bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, int epilogue);
+int gemm_residual_ssq_pieces(int M, int N);
 int gptq_matmul_fused(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                       const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                       void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse);
@@ -591,14 +592,15 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                                     s.gptq_ws, s.gptq_ws_bytes);
     };
 
-    // With few rows the residual add and RMSNorm around the linears are folded into
-    // them: o and down add their result to the residual stream and leave per-tile
+    // The residual add and RMSNorm around the linears are folded into them where the
+    // small-M product kernel serves the shapes: o and down add their result to the residual stream and leave per-tile
     // sums of squares, qkv and gate|up normalise that stream while staging it.
-    const bool fused_norm = gemm_norm_fusion_supported(batch, c.hidden, c.n_q_heads * c.head_dim, c.group_size, c.bits) &&
-                            gemm_norm_fusion_supported(batch, c.hidden, c.ffn, c.group_size, c.bits) &&
-                            gemm_norm_fusion_supported(batch, qkv_n, c.hidden, c.group_size, c.bits) &&
-                            gemm_norm_fusion_supported(batch, 2 * c.ffn, c.hidden, c.group_size, c.bits) && fused_silu;
-    const int res_tiles = c.hidden / 256;
+    const bool fused_norm =
+        gemm_norm_fusion_supported(batch, c.hidden, c.n_q_heads * c.head_dim, c.group_size, c.bits, kEpilogueResidual) &&
+        gemm_norm_fusion_supported(batch, c.hidden, c.ffn, c.group_size, c.bits, kEpilogueResidual) &&
+        gemm_norm_fusion_supported(batch, qkv_n, c.hidden, c.group_size, c.bits, kEpilogueRopeAppend) &&
+        gemm_norm_fusion_supported(batch, 2 * c.ffn, c.hidden, c.group_size, c.bits, kEpilogueSiluPairs) && fused_silu;
+    const int res_tiles = gemm_residual_ssq_pieces(batch, c.hidden);
     auto fused = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k, int epilogue,
                      const SmallFuse& fuse) -> int {
         return gptq_matmul_fused(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
@@ -626,12 +628,10 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                 f.kv_heads = c.n_kv_heads;
                 f.max_seq = c.max_seq;
                 const half_t* x = s.xn;
-                if (l > 0) {  // normalise the residual stream left by the previous down projection
+                if (l > 0) {  // s.xn holds h * input_norm from the previous down projection
                     f.ssq_in = s.ssq_a;
                     f.ssq_tiles = res_tiles;
-                    f.norm_w = (const half_t*)L.input_norm;
                     f.eps = c.rms_eps;
-                    x = s.h;
                 }
                 rc = fused(x, L.qkv, s.qkv, qkv_n, c.hidden, kEpilogueRopeAppend, f);
                 if (rc) return rc;
@@ -649,18 +649,20 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                 default: launch_attn<8>(st, *m, s, L, positions, batch, splits); break;
             }
             if (fused_norm) {
-                SmallFuse res;
+                SmallFuse res;  // h += o; s.xn = h * post_norm
                 res.ssq_out = s.ssq_b;
+                res.next_norm_w = (const half_t*)L.post_norm;
+                res.xw_out = s.xn;
                 rc = fused(s.attn, L.o, s.h, c.hidden, c.n_q_heads * c.head_dim, kEpilogueResidual, res);
                 if (rc) return rc;
                 SmallFuse f;
                 f.ssq_in = s.ssq_b;
                 f.ssq_tiles = res_tiles;
-                f.norm_w = (const half_t*)L.post_norm;
                 f.eps = c.rms_eps;
-                rc = fused(s.h, L.gate_up, s.act, 2 * c.ffn, c.hidden, kEpilogueSiluPairs, f);
+                rc = fused(s.xn, L.gate_up, s.act, 2 * c.ffn, c.hidden, kEpilogueSiluPairs, f);
                 if (rc) return rc;
-                res.ssq_out = s.ssq_a;
+                res.ssq_out = s.ssq_a;  // h += down; s.xn = h * the next layer's input_norm
+                res.next_norm_w = (const half_t*)(l + 1 < c.n_layers ? m->layers[l + 1].input_norm : m->final_norm);
                 rc = fused(s.act, L.down, s.h, c.hidden, c.ffn, kEpilogueResidual, res);
                 if (rc) return rc;
                 continue;

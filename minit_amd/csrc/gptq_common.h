@@ -140,15 +140,20 @@ constexpr int kEpilogueResidual = 2;
 constexpr int kEpilogueRopeAppend = 3;
 
 // Optional fusions of the small-M product kernel around RMSNorm
-// (minit/cuda/kernel/cuda/rms_norm.py:69-89): a producer with kEpilogueResidual
-// fills ssq_out; a consumer given ssq_in / norm_w normalises its activations while
-// staging them.
+// (minit/cuda/kernel/cuda/rms_norm.py:69-89), which is split in two:
+//   norm(h)[k] = (h[k] * w[k]) * (1 / sqrt(sum h^2 / K + eps)).
+// A producer with kEpilogueResidual writes the new residual stream h, the
+// element-wise half xw = fp16(h * next_norm_w) and per-piece sums of squares; a
+// consumer given ssq_in takes xw as its activations and multiplies its fp32
+// accumulators by the row factor at the end.  Against normalise-then-round the one
+// fp16 rounding per activation moves from after both factors to after the first.
 struct SmallFuse {
-    const float* ssq_in = nullptr;   // [M, ssq_tiles]
+    const float* ssq_in = nullptr;   // [M, ssq_tiles]: consumer
     int ssq_tiles = 0;
-    const half_t* norm_w = nullptr;  // [K]
     float eps = 0.f;
-    float* ssq_out = nullptr;        // [M, N / 256]
+    float* ssq_out = nullptr;             // [M, pieces]: kEpilogueResidual
+    const half_t* next_norm_w = nullptr;  // [N]
+    half_t* xw_out = nullptr;             // [M, N]
     // kEpilogueRopeAppend
     const float* rope_cos = nullptr;  // [T, 64]
     const float* rope_sin = nullptr;

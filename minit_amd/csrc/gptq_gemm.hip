@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_kernel(
 }
 
 void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
-                            int epilogue);
+                            int epilogue, const SmallFuse& fuse);
 
 // ---- small-M variant (M <= 32: decode batches) --------------------------------------------------
 // Same operand mapping, a schedule built around two facts measured on this part:
@@ -237,13 +237,11 @@ void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out,
 // weights per wave in flight at all times.
 constexpr int kSmallDepth = 8;  // steps per stage = ring depth
 
-// NORM: the product is taken of the RMS-normalised activations without a pass
-// over the row: while staging, x'[m, k] = fp16(x[m, k] * norm_w[k]) (one packed
-// fp16 multiply per two elements); the row factor 1 / sqrt(ssq[m] / K + eps), with
-// ssq[m] the sum of the fuse.ssq_tiles per-tile sums of squares that the producer
-// of x left behind (kEpilogueResidual), scales the fp32 accumulators at the end.
-// Against normalise-then-round the one fp16 rounding per activation moves from
-// after both factors to after the first.
+// NORM: x is the element-wise half of an RMSNorm, fp16(h * norm_w), written by the
+// producer of h (kEpilogueResidual); the row factor 1 / sqrt(ssq[m] / K + eps), with
+// ssq[m] the sum of the fuse.ssq_tiles partial sums of squares the producer left
+// behind, scales the fp32 accumulators at the end, so the row never needs a pass
+// of its own.
 template <int BITS, int MT, int SPG, bool NORM>
 __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
@@ -286,8 +284,13 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     uint32_t lane_off[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) lane_off[j] = (uint32_t)((kq * LOADS + j) * N + colc) * 4u;
+    // The ring is refilled at a fixed place of the loop body, also in the block's
+    // last stage, where there is nothing left to fetch: those loads re-read the
+    // block's own last step (a cache hit) instead of running on into the K range of
+    // the next split, which would cost the CU a stage's worth of memory requests.
+    const int ring_last = min(step_begin + stages_per_block * D - 1, last_step);
     auto load_q = [&](int step, uint4_t* dst) {
-        const int s = min(step, last_step);
+        const int s = min(step, last_step);  // a block's last stage runs on into the next split's range
         const char* base = reinterpret_cast<const char*>(qweight) + (size_t)s * ROWS_PER_STEP * N * 4;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j)
@@ -298,7 +301,6 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 
     // ---- staging of activations and constants: global -> registers -> LDS
     uint4 xr[XL];
-    uint4 wr[NORM ? XL : 1];  // norm weights of the same k
     uint4 sr;       // eight scales of one group
     uint32_t zr[8 / P];
     int x_row[XL], x_chunk[XL];
@@ -315,11 +317,6 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 #pragma unroll
         for (int u = 0; u < XL; ++u)
             xr[u] = *reinterpret_cast<const uint4*>(x + (size_t)x_row[u] * K + (size_t)sclamp * 32 + x_chunk[u] * 8);
-        if constexpr (NORM) {
-#pragma unroll
-            for (int u = 0; u < XL; ++u)
-                wr[u] = *reinterpret_cast<const uint4*>(fuse.norm_w + (size_t)sclamp * 32 + x_chunk[u] * 8);
-        }
         const int g = min(sclamp / SPG + c_group, g_last);
         sr = *reinterpret_cast<const uint4*>(scales + (size_t)g * N + c_colg);
 #pragma unroll
@@ -328,12 +325,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     auto store_stage = [&](int buf, int stage_step) {
 #pragma unroll
         for (int u = 0; u < XL; ++u) {
-            uint32_t in[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
-            if constexpr (NORM) {  // x * w in fp16; the row's 1 / rms scales the accumulators at the end
-                const uint32_t wv[4] = {wr[u].x, wr[u].y, wr[u].z, wr[u].w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) in[e] = as_u32(as_half2(in[e]) * as_half2(wv[e]));
-            }
+            const uint32_t in[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
             uint32_t o[4];
             if constexpr (BITS == 4) {
                 pair_activations<4>(in, o);
@@ -365,7 +357,6 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         // lanes per row read the tiles in parallel (the loads travel with those of
         // the first stage) and are folded by shuffles, a fixed order; read back
         // after the K loop
-        static_assert(BM * 32 <= 512, "two passes of the 256 threads cover every row");
 #pragma unroll
         for (int pass = 0; pass < (BM * 32 + 255) / 256; ++pass) {
             const int row = pass * 8 + (tid >> 5), t0 = tid & 31;
@@ -547,6 +538,9 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
                 const half4_t h = *reinterpret_cast<const half4_t*>(hp) + y;  // fp16 add, one rounding
                 *reinterpret_cast<half4_t*>(hp) = h;
+                if (fuse.xw_out)
+                    *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) =
+                        h * *reinterpret_cast<const half4_t*>(fuse.next_norm_w + c);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
             }
@@ -650,13 +644,18 @@ bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits) {
     return gemm_supported(M, N, K, group_size, bits) && use_small(M, group_size) && N % kGemmCols == 0;
 }
 
-// Residual-add epilogue and normalise-while-staging prologue: the in-kernel
-// reduction of the small-M kernel only (a second kernel could not see whole tiles
-// per wave), i.e. M <= kFusedReduceMaxM.
-bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits) {
-    return gemm_supported(M, N, K, group_size, bits) && use_small(M, group_size) && M <= kFusedReduceMaxM &&
-           N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
+// Residual-add / RoPE epilogues and the normalise-while-staging prologue: the
+// small-M kernel.  Up to kFusedReduceMaxM rows the epilogue runs in the kernel's own
+// reduction (sums of squares per 256-column tile); above, in the second stage
+// (per 1024 columns, so N must be a multiple of that).
+bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
+    if (!gemm_supported(M, N, K, group_size, bits) || !use_small(M, group_size)) return false;
+    if (M <= kFusedReduceMaxM) return N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
+    return N % (epilogue == kEpilogueResidual ? 1024 : kGemmCols) == 0;
 }
+
+// Per-row pieces a kEpilogueResidual producer leaves in ssq_out for this shape.
+int gemm_residual_ssq_pieces(int M, int N) { return M <= kFusedReduceMaxM ? N / kGemmCols : N / 1024; }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)bits;
@@ -676,7 +675,7 @@ static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, co
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size / 32,
                        p.steps_total, p.steps_per_block, p.split_k);
-    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone);
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, SmallFuse{});
 }
 
 template <int BITS, int MT>
@@ -695,15 +694,12 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
                        (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,      \
                        partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k,      \
                        epilogue, fuse)
-#define MH_LAUNCH_SMALL(SPG)                              \
-    do {                                                  \
-        if constexpr (MT == 1) {                          \
-            if (norm) {                                   \
-                MH_LAUNCH_SMALL_N(SPG, true);             \
-                break;                                    \
-            }                                             \
-        }                                                 \
-        MH_LAUNCH_SMALL_N(SPG, false);                    \
+#define MH_LAUNCH_SMALL(SPG)                 \
+    do {                                     \
+        if (norm)                            \
+            MH_LAUNCH_SMALL_N(SPG, true);    \
+        else                                 \
+            MH_LAUNCH_SMALL_N(SPG, false);   \
     } while (0)
     switch (group_size / 32) {
         case 1: MH_LAUNCH_SMALL(1); break;
@@ -714,7 +710,7 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
 #undef MH_LAUNCH_SMALL
 #undef MH_LAUNCH_SMALL_N
     if (counters == nullptr && (p.split_k > 1 || epilogue != kEpilogueNone))
-        launch_splitk_finalize(stream, partial, out, M, N, p.split_k, epilogue);
+        launch_splitk_finalize(stream, partial, out, M, N, p.split_k, epilogue, fuse);
 }
 
 template <int BITS>
@@ -743,9 +739,9 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
     const GemmPlan p = plan_gemm(M, N, K, group_size);
     if ((fuse.ssq_in != nullptr || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
-        !gemm_norm_fusion_supported(M, N, K, group_size, bits))
-        return fail(MH_ERR_INVALID, "gptq gemm: RMSNorm fusion needs M <= %d, N %% 256 == 0 and a group of 32..256",
-                    kFusedReduceMaxM);
+        !gemm_norm_fusion_supported(M, N, K, group_size, bits, epilogue))
+        return fail(MH_ERR_INVALID, "gptq gemm: RMSNorm / RoPE fusion needs M <= %d, a group of 32..256 and N %% 256 == 0 "
+                    "(N %% 1024 == 0 above %d rows)", kSmallMaxM, kFusedReduceMaxM);
     const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
     if (epilogue != kEpilogueNone && !gemm_silu_pairs_supported(M, N, K, group_size, bits))
         return fail(MH_ERR_INVALID, "gptq gemm: the SiLU-pair epilogue needs M <= %d, N %% 256 == 0 and a group of 32..256",

@@ -195,8 +195,76 @@ __global__ __launch_bounds__(256) void splitk_finalize_silu_kernel(const float* 
     *reinterpret_cast<half4_t*>(out + o) = h;
 }
 
+// kEpilogueResidual in the second stage: a workgroup covers 1024 consecutive
+// columns of one row (N is a multiple of 1024), adds into the residual stream
+// and leaves that piece's sum of squares in ssq_out[m, N / 1024].
+__global__ __launch_bounds__(256) void splitk_finalize_residual_kernel(const float* __restrict__ partial, half_t* h,
+                                                                       SmallFuse fuse, int M, int N, int split_k) {
+    __shared__ float smem[16];
+    const size_t mn = (size_t)M * N;
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;  // within one row: N % 1024 == 0
+    float4_t s = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < split_k; ++sp) s += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
+    const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+    const half4_t r = *reinterpret_cast<const half4_t*>(h + i) + y;  // fp16 add, one rounding
+    *reinterpret_cast<half4_t*>(h + i) = r;
+    if (fuse.xw_out)
+        *reinterpret_cast<half4_t*>(fuse.xw_out + i) = r * *reinterpret_cast<const half4_t*>(fuse.next_norm_w + i % N);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += (float)r[e] * (float)r[e];
+    ss = block_sum(ss, smem);
+    if (threadIdx.x == 0) fuse.ssq_out[blockIdx.x] = ss;  // blocks are numbered row-major over [M, N / 1024]
+}
+
+// kEpilogueRopeAppend in the second stage: four consecutive columns = two
+// interleaved pairs of one head.
+__global__ __launch_bounds__(256) void splitk_finalize_rope_kernel(const float* __restrict__ partial, SmallFuse fuse,
+                                                                   int M, int N, int split_k) {
+    const size_t mn = (size_t)M * N;
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= mn) return;
+    float4_t sum = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < split_k; ++sp) sum += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
+    const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+    const int m = (int)(i / N), c = (int)(i % N);
+    const int head = c / 128, d = c % 128;
+    const int pos = fuse.positions[m];
+    if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
+        half_t* dst = fuse.vt_cache +
+                      (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
+        return;
+    }
+    const float* cr = fuse.rope_cos + (size_t)pos * 64 + d / 2;
+    const float* sr = fuse.rope_sin + (size_t)pos * 64 + d / 2;
+    half4_t o;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const float re = (float)y[2 * j], im = (float)y[2 * j + 1];
+        o[2 * j] = (half_t)(re * cr[j] - im * sr[j]);
+        o[2 * j + 1] = (half_t)(im * cr[j] + re * sr[j]);
+    }
+    half_t* dst = head < fuse.q_heads
+                      ? fuse.q_out + ((size_t)m * fuse.q_heads + head) * 128 + d
+                      : fuse.k_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads)) * fuse.max_seq + pos) * 128 + d;
+    *reinterpret_cast<half4_t*>(dst) = o;
+}
+
 void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
-                            int epilogue) {
+                            int epilogue, const SmallFuse& fuse) {
+    if (epilogue == kEpilogueResidual) {
+        hipLaunchKernelGGL(splitk_finalize_residual_kernel, dim3((unsigned)((size_t)M * N / 1024)), dim3(256), 0, stream,
+                           partial, (half_t*)out, fuse, M, N, split_k);
+        return;
+    }
+    if (epilogue == kEpilogueRopeAppend) {
+        const size_t threads = ((size_t)M * N + 3) / 4;
+        hipLaunchKernelGGL(splitk_finalize_rope_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                           partial, fuse, M, N, split_k);
+        return;
+    }
     if (epilogue == kEpilogueSiluPairs) {
         const size_t threads = ((size_t)M * (N / 2) + 3) / 4;
         hipLaunchKernelGGL(splitk_finalize_silu_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
@@ -267,7 +335,7 @@ static void launch_gemv(hipStream_t stream, const GemvPlan& p, const void* x, co
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,
                        (const half_t*)scales, (half_t*)out, partial, N, K, group_size / P,
                        p.steps_total, p.steps_per_wave, p.split_k);
-    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone);
+    if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, SmallFuse{});
 }
 
 template <int BITS, int M>

@@ -86,6 +86,30 @@ def test_greedy_decode_matches_oracle(hip, batch, context):
     np.testing.assert_array_equal(kc[:, :, :context], k_cache[0][:, :, :context])
 
 
+def test_decode_second_stage_fusions(hip):
+    """Nine rows and a hidden size of 1024: residual add, norm, RoPE and SiLU*up ride
+    on the second stage of split-K instead of the in-kernel reduction."""
+    from minit_amd.decode import LlamaDecoder
+    cfg = dict(CFG, n_layers=2, hidden=1024, ffn=256)
+    batch, context, max_seq = 9, 10, 64
+    model = _host_model(cfg, seed=11)
+    rng = np.random.default_rng(12)
+    shape = (batch, cfg["n_kv_heads"], max_seq, 128)
+    k_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    v_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    for c in k_cache + v_cache:
+        c[:, :, :context] = rng.normal(0, 1, (batch, cfg["n_kv_heads"], context, 128))
+    tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
+    positions = np.full(batch, context, np.int32)
+    dec = LlamaDecoder(cfg, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+    _, got = dec.decode(tokens, positions, 1, want_logits=True)
+    ref = OD.decode_step(model, tokens, positions, [c.copy() for c in k_cache], [c.copy() for c in v_cache])
+    g, r = got.astype(np.float64), ref.astype(np.float64)
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+    assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
+
+
 def test_attention_split_kv_consistency(hip):
     """A longer context forces several KV splits; one step must still match."""
     from minit_amd.decode import LlamaDecoder
