@@ -134,7 +134,10 @@ def test_gemm_matches_oracle(hip, m):
     assert_fp16_close(got, ref, what=f"gemm M={m}")
 
 
-@pytest.mark.parametrize("m,k,n,group_size,bits", [(8, 1536, 512, 64, 8), (33, 4096, 256, 32, 4)])
+@pytest.mark.parametrize("m,k,n,group_size,bits", [
+    (8, 1536, 512, 64, 8), (33, 4096, 256, 32, 4),
+    # group sizes the small-M kernel does not serve go to the staged MFMA kernel
+    (5, 1024, 264, 512, 4), (40, 1536, 256, 96, 4), (130, 1024, 520, 512, 4)])
 def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     from minit_amd import synthetic
     qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=8)
