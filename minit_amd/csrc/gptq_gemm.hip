@@ -291,18 +291,35 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const int ring_last = min(step_begin + stages_per_block * D - 1, last_step);
     auto load_q = [&](int step, uint4_t* dst) {
         const int s = min(step, last_step);  // a block's last stage runs on into the next split's range
-        const char* base = reinterpret_cast<const char*>(qweight) + (size_t)s * ROWS_PER_STEP * N * 4;
+        // the step's base address stays in scalar registers (opaque to the compiler,
+        // which otherwise folds it into a 64-bit vector multiply-add per load); the
+        // load then takes it as its scalar base next to the lane's fixed 32-bit offset
+        const uint64_t b = reinterpret_cast<uint64_t>(qweight) + (uint64_t)s * ROWS_PER_STEP * N * 4;
+        uint32_t b_lo = (uint32_t)b, b_hi = (uint32_t)(b >> 32);
+        asm("" : "+s"(b_lo), "+s"(b_hi));
+        typedef const char __attribute__((address_space(1))) * global_bytes;
+        typedef const uint4_t __attribute__((address_space(1))) * global_words;
+        const global_bytes base = (global_bytes)(((uint64_t)b_hi << 32) | b_lo);
 #pragma unroll
-        for (int j = 0; j < LOADS; ++j)
-            dst[j] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(base + lane_off[j]));
+        for (int j = 0; j < LOADS; ++j) {
+            uint32_t off = lane_off[j];
+            asm("" : "+v"(off));  // keeps the zero-extension next to the load
+            dst[j] = __builtin_nontemporal_load((global_words)(base + off));
+        }
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) load_q(step_begin + d, qb[d]);
 
     // ---- staging of activations and constants: global -> registers -> LDS
     uint4 xr[XL];
-    uint4 sr;       // eight scales of one group
-    uint32_t zr[8 / P];
+    // Constants of a stage: GPS groups x 256 columns, CE adjacent columns of one
+    // group per thread, so that every wave runs the same (short) instruction
+    // sequence -- a wave pays for an instruction whatever the number of live lanes.
+    constexpr int CE = GPS;                    // 1, 2, 4 or 8
+    constexpr int CT = kGemmCols / CE;         // threads per group
+    constexpr int ZW = CE > P ? CE / P : 1;    // packed zero words per thread
+    uint32_t sr[(CE + 1) / 2];                 // CE scales
+    uint32_t zr[ZW];
     int x_row[XL], x_chunk[XL];
 #pragma unroll
     for (int u = 0; u < XL; ++u) {
@@ -310,17 +327,25 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         x_row[u] = min(idx / XCH, M - 1);  // rows >= M only feed accumulator rows that are never stored
         x_chunk[u] = idx % XCH;
     }
-    const int c_group = (tid >> 5) % GPS, c_col8 = tid & 31;  // threads 0 .. 32*GPS-1 stage the constants
-    const int c_colg = min(tile * kGemmCols + c_col8 * 8, N - 8);
+    const int c_group = tid / CT, c_col0 = tid % CT * CE;
+    const int c_colg = min(tile * kGemmCols + c_col0, N - CE);  // N is a multiple of 8: stays aligned to CE
     auto fetch_stage = [&](int stage_step) {
         const int sclamp = min(stage_step, (last_step / D) * D);  // never read past K
 #pragma unroll
         for (int u = 0; u < XL; ++u)
             xr[u] = *reinterpret_cast<const uint4*>(x + (size_t)x_row[u] * K + (size_t)sclamp * 32 + x_chunk[u] * 8);
         const int g = min(sclamp / SPG + c_group, g_last);
-        sr = *reinterpret_cast<const uint4*>(scales + (size_t)g * N + c_colg);
+        const half_t* sp = scales + (size_t)g * N + c_colg;
+        if constexpr (CE == 1) {
+            sr[0] = *reinterpret_cast<const uint16_t*>(sp);
+        } else {
+            struct alignas(CE * 2) ScaleWords { uint32_t w[CE / 2]; };
+            const ScaleWords v = *reinterpret_cast<const ScaleWords*>(sp);
 #pragma unroll
-        for (int j = 0; j < 8 / P; ++j) zr[j] = qzeros[(size_t)g * (N / P) + c_colg / P + j];
+            for (int j = 0; j < CE / 2; ++j) sr[j] = v.w[j];
+        }
+#pragma unroll
+        for (int j = 0; j < ZW; ++j) zr[j] = qzeros[(size_t)g * (N / P) + c_colg / P + j];
     };
     auto store_stage = [&](int buf, int stage_step) {
 #pragma unroll
@@ -338,15 +363,26 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             xs[buf][(u * 256 + tid) / XCH * RS + x_chunk[u]] =
                 live ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
         }
-        if (tid < 32 * GPS) {
-            const half_t* sh = reinterpret_cast<const half_t*>(&sr);
+        {
+            const int zsub = CE >= P ? 0 : c_colg % P;  // first sub-word of this thread in zr[0]
+            uint32_t k_scale[CE], k_lo[CE], k_hi[CE];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t z = (zr[j / P] >> ((j % P) * BITS)) & MASK;
-                const ColumnConst k = make_column_const(sh[j], z);
-                cs[buf][c_group][0][c_col8 * 8 + j] = as_u32(k.scale);
-                cs[buf][c_group][1][c_col8 * 8 + j] = as_u32(k.zero_lo);
-                cs[buf][c_group][2][c_col8 * 8 + j] = as_u32(k.zero_hi);
+            for (int j = 0; j < CE; ++j) {
+                const uint32_t z = (zr[j / P] >> ((zsub + j % P) * BITS)) & MASK;
+                const uint16_t sbits = (uint16_t)(sr[j / 2] >> (j % 2 * 16));
+                const ColumnConst k = make_column_const(__builtin_bit_cast(half_t, sbits), z);
+                k_scale[j] = as_u32(k.scale);
+                k_lo[j] = as_u32(k.zero_lo);
+                k_hi[j] = as_u32(k.zero_hi);
+            }
+            struct alignas(CE * 4) ConstWords { uint32_t w[CE]; };
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const uint32_t* src = r == 0 ? k_scale : r == 1 ? k_lo : k_hi;
+                ConstWords v;
+#pragma unroll
+                for (int j = 0; j < CE; ++j) v.w[j] = src[j];
+                *reinterpret_cast<ConstWords*>(&cs[buf][c_group][r][c_col0]) = v;
             }
         }
     };
