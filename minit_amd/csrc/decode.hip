@@ -25,7 +25,7 @@ int gptq_matmul_dispatch(hipStream_t stream, const void* x, const int32_t* qweig
                          void* workspace, size_t workspace_bytes);
 bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
 bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, int epilogue);
-int gemm_residual_ssq_pieces(int M, int N);
+int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits);
 int gptq_matmul_fused(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                       const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                       void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse);
@@ -444,7 +444,7 @@ struct Llama {
 struct Scratch {
     half_t *h, *xn, *qkv, *q, *attn, *delta, *gu, *act, *logits;
     float* attn_partial;
-    float *ssq_a, *ssq_b;  // per-tile sums of squares of the residual stream, [batch, hidden / 256]
+    float *ssq_a, *ssq_b;  // per-piece sums of squares of the residual stream, [batch, at most hidden / 32]
     unsigned* attn_counters;
     void* gptq_ws;
     size_t gptq_ws_bytes;
@@ -494,8 +494,8 @@ static Scratch carve(const Llama& m, int batch, char* base) {
     s.act = (half_t*)take((size_t)batch * c.ffn * 2);
     s.logits = (half_t*)take((size_t)batch * c.vocab * 2);
     s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 4) * 4);
-    s.ssq_a = (float*)take((size_t)batch * ((c.hidden + 255) / 256) * 4);
-    s.ssq_b = (float*)take((size_t)batch * ((c.hidden + 255) / 256) * 4);
+    s.ssq_a = (float*)take((size_t)batch * ((c.hidden + 31) / 32) * 4);
+    s.ssq_b = (float*)take((size_t)batch * ((c.hidden + 31) / 32) * 4);
     s.total = off;
     return s;
 }
@@ -600,7 +600,9 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
         gemm_norm_fusion_supported(batch, c.hidden, c.ffn, c.group_size, c.bits, kEpilogueResidual) &&
         gemm_norm_fusion_supported(batch, qkv_n, c.hidden, c.group_size, c.bits, kEpilogueRopeAppend) &&
         gemm_norm_fusion_supported(batch, 2 * c.ffn, c.hidden, c.group_size, c.bits, kEpilogueSiluPairs) && fused_silu;
-    const int res_tiles = gemm_residual_ssq_pieces(batch, c.hidden);
+    // pieces the o and the down projection leave per row (they may run on different kernels)
+    const int o_pieces = gemm_residual_ssq_pieces(batch, c.hidden, c.n_q_heads * c.head_dim, c.group_size, c.bits);
+    const int down_pieces = gemm_residual_ssq_pieces(batch, c.hidden, c.ffn, c.group_size, c.bits);
     auto fused = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k, int epilogue,
                      const SmallFuse& fuse) -> int {
         return gptq_matmul_fused(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
@@ -630,7 +632,7 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                 const half_t* x = s.xn;
                 if (l > 0) {  // s.xn holds h * input_norm from the previous down projection
                     f.ssq_in = s.ssq_a;
-                    f.ssq_tiles = res_tiles;
+                    f.ssq_tiles = down_pieces;
                     f.eps = c.rms_eps;
                 }
                 rc = fused(x, L.qkv, s.qkv, qkv_n, c.hidden, kEpilogueRopeAppend, f);
@@ -657,7 +659,7 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                 if (rc) return rc;
                 SmallFuse f;
                 f.ssq_in = s.ssq_b;
-                f.ssq_tiles = res_tiles;
+                f.ssq_tiles = o_pieces;
                 f.eps = c.rms_eps;
                 rc = fused(s.xn, L.gate_up, s.act, 2 * c.ffn, c.hidden, kEpilogueSiluPairs, f);
                 if (rc) return rc;

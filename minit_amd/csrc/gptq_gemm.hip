@@ -594,6 +594,12 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     }
 }
 
+// gptq_gemm_cols.hip
+bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epilogue);
+int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                          const void* scales, void* out, int M, int N, int K, int group_size, int bits, int epilogue,
+                          const SmallFuse& fuse);
+
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
     int col_tiles;
@@ -686,12 +692,16 @@ bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits) {
 // (per 1024 columns, so N must be a multiple of that).
 bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
     if (!gemm_supported(M, N, K, group_size, bits) || !use_small(M, group_size)) return false;
+    if (epilogue == kEpilogueResidual && gemm_cols_preferred(M, N, K, group_size, bits, epilogue)) return true;
     if (M <= kFusedReduceMaxM) return N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
     return N % (epilogue == kEpilogueResidual ? 1024 : kGemmCols) == 0;
 }
 
 // Per-row pieces a kEpilogueResidual producer leaves in ssq_out for this shape.
-int gemm_residual_ssq_pieces(int M, int N) { return M <= kFusedReduceMaxM ? N / kGemmCols : N / 1024; }
+int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
+    if (gemm_cols_preferred(M, N, K, group_size, bits, kEpilogueResidual)) return N / 32;
+    return M <= kFusedReduceMaxM ? N / kGemmCols : N / 1024;
+}
 
 static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_small(kSmallMaxM, group_size); }
 
@@ -776,6 +786,9 @@ static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x,
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
+    // a narrow output goes to the kernel whose workgroups own their columns over all of K
+    if (fuse.ssq_in == nullptr && gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
+        return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse);
     if (row_blocked(M, group_size)) {
         // Above kSmallMaxM rows the product is taken 32 rows at a time by the small-M
         // kernel: the packed weights are re-read per block of rows (from the

@@ -1,0 +1,277 @@
+// GPTQ w4a16 / w8a16 product for a few rows where the output is narrow: one
+// workgroup owns 32 output columns over all of K.
+//
+// The small-M kernel (gptq_gemm.hip) cuts a narrow output into 256-column tiles
+// and needs 11-16 K splits per tile to fill the GPU; the partial sums then cross
+// workgroups (agent-scope stores, an arrival counter, a reload by the last
+// workgroup), three dependent memory round trips of about a microsecond each at
+// the end of a 10 us kernel.  Here K is split over the eight waves of the one
+// workgroup that owns the columns and the partial sums meet in LDS.
+//
+// A wave walks its own contiguous K range, so it shares nothing with the other
+// waves until the end and the K loop has no barrier.  Per step of 32 k a lane
+// (column pair nl = lane % 16, k chunk kq = lane / 16) loads 8 bytes: the packed
+// words of its two columns, which are the B operands of two
+// v_mfma_f32_16x16x32_f16.  Everything a step needs is requested 16 steps ahead
+// and in the order of use (activations of a 256-k stage, scale/zero words of a
+// group, packed weights), so each s_waitcnt vmcnt(n) leaves the 16 steps behind it
+// in flight: 8 KiB per wave, 64 KiB per CU.  More in flight measured slower (a
+// 16-byte-per-lane variant with 128 KiB per CU lost 25 %), and beyond about 34
+// loads in flight per wave the compiler's vmcnt bookkeeping falls back to
+// draining the queue at the top of the loop.  Activations go through a
+// wave-private LDS area (re-ordered to the pair order of dequant_word on the way);
+// LDS instructions of one wave execute in order, so the area needs neither a
+// second buffer nor a barrier.
+//
+// Measured against the small-M kernel (M = 1, us): 8192x8192 12.2 / 15.3,
+// 4096x4096 7.4 / 9.1, 16384x8192 18.1 / 22.3; with more 32-column tiles than CUs
+// (10240 columns: 19.0 / 15.2) or half the CUs idle on a long K (14336x4096:
+// 16.6 / 14.8) it loses, see gemm_cols_preferred.
+#include "gptq_common.h"
+
+namespace mh {
+
+#pragma clang fp contract(off)
+
+constexpr int kColsTile = 32;   // columns per workgroup
+constexpr int kColsWaves = 8;   // K ranges per workgroup
+constexpr int kColsStage = 8;   // steps per activation stage
+constexpr int kColsRing = 16;   // steps in flight per wave
+
+// (s, s), (1024 + z + 1) twice, (64 + z + 1) twice from the bits of s and the
+// zero point: below 2048 an fp16 integer n + 1024 is the bit pattern 0x6400 + n,
+// and 64 + n (n < 64) is 0x5400 + 16 n, so each pair is one multiply-add.
+__device__ __forceinline__ ColumnConst column_const_from_bits(uint32_t sbits, uint32_t z) {
+    ColumnConst c;
+    c.scale = as_half2(sbits * 0x00010001u);
+    c.zero_lo = as_half2((z + 1u) * 0x00010001u + 0x64006400u);
+    c.zero_hi = as_half2((z + 1u) * 0x00100010u + 0x54005400u);
+    return c;
+}
+
+template <int BITS, int SPG, int MROWS>
+__global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
+    const half_t* __restrict__ scales, half_t* out, int M, int N, int K, int steps_total, int steps_per_wave,
+    int epilogue, SmallFuse fuse) {
+    constexpr int P = Packing<BITS>::kPerWord;
+    constexpr int PAIRS = Packing<BITS>::kPairs;
+    constexpr uint32_t MASK = Packing<BITS>::kMask;
+    constexpr int R = kColsRing;
+    constexpr int ROWS_PER_STEP = 32 / P;
+    constexpr int LOADS = ROWS_PER_STEP / 4;
+    constexpr int CS = R / SPG;                          // scale/zero slots
+    constexpr int XS = R / kColsStage;                   // activation stage slots
+    constexpr int XP = MROWS * 32 > 64 ? MROWS * 32 / 64 : 1;  // 16-byte chunks per lane and stage
+    constexpr int RS = 33;                               // padded row stride of the staging area
+    static_assert(R % kColsStage == 0 && R % SPG == 0, "slots must divide the ring");
+
+    __shared__ uint4 xs[kColsWaves][MROWS * RS];
+    __shared__ float red[kColsWaves][MROWS][kColsTile];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nl = lane & 15, kq = lane >> 4;
+    const int tile = blockIdx.x;
+    const int col0 = tile * kColsTile + nl * 2;
+
+    const int begin = wave * steps_per_wave;
+    const int end = min(begin + steps_per_wave, steps_total);
+    const int last_step = steps_total - 1;
+    const int last_stage_step = (last_step / kColsStage) * kColsStage;
+
+    typedef const char __attribute__((address_space(1))) * global_bytes;
+
+    // ---- packed weights
+    uint2_t qb[R][LOADS];
+    uint32_t lane_off[LOADS];
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) lane_off[j] = (uint32_t)((kq * LOADS + j) * N + col0) * 4u;
+    auto load_q = [&](int step, uint2_t* dst) {
+        const int s = min(step, last_step);  // past the end of K: re-read the last step, its activations are zero
+        const uint64_t b = reinterpret_cast<uint64_t>(qweight) + (uint64_t)s * ROWS_PER_STEP * N * 4;
+        uint32_t b_lo = (uint32_t)b, b_hi = (uint32_t)(b >> 32);
+        asm("" : "+s"(b_lo), "+s"(b_hi));  // scalar base + 32-bit lane offset: no vector address arithmetic
+        const global_bytes base = (global_bytes)(((uint64_t)b_hi << 32) | b_lo);
+        typedef const uint2_t __attribute__((address_space(1))) * global_words;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) {
+            uint32_t off = lane_off[j];
+            asm("" : "+v"(off));
+            dst[j] = __builtin_nontemporal_load((global_words)(base + off));
+        }
+    };
+
+    // ---- scales and zero points of a group: one word each for the lane's two columns
+    uint32_t cs_scale[CS], cs_zero[CS];
+    const int zsub = col0 % P;
+    auto load_c = [&](int step, int slot) {
+        const int g = min(step, last_step) / SPG;
+        cs_scale[slot] = *reinterpret_cast<const uint32_t*>(scales + (size_t)g * N + col0);
+        cs_zero[slot] = qzeros[(size_t)g * (N / P) + col0 / P];
+    };
+
+    // ---- activations of a stage: lane -> (row, 16-byte chunk) of its wave's stage
+    uint4 xr[XS][XP];
+    int x_row[XP], x_chunk[XP];
+#pragma unroll
+    for (int u = 0; u < XP; ++u) {
+        const int item = u * 64 + lane;
+        x_row[u] = min(item / 32, M - 1);
+        x_chunk[u] = item % 32;
+    }
+    auto load_x = [&](int step, int slot) {
+        const int s = min(step, last_stage_step);
+#pragma unroll
+        for (int u = 0; u < XP; ++u)
+            xr[slot][u] = *reinterpret_cast<const uint4*>(x + (size_t)x_row[u] * K + (size_t)s * 32 + x_chunk[u] * 8);
+    };
+    auto store_x = [&](int step, int slot) {
+#pragma unroll
+        for (int u = 0; u < XP; ++u) {
+            const uint32_t in[4] = {xr[slot][u].x, xr[slot][u].y, xr[slot][u].z, xr[slot][u].w};
+            uint32_t o[4];
+            if constexpr (BITS == 4) {
+                pair_activations<4>(in, o);
+            } else {
+                pair_activations<8>(in, o);
+                pair_activations<8>(in + 2, o + 2);
+            }
+            const bool live = step + x_chunk[u] / 4 < end;  // steps of another wave or past K add nothing
+            if (u * 64 + lane < MROWS * 32)
+                xs[wave][(u * 64 + lane) / 32 * RS + x_chunk[u]] =
+                    live ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    // requests in the order of use
+#pragma unroll
+    for (int d = 0; d < R; ++d) {
+        if (d % kColsStage == 0) load_x(begin + d, d / kColsStage);
+        if (d % SPG == 0) load_c(begin + d, d / SPG);
+        load_q(begin + d, qb[d]);
+    }
+
+    DequantRegs regs;
+    regs.init(BITS);
+    float4_t acc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+    ColumnConst cc[2];
+    const int a_row = min(nl, M - 1);
+
+    for (int base = 0; base < steps_per_wave; base += R) {
+#pragma unroll
+        for (int d = 0; d < R; ++d) {
+            const int step = begin + base + d;
+            if (d % kColsStage == 0) {
+                store_x(step, d / kColsStage);
+                load_x(step + R, d / kColsStage);
+            }
+            if (d % SPG == 0) {
+                const uint32_t sw = cs_scale[d / SPG], zw = cs_zero[d / SPG];
+                cc[0] = column_const_from_bits(sw & 0xFFFFu, (zw >> (zsub * BITS)) & MASK);
+                cc[1] = column_const_from_bits(sw >> 16, (zw >> ((zsub + 1) * BITS)) & MASK);
+                load_c(step + R, d / SPG);
+            }
+            half8_t b[2];
+            uint2_t* q = qb[d];
+            const uint32_t qa[2] = {q[0].x, q[0].y};
+            const uint32_t qc[2] = {q[LOADS - 1].x, q[LOADS - 1].y};
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                half2_t w[4];
+                dequant_word<BITS>(qa[t], cc[t], regs, w);
+                if constexpr (BITS == 8) dequant_word<BITS>(qc[t], cc[t], regs, w + PAIRS);
+                const uint4_t packed = {as_u32(w[0]), as_u32(w[1]), as_u32(w[2]), as_u32(w[3])};
+                b[t] = __builtin_bit_cast(half8_t, packed);
+            }
+            load_q(step + R, q);
+            __builtin_amdgcn_sched_barrier(0);  // keeps the reload at this place of the body
+            const half8_t a = __builtin_bit_cast(half8_t, xs[wave][a_row * RS + (d % kColsStage) * 4 + kq]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[t], 0, 0, 0);
+        }
+    }
+
+    // ---- the eight partial sums of a column meet in LDS, in wave order
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int m = kq * 4 + r;
+        if (m < M) *reinterpret_cast<float2*>(&red[wave][m][nl * 2]) = make_float2(acc[0][r], acc[1][r]);
+    }
+    __syncthreads();
+    if (tid >= M * (kColsTile / 2)) return;
+    const int m = tid / (kColsTile / 2), c = tid % (kColsTile / 2) * 2;
+    float2 sum = make_float2(0.f, 0.f);
+#pragma unroll
+    for (int w = 0; w < kColsWaves; ++w) {
+        const float2 v = *reinterpret_cast<const float2*>(&red[w][m][c]);
+        sum.x += v.x;
+        sum.y += v.y;
+    }
+    const int col = tile * kColsTile + c;
+    const half2_t y = {(half_t)sum.x, (half_t)sum.y};
+    half2_t* op = reinterpret_cast<half2_t*>(out + (size_t)m * N + col);
+    if (epilogue == kEpilogueResidual) {
+        // out is the residual stream: h += y in fp16, h * next_norm_w for the consumer,
+        // and the sum of squares of the tile's 32 new values (the row's 16 threads
+        // are adjacent lanes of one wave)
+        const half2_t h = *op + y;
+        *op = h;
+        if (fuse.xw_out)
+            *reinterpret_cast<half2_t*>(fuse.xw_out + (size_t)m * N + col) =
+                h * *reinterpret_cast<const half2_t*>(fuse.next_norm_w + col);
+        float ss = (float)h[0] * (float)h[0] + (float)h[1] * (float)h[1];
+#pragma unroll
+        for (int off = 1; off < kColsTile / 2; off <<= 1) ss += __shfl_xor(ss, off);
+        if (c == 0) fuse.ssq_out[(size_t)m * gridDim.x + tile] = ss;
+        return;
+    }
+    *op = y;
+}
+
+bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
+    static const char* off = getenv("MH_GEMM_NO_COLS");
+    if (off && *off && atoi(off)) return false;
+    if (bits != 4 || group_size != 128 || M < 1 || M > 8) return false;
+    if (N % kColsTile != 0 || K % (32 * kColsStage) != 0) return false;
+    return epilogue == kEpilogueNone || epilogue == kEpilogueResidual;
+}
+
+// Where it measured faster than the small-M kernel: every CU gets at most one
+// 32-column tile, and either the tiles cover more than half the CUs or K is short
+// enough for the kernel to be bound by its dependent round trips rather than by
+// the CUs left idle.
+bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
+    if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue)) return false;
+    const int tiles = N / kColsTile, cus = compute_units();
+    return tiles <= cus && K <= 16384 && (K <= 8192 || 2 * tiles > cus);
+}
+
+int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                          const void* scales, void* out, int M, int N, int K, int group_size, int bits, int epilogue,
+                          const SmallFuse& fuse) {
+    if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue) || fuse.ssq_in != nullptr)
+        return fail(MH_ERR_INVALID, "gptq column-owner kernel: unsupported shape or fusion");
+    const int steps_total = K / 32;
+    int spw = (steps_total + kColsWaves - 1) / kColsWaves;
+    spw = (spw + kColsStage - 1) / kColsStage * kColsStage;  // whole stages, hence whole groups
+    const dim3 grid(N / kColsTile);
+#define MH_LAUNCH_COLS(MROWS)                                                                                     \
+    hipLaunchKernelGGL((gptq_gemm_cols_kernel<4, 4, MROWS>), grid, dim3(512), 0, stream, (const half_t*)x,         \
+                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out, M, \
+                       N, K, steps_total, spw, epilogue, fuse)
+    if (M == 1)
+        MH_LAUNCH_COLS(1);
+    else if (M == 2)
+        MH_LAUNCH_COLS(2);
+    else if (M <= 4)
+        MH_LAUNCH_COLS(4);
+    else
+        MH_LAUNCH_COLS(8);
+#undef MH_LAUNCH_COLS
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+}  // namespace mh
