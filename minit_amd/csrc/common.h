@@ -36,6 +36,12 @@ inline hipStream_t as_stream(mh_stream_t s) { return reinterpret_cast<hipStream_
 int compute_units();
 
 typedef _Float16 half_t;
+// Buffer resource word 3 for raw (untyped, offset-addressed) buffer loads on gfx9:
+// DATA_FORMAT = 32 bit; and the cache-policy operand of the buffer load builtins:
+// bit 0 sc0, bit 1 nt, bit 4 sc1 (sc1 alone = agent scope).
+constexpr int kBufferRsrcFlags = 0x00020000;
+constexpr int kBufferStreamAgent = 2 | 16;
+
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));

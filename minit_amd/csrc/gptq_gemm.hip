@@ -289,23 +289,19 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     // block's own last step (a cache hit) instead of running on into the K range of
     // the next split, which would cost the CU a stage's worth of memory requests.
     const int ring_last = min(step_begin + stages_per_block * D - 1, last_step);
+    // Buffer loads: the scalar offset of the step and the lane's fixed 32-bit offset
+    // go to the instruction as they are (no vector address arithmetic, and measured
+    // 3-4 % faster than global_load with a 64-bit address pair on the large shapes);
+    // streaming hint, agent scope: every packed word is read once.
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(qweight), 0, (int)((size_t)(K / P) * N * 4), kBufferRsrcFlags);
     auto load_q = [&](int step, uint4_t* dst) {
         const int s = min(step, last_step);  // a block's last stage runs on into the next split's range
-        // the step's base address stays in scalar registers (opaque to the compiler,
-        // which otherwise folds it into a 64-bit vector multiply-add per load); the
-        // load then takes it as its scalar base next to the lane's fixed 32-bit offset
-        const uint64_t b = reinterpret_cast<uint64_t>(qweight) + (uint64_t)s * ROWS_PER_STEP * N * 4;
-        uint32_t b_lo = (uint32_t)b, b_hi = (uint32_t)(b >> 32);
-        asm("" : "+s"(b_lo), "+s"(b_hi));
-        typedef const char __attribute__((address_space(1))) * global_bytes;
-        typedef const uint4_t __attribute__((address_space(1))) * global_words;
-        const global_bytes base = (global_bytes)(((uint64_t)b_hi << 32) | b_lo);
+        const int soff = s * ROWS_PER_STEP * N * 4;
 #pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            uint32_t off = lane_off[j];
-            asm("" : "+v"(off));  // keeps the zero-extension next to the load
-            dst[j] = __builtin_nontemporal_load((global_words)(base + off));
-        }
+        for (int j = 0; j < LOADS; ++j)
+            dst[j] = __builtin_bit_cast(
+                uint4_t, __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)lane_off[j], soff, kBufferStreamAgent));
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) load_q(step_begin + d, qb[d]);
@@ -786,6 +782,9 @@ static void launch_gemm_mt(hipStream_t stream, const GemmPlan& p, const void* x,
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
+    // the MFMA kernels address the packed weights with 32-bit buffer offsets
+    if ((size_t)K * N * bits / 8 >= ((size_t)1 << 31))
+        return fail(MH_ERR_INVALID, "gptq gemm: packed weights of 2 GiB or more are not supported");
     // a narrow output goes to the kernel whose workgroups own their columns over all of K
     if (fuse.ssq_in == nullptr && gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse);

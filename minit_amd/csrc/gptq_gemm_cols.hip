@@ -81,26 +81,22 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     const int last_step = steps_total - 1;
     const int last_stage_step = (last_step / kColsStage) * kColsStage;
 
-    typedef const char __attribute__((address_space(1))) * global_bytes;
-
     // ---- packed weights
     uint2_t qb[R][LOADS];
     uint32_t lane_off[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) lane_off[j] = (uint32_t)((kq * LOADS + j) * N + col0) * 4u;
+    // buffer loads: scalar offset of the step + the lane's fixed 32-bit offset, no
+    // vector address arithmetic; streaming hint, agent scope
+    const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(qweight), 0, (int)((size_t)(K / P) * N * 4), kBufferRsrcFlags);
     auto load_q = [&](int step, uint2_t* dst) {
         const int s = min(step, last_step);  // past the end of K: re-read the last step, its activations are zero
-        const uint64_t b = reinterpret_cast<uint64_t>(qweight) + (uint64_t)s * ROWS_PER_STEP * N * 4;
-        uint32_t b_lo = (uint32_t)b, b_hi = (uint32_t)(b >> 32);
-        asm("" : "+s"(b_lo), "+s"(b_hi));  // scalar base + 32-bit lane offset: no vector address arithmetic
-        const global_bytes base = (global_bytes)(((uint64_t)b_hi << 32) | b_lo);
-        typedef const uint2_t __attribute__((address_space(1))) * global_words;
+        const int soff = s * ROWS_PER_STEP * N * 4;
 #pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            uint32_t off = lane_off[j];
-            asm("" : "+v"(off));
-            dst[j] = __builtin_nontemporal_load((global_words)(base + off));
-        }
+        for (int j = 0; j < LOADS; ++j)
+            dst[j] = __builtin_bit_cast(
+                uint2_t, __builtin_amdgcn_raw_buffer_load_b64(q_rsrc, (int)lane_off[j], soff, kBufferStreamAgent));
     };
 
     // ---- scales and zero points of a group: one word each for the lane's two columns
