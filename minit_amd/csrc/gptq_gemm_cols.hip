@@ -12,21 +12,22 @@
 // waves until the end and the K loop has no barrier.  Per step of 32 k a lane
 // (column pair nl = lane % 16, k chunk kq = lane / 16) loads 8 bytes: the packed
 // words of its two columns, which are the B operands of two
-// v_mfma_f32_16x16x32_f16.  Everything a step needs is requested 16 steps ahead
+// v_mfma_f32_16x16x32_f16.  Everything a step needs is requested 8 steps ahead
 // and in the order of use (activations of a 256-k stage, scale/zero words of a
-// group, packed weights), so each s_waitcnt vmcnt(n) leaves the 16 steps behind it
-// in flight: 8 KiB per wave, 64 KiB per CU.  More in flight measured slower (a
-// 16-byte-per-lane variant with 128 KiB per CU lost 25 %), and beyond about 34
-// loads in flight per wave the compiler's vmcnt bookkeeping falls back to
-// draining the queue at the top of the loop.  Activations go through a
-// wave-private LDS area (re-ordered to the pair order of dequant_word on the way);
-// LDS instructions of one wave execute in order, so the area needs neither a
-// second buffer nor a barrier.
+// group, packed weights), so each s_waitcnt vmcnt(n) leaves the 8 steps behind it
+// in flight: 4 KiB per wave, 32 KiB per CU.  More in flight measured slower (16
+// steps: 8192x8192 in 11.4 us instead of 9.8; a 16-byte-per-lane variant with
+// 128 KiB per CU: 14.7 us), and beyond about 34 loads in flight per wave the
+// compiler's vmcnt bookkeeping falls back to draining the queue at the top of the
+// loop.  Activations go through a wave-private LDS area (re-ordered to the pair
+// order of dequant_word on the way); LDS instructions of one wave execute in
+// order, so the area needs neither a second buffer nor a barrier.
 //
-// Measured against the small-M kernel (M = 1, us): 8192x8192 12.2 / 15.3,
-// 4096x4096 7.4 / 9.1, 16384x8192 18.1 / 22.3; with more 32-column tiles than CUs
-// (10240 columns: 19.0 / 15.2) or half the CUs idle on a long K (14336x4096:
-// 16.6 / 14.8) it loses, see gemm_cols_preferred.
+// Measured against the small-M kernel (M = 1, us): 8192x8192 9.8 / 15.3,
+// 4096x4096 5.8 / 9.1, 16384x8192 15.7 / 22.3, 28672x8192 24.5 / 26.2 (at 8 rows
+// 29.8 / 28.2); with more 32-column tiles than CUs (10240 columns: 15.9 / 15.0) or
+// half the CUs idle on a long K (14336x4096: 16.6 / 14.8) it loses, see
+// gemm_cols_preferred.
 #include "gptq_common.h"
 
 namespace mh {
@@ -36,7 +37,7 @@ namespace mh {
 constexpr int kColsTile = 32;   // columns per workgroup
 constexpr int kColsWaves = 8;   // K ranges per workgroup
 constexpr int kColsStage = 8;   // steps per activation stage
-constexpr int kColsRing = 16;   // steps in flight per wave
+constexpr int kColsRing = 8;    // steps in flight per wave
 
 // (s, s), (1024 + z + 1) twice, (64 + z + 1) twice from the bits of s and the
 // zero point: below 2048 an fp16 integer n + 1024 is the bit pattern 0x6400 + n,
@@ -240,8 +241,10 @@ bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epil
 // the CUs left idle.
 bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
     if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue)) return false;
+    static const char* force = getenv("MH_GEMM_COLS_FORCE");
+    if (force && *force && atoi(force)) return true;
     const int tiles = N / kColsTile, cus = compute_units();
-    return tiles <= cus && K <= 16384 && (K <= 8192 || 2 * tiles > cus);
+    return tiles <= cus && (K <= 8192 || 2 * tiles > cus) && (K <= 16384 || M <= 2);
 }
 
 int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
