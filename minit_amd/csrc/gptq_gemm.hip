@@ -242,12 +242,15 @@ constexpr int kSmallDepth = 8;  // steps per stage = ring depth
 // ssq[m] the sum of the fuse.ssq_tiles partial sums of squares the producer left
 // behind, scales the fp32 accumulators at the end, so the row never needs a pass
 // of its own.
-template <int BITS, int MT, int SPG, bool NORM>
+// STREAM: the balanced plan described below (it costs registers: a second set of
+// accumulators), otherwise only the regular one.
+template <int BITS, int MT, int SPG, bool NORM, bool STREAM>
 __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
     half_t* out, float* partial, unsigned* counters,
-    int M, int N, int K, int steps_total, int stages_per_block, int split_k, int epilogue, SmallFuse fuse) {
+    int M, int N, int K, int steps_total, int stages_per_block, int split_k, int stream_units, int epilogue,
+    SmallFuse fuse) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
     constexpr uint32_t MASK = Packing<BITS>::kMask;
@@ -269,42 +272,67 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 15, kq = lane >> 4;
-    const int tile = blockIdx.x, split = blockIdx.y;
     const int lcol = wave * 64 + nl * 4;
-    const int col = tile * kGemmCols + lcol;
-    const bool active = col < N;
-    const int colc = active ? col : 0;
-
-    const int step_begin = split * stages_per_block * D;
     const int last_step = steps_total - 1;
     const int g_last = last_step / SPG;
+
+    // The work of a workgroup is stages_per_block consecutive stages of a walk over
+    // (column tile, stage) pairs, tile by tile.  Regular plan (stream_units == 0):
+    // grid (tiles, splits), a workgroup stays inside its tile.  Balanced plan: 1-D
+    // grid over a walk with stream_units stages per tile, cut into equal ranges; a
+    // range may end one tile and begin the next (n0 stages of tile t0 from stage
+    // s0, then n1 stages of tile t0 + 1 from its stage 0).  The K loop runs through
+    // both without a break; the first tile's accumulators are set aside at the
+    // border.  A tile's contributors are consecutive workgroups, which gives each
+    // its slot among the partial sums and every tile its count.
+    int t0, s0, n0, n1, slot0, nseg0, nseg1;
+    if (!STREAM || stream_units == 0) {
+        t0 = blockIdx.x;
+        s0 = blockIdx.y * stages_per_block;
+        n0 = stages_per_block;
+        n1 = 0;
+        slot0 = blockIdx.y;
+        nseg0 = split_k;
+        nseg1 = 0;
+    } else {
+        const int S = stream_units, q = stages_per_block;
+        const int lo = blockIdx.x * q, hi = min(lo + q, (N + kGemmCols - 1) / kGemmCols * S);
+        t0 = lo / S;
+        s0 = lo - t0 * S;
+        n0 = min(S - s0, hi - lo);
+        n1 = hi - lo - n0;
+        slot0 = blockIdx.x - t0 * S / q;
+        nseg0 = (t0 * S + S - 1) / q - t0 * S / q + 1;
+        nseg1 = ((t0 + 1) * S + S - 1) / q - (t0 + 1) * S / q + 1;  // this workgroup holds slot 0 there
+    }
+    const int n_stages = n0 + n1;
+    // stage i of the range: its tile and its first step within K
+    auto tile_of = [&](int i) { return i < n0 ? t0 : t0 + 1; };
+    auto step_of = [&](int i) { return (i < n0 ? s0 + i : i - n0) * D; };
 
     // ---- weight ring
     uint4_t qb[D][LOADS];
     uint32_t lane_off[LOADS];
 #pragma unroll
-    for (int j = 0; j < LOADS; ++j) lane_off[j] = (uint32_t)((kq * LOADS + j) * N + colc) * 4u;
-    // The ring is refilled at a fixed place of the loop body, also in the block's
-    // last stage, where there is nothing left to fetch: those loads re-read the
-    // block's own last step (a cache hit) instead of running on into the K range of
-    // the next split, which would cost the CU a stage's worth of memory requests.
-    const int ring_last = min(step_begin + stages_per_block * D - 1, last_step);
+    for (int j = 0; j < LOADS; ++j) lane_off[j] = (uint32_t)((kq * LOADS + j) * N + lcol) * 4u;
     // Buffer loads: the scalar offset of the step and the lane's fixed 32-bit offset
     // go to the instruction as they are (no vector address arithmetic, and measured
     // 3-4 % faster than global_load with a 64-bit address pair on the large shapes);
-    // streaming hint, agent scope: every packed word is read once.
+    // streaming hint, agent scope: every packed word is read once.  The tile's first
+    // column travels in the scalar offset; columns past N (last tile) read the
+    // neighbouring row or, past the end of the buffer, zero, and are never stored.
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint32_t*>(qweight), 0, (int)((size_t)(K / P) * N * 4), kBufferRsrcFlags);
-    auto load_q = [&](int step, uint4_t* dst) {
-        const int s = min(step, last_step);  // a block's last stage runs on into the next split's range
-        const int soff = s * ROWS_PER_STEP * N * 4;
+    auto load_q = [&](int tile, int step, uint4_t* dst) {
+        const int s = min(step, last_step);  // the last stage's refills run on into the range that follows
+        const int soff = (s * ROWS_PER_STEP * N + tile * kGemmCols) * 4;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j)
             dst[j] = __builtin_bit_cast(
                 uint4_t, __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)lane_off[j], soff, kBufferStreamAgent));
     };
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_q(step_begin + d, qb[d]);
+    for (int d = 0; d < D; ++d) load_q(t0, s0 * D + d, qb[d]);
 
     // ---- staging of activations and constants: global -> registers -> LDS
     uint4 xr[XL];
@@ -324,26 +352,46 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         x_chunk[u] = idx % XCH;
     }
     const int c_group = tid / CT, c_col0 = tid % CT * CE;
-    const int c_colg = min(tile * kGemmCols + c_col0, N - CE);  // N is a multiple of 8: stays aligned to CE
-    auto fetch_stage = [&](int stage_step) {
-        const int sclamp = min(stage_step, (last_step / D) * D);  // never read past K
+    // Buffer loads again: a fixed per-thread offset plus a scalar one that carries the
+    // stage (group row, k) and the tile, so that moving on to the next stage or tile
+    // costs no vector arithmetic.  Columns past N pick up the next row's values or,
+    // past the end, zero: they only feed columns that are never stored.
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, (int)((size_t)M * K * 2), kBufferRsrcFlags);
+    const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<half_t*>(scales), 0, (int)((size_t)(g_last + 1) * N * 2), kBufferRsrcFlags);
+    const __amdgpu_buffer_rsrc_t z_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(qzeros), 0, (int)((size_t)(g_last + 1) * (N / P) * 4), kBufferRsrcFlags);
+    int x_off[XL];
+#pragma unroll
+    for (int u = 0; u < XL; ++u) x_off[u] = (x_row[u] * K + x_chunk[u] * 8) * 2;
+    const int s_off = (c_group * N + c_col0) * 2, z_off = (c_group * (N / P) + c_col0 / P) * 4;
+    auto fetch_stage = [&](int i) {
+        const int sclamp = min(step_of(i), (last_step / D) * D);  // never read past K
+        const int g0 = sclamp / SPG, tile = tile_of(i);  // groups past the last one (dead steps) read zero
 #pragma unroll
         for (int u = 0; u < XL; ++u)
-            xr[u] = *reinterpret_cast<const uint4*>(x + (size_t)x_row[u] * K + (size_t)sclamp * 32 + x_chunk[u] * 8);
-        const int g = min(sclamp / SPG + c_group, g_last);
-        const half_t* sp = scales + (size_t)g * N + c_colg;
+            xr[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, x_off[u], sclamp * 64, 0));
+        const int s_soff = (g0 * N + tile * kGemmCols) * 2;
         if constexpr (CE == 1) {
-            sr[0] = *reinterpret_cast<const uint16_t*>(sp);
+            sr[0] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, s_off, s_soff, 0);
+        } else if constexpr (CE == 2) {
+            sr[0] = __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, s_off, s_soff, 0);
+        } else if constexpr (CE == 4) {
+            const uint2_t v = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(s_rsrc, s_off, s_soff, 0));
+            sr[0] = v[0];
+            sr[1] = v[1];
         } else {
-            struct alignas(CE * 2) ScaleWords { uint32_t w[CE / 2]; };
-            const ScaleWords v = *reinterpret_cast<const ScaleWords*>(sp);
+            const uint4_t v = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(s_rsrc, s_off, s_soff, 0));
 #pragma unroll
-            for (int j = 0; j < CE / 2; ++j) sr[j] = v.w[j];
+            for (int j = 0; j < 4; ++j) sr[j] = v[j];
         }
+        const int z_soff = (g0 * (N / P) + tile * (kGemmCols / P)) * 4;
 #pragma unroll
-        for (int j = 0; j < ZW; ++j) zr[j] = qzeros[(size_t)g * (N / P) + c_colg / P + j];
+        for (int j = 0; j < ZW; ++j) zr[j] = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc, z_off + j * 4, z_soff, 0);
     };
-    auto store_stage = [&](int buf, int stage_step) {
+    auto store_stage = [&](int buf, int i) {
+        const int stage_step = step_of(i);
 #pragma unroll
         for (int u = 0; u < XL; ++u) {
             const uint32_t in[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
@@ -360,7 +408,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 live ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
         }
         {
-            const int zsub = CE >= P ? 0 : c_colg % P;  // first sub-word of this thread in zr[0]
+            const int zsub = CE >= P ? 0 : c_col0 % P;  // first sub-word of this thread in zr[0]
             uint32_t k_scale[CE], k_lo[CE], k_hi[CE];
 #pragma unroll
             for (int j = 0; j < CE; ++j) {
@@ -383,7 +431,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         }
     };
 
-    fetch_stage(step_begin);
+    fetch_stage(0);
     if constexpr (NORM) {
         // 1 / rms of every row from the producer's per-tile sums of squares: 32
         // lanes per row read the tiles in parallel (the loads travel with those of
@@ -391,17 +439,17 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         // after the K loop
 #pragma unroll
         for (int pass = 0; pass < (BM * 32 + 255) / 256; ++pass) {
-            const int row = pass * 8 + (tid >> 5), t0 = tid & 31;
+            const int row = pass * 8 + (tid >> 5), p0 = tid & 31;
             float ss = 0.f;
             if (row < M)
-                for (int t = t0; t < fuse.ssq_tiles; t += 32) ss += fuse.ssq_in[(size_t)row * fuse.ssq_tiles + t];
+                for (int t = p0; t < fuse.ssq_tiles; t += 32) ss += fuse.ssq_in[(size_t)row * fuse.ssq_tiles + t];
 #pragma unroll
             for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
-            if (t0 == 0 && row < BM) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+            if (p0 == 0 && row < BM) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
         }
     }
-    store_stage(0, step_begin);
-    fetch_stage(step_begin + D);
+    store_stage(0, 0);
+    fetch_stage(1);
     __syncthreads();
 
     DequantRegs regs;
@@ -411,11 +459,16 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[mt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float4_t acc_first[STREAM ? MT : 1][4];  // the first tile's sums when the range goes on into a second tile
+#pragma unroll
+    for (int mt = 0; mt < (STREAM ? MT : 1); ++mt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc_first[mt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
     ColumnConst cc[4];
 
-    for (int stage = 0; stage < stages_per_block; ++stage) {
+    for (int stage = 0; stage < n_stages; ++stage) {
         const int buf = stage & 1;
-        const int stage_step = step_begin + stage * D;
+        const int next_tile = tile_of(stage + 1), next_step = step_of(stage + 1);
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             if (d % SPG == 0) {  // compile-time: a new group starts here
@@ -439,7 +492,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 const uint4_t packed = {as_u32(w[0]), as_u32(w[1]), as_u32(w[2]), as_u32(w[3])};
                 b[t] = __builtin_bit_cast(half8_t, packed);
             }
-            load_q(stage_step + d + D, q);
+            load_q(next_tile, next_step + d, q);
             __builtin_amdgcn_sched_barrier(0);  // keep the reload here (see above)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
@@ -449,44 +502,54 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                     acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[mt][t], 0, 0, 0);
             }
         }
-        store_stage(buf ^ 1, stage_step + D);
-        fetch_stage(stage_step + 2 * D);
+        store_stage(buf ^ 1, stage + 1);
+        fetch_stage(stage + 2);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        if (STREAM && stage == n0 - 1 && n1 > 0) {  // border between the two tiles: registers only
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    acc_first[mt][t] = acc[mt][t];
+                    acc[mt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+        }
     }
 
-    // ---- results.  With K split over several workgroups every one publishes
-    // its fp32 partial tile with agent-scope stores (they go through to memory,
-    // which is what workgroups on other XCDs see) and counts itself in; the one
-    // that arrives last adds the partials in split order -- a fixed order, so the
-    // result does not depend on which workgroup that is -- and puts the counter
-    // back to zero for the next launch.  The SiLU-pair epilogue always takes this
-    // route (its two operands sit in different waves' accumulators).
-    if constexpr (NORM) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float inv = inv_rms_s[mt * 16 + kq * 4 + r];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) acc[mt][t][r] *= inv;
-            }
-    }
-    const bool direct = split_k == 1 && epilogue == kEpilogueNone;  // the other epilogues need the whole tile
-    if (active) {
+    // ---- results.  A tile with several contributors: every one publishes its
+    // fp32 partial tile with agent-scope stores (they go through to memory, which
+    // is what workgroups on other XCDs see) and counts itself in; the one that
+    // arrives last adds the partials in slot order -- a fixed order, so the result
+    // does not depend on which workgroup that is -- and puts the counter back to
+    // zero for the next launch.  The SiLU-pair, residual and RoPE epilogues always
+    // take this route (they need the whole tile).  A workgroup that worked on two
+    // tiles publishes both, waits once, and may be the last one of either.
+    const int n_seg = STREAM && n1 > 0 ? 2 : 1;
+    __shared__ int is_last[2];
+    bool need_reduce = false;
+    for (int sg = 0; sg < n_seg; ++sg) {
+        const int tile = t0 + sg, slot = sg == 0 ? slot0 : 0, nseg = sg == 0 ? nseg0 : nseg1;
+        const int col = tile * kGemmCols + lcol;
+        const bool first_of_two = STREAM && sg == 0 && n1 > 0;
+        const bool direct = nseg == 1 && epilogue == kEpilogueNone;
+        need_reduce = need_reduce || !direct;
+        if (col >= N) continue;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = mt * 16 + kq * 4 + r;
                 if (m >= M) continue;
+                float4_t v;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = first_of_two ? acc_first[STREAM ? mt : 0][t][r] : acc[mt][t][r];
+                if constexpr (NORM) v *= inv_rms_s[m];
                 if (direct) {
-                    const half4_t h = {(half_t)acc[mt][0][r], (half_t)acc[mt][1][r], (half_t)acc[mt][2][r],
-                                       (half_t)acc[mt][3][r]};
+                    const half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
                 } else {
-                    const float4_t v = {acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
-                    float* dst = partial + ((size_t)split * M + m) * N + col;
+                    float* dst = partial + ((size_t)slot * M + m) * N + col;
                     if (counters)
                         store_agent4(dst, v);
                     else
@@ -494,100 +557,120 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 }
             }
     }
-    if (direct || counters == nullptr) return;  // without counters a second kernel adds the partials
+    if (!need_reduce || counters == nullptr) return;  // without counters a second kernel adds the partials
 
-    __shared__ int is_last;
-    if (!arrive_and_check_last(&counters[tile], (unsigned)split_k, &is_last)) return;
-    constexpr int BATCH = 16;  // partial loads in flight per thread
-    const size_t plane = (size_t)M * N;
-    auto sum_splits = [&](const float* p) {
-        float4_t s = {0.f, 0.f, 0.f, 0.f};
-        for (int sp = 0; sp < split_k; sp += BATCH) {
-            float4_t v[BATCH];
-#pragma unroll
-            for (int u = 0; u < BATCH; ++u)
-                v[u] = sp + u < split_k ? load_agent4(p + (size_t)(sp + u) * plane) : float4_t{0.f, 0.f, 0.f, 0.f};
-            wait_agent_loads(v);
-#pragma unroll
-            for (int u = 0; u < BATCH; ++u)
-                if (sp + u < split_k) s += v[u];
+    // every thread's stores acknowledged, then one arrival per tile
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+        for (int sg = 0; sg < n_seg; ++sg) {
+            const unsigned expected = sg == 0 ? nseg0 : nseg1;
+            int last = 0;
+            if (!(expected == 1 && epilogue == kEpilogueNone)) {
+                const unsigned prev =
+                    __hip_atomic_fetch_add(&counters[t0 + sg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = prev == expected - 1;
+                if (last) __hip_atomic_store(&counters[t0 + sg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            is_last[sg] = last;
         }
-        return s;
-    };
-    if (epilogue == kEpilogueSiluPairs) {
-        // columns [0, 128) of the tile are gate, [128, 256) the matching up columns
-        for (int item = tid; item < M * (kGemmCols / 8); item += 256) {
-            const int m = item / (kGemmCols / 8), c4 = item % (kGemmCols / 8) * 4;
-            const float* p = partial + (size_t)m * N + tile * kGemmCols + c4;
-            const float4_t g = sum_splits(p), u = sum_splits(p + kGemmCols / 2);
-            half4_t h;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
-            *reinterpret_cast<half4_t*>(out + (size_t)m * (N / 2) + tile * (kGemmCols / 2) + c4) = h;
-        }
-        return;
     }
-    if (epilogue == kEpilogueRopeAppend) {
-        // four consecutive columns = two interleaved pairs of one head
+    __syncthreads();
+
+    auto reduce_tile = [&](int tile, int nseg) {
+        constexpr int BATCH = 16;  // partial loads in flight per thread
+        const size_t plane = (size_t)M * N;
+        auto sum_splits = [&](const float* p) {
+            float4_t s = {0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < nseg; sp += BATCH) {
+                float4_t v[BATCH];
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u)
+                    v[u] = sp + u < nseg ? load_agent4(p + (size_t)(sp + u) * plane) : float4_t{0.f, 0.f, 0.f, 0.f};
+                wait_agent_loads(v);
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u)
+                    if (sp + u < nseg) s += v[u];
+            }
+            return s;
+        };
+        if (epilogue == kEpilogueSiluPairs) {
+            // columns [0, 128) of the tile are gate, [128, 256) the matching up columns
+            for (int item = tid; item < M * (kGemmCols / 8); item += 256) {
+                const int m = item / (kGemmCols / 8), c4 = item % (kGemmCols / 8) * 4;
+                const float* p = partial + (size_t)m * N + tile * kGemmCols + c4;
+                const float4_t g = sum_splits(p), u = sum_splits(p + kGemmCols / 2);
+                half4_t h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
+                *reinterpret_cast<half4_t*>(out + (size_t)m * (N / 2) + tile * (kGemmCols / 2) + c4) = h;
+            }
+            return;
+        }
+        if (epilogue == kEpilogueRopeAppend) {
+            // four consecutive columns = two interleaved pairs of one head
+            for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
+                const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
+                const float4_t sum = sum_splits(partial + (size_t)m * N + c);
+                const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                const int head = c / 128, d = c % 128;
+                const int pos = fuse.positions[m];
+                if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
+                    half_t* dst = fuse.vt_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) *
+                                                      fuse.max_seq + pos;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
+                    continue;
+                }
+                const float* cr = fuse.rope_cos + (size_t)pos * 64 + d / 2;
+                const float* sr = fuse.rope_sin + (size_t)pos * 64 + d / 2;
+                half4_t o;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float re = (float)y[2 * j], im = (float)y[2 * j + 1];
+                    o[2 * j] = (half_t)(re * cr[j] - im * sr[j]);
+                    o[2 * j + 1] = (half_t)(im * cr[j] + re * sr[j]);
+                }
+                half_t* dst = head < fuse.q_heads
+                                  ? fuse.q_out + ((size_t)m * fuse.q_heads + head) * 128 + d
+                                  : fuse.k_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads)) * fuse.max_seq + pos) * 128 + d;
+                *reinterpret_cast<half4_t*>(dst) = o;
+            }
+            return;
+        }
+        if (epilogue == kEpilogueResidual) {
+            // a wave owns one row of the tile per pass (64 lanes x 4 columns), so the
+            // row's sum of squares is one wave reduction; N is a multiple of 256
+            for (int base = 0; base < M * (kGemmCols / 4); base += 256) {
+                const int m = base / (kGemmCols / 4) + wave, c = tile * kGemmCols + lane * 4;
+                float ss = 0.f;
+                if (m < M) {
+                    const float4_t s = sum_splits(partial + (size_t)m * N + c);
+                    half_t* hp = out + (size_t)m * N + c;
+                    const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+                    const half4_t h = *reinterpret_cast<const half4_t*>(hp) + y;  // fp16 add, one rounding
+                    *reinterpret_cast<half4_t*>(hp) = h;
+                    if (fuse.xw_out)
+                        *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) =
+                            h * *reinterpret_cast<const half4_t*>(fuse.next_norm_w + c);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
+                }
+                ss = wave_sum(ss);
+                if (lane == 0 && m < M) fuse.ssq_out[(size_t)m * (N / kGemmCols) + tile] = ss;
+            }
+            return;
+        }
         for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
             const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
-            const float4_t sum = sum_splits(partial + (size_t)m * N + c);
-            const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
-            const int head = c / 128, d = c % 128;
-            const int pos = fuse.positions[m];
-            if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
-                half_t* dst = fuse.vt_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) *
-                                                  fuse.max_seq + pos;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
-                continue;
-            }
-            const float* cr = fuse.rope_cos + (size_t)pos * 64 + d / 2;
-            const float* sr = fuse.rope_sin + (size_t)pos * 64 + d / 2;
-            half4_t o;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const float re = (float)y[2 * j], im = (float)y[2 * j + 1];
-                o[2 * j] = (half_t)(re * cr[j] - im * sr[j]);
-                o[2 * j + 1] = (half_t)(im * cr[j] + re * sr[j]);
-            }
-            half_t* dst = head < fuse.q_heads
-                              ? fuse.q_out + ((size_t)m * fuse.q_heads + head) * 128 + d
-                              : fuse.k_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads)) * fuse.max_seq + pos) * 128 + d;
-            *reinterpret_cast<half4_t*>(dst) = o;
+            if (c >= N) continue;
+            const float4_t s = sum_splits(partial + (size_t)m * N + c);
+            const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+            *reinterpret_cast<half4_t*>(out + (size_t)m * N + c) = h;
         }
-        return;
-    }
-    if (epilogue == kEpilogueResidual) {
-        // a wave owns one row of the tile per pass (64 lanes x 4 columns), so the
-        // row's sum of squares is one wave reduction; N is a multiple of 256
-        for (int base = 0; base < M * (kGemmCols / 4); base += 256) {
-            const int m = base / (kGemmCols / 4) + wave, c = tile * kGemmCols + lane * 4;
-            float ss = 0.f;
-            if (m < M) {
-                const float4_t s = sum_splits(partial + (size_t)m * N + c);
-                half_t* hp = out + (size_t)m * N + c;
-                const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
-                const half4_t h = *reinterpret_cast<const half4_t*>(hp) + y;  // fp16 add, one rounding
-                *reinterpret_cast<half4_t*>(hp) = h;
-                if (fuse.xw_out)
-                    *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) =
-                        h * *reinterpret_cast<const half4_t*>(fuse.next_norm_w + c);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
-            }
-            ss = wave_sum(ss);
-            if (lane == 0 && m < M) fuse.ssq_out[(size_t)m * gridDim.x + tile] = ss;
-        }
-        return;
-    }
-    for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
-        const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
-        if (c >= N) continue;
-        const float4_t s = sum_splits(partial + (size_t)m * N + c);
-        const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
-        *reinterpret_cast<half4_t*>(out + (size_t)m * N + c) = h;
-    }
+    };
+    for (int sg = 0; sg < n_seg; ++sg)
+        if (is_last[sg]) reduce_tile(t0 + sg, sg == 0 ? nseg0 : nseg1);
 }
 
 // gptq_gemm_cols.hip
@@ -600,9 +683,11 @@ struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
     int col_tiles;
     int m_blocks;
-    int split_k;
+    int split_k;  // partial-sum slots per tile
     int steps_total;
     int steps_per_block;
+    int stream_units = 0;  // small-M kernel, balanced plan: stages per tile of the walk (0: regular plan)
+    int blocks = 0;        // balanced plan: workgroups
 };
 
 static int env_int_gemm(const char* name, int fallback) {
@@ -617,7 +702,7 @@ constexpr int kFusedReduceMaxM = 8;
 // Plan of the small-M kernel: column tiles x K splits sized so the GPU holds
 // about MH_GEMM_SMALL_WAVES_PER_CU waves per CU; a block walks whole stages.
 // GemmPlan::steps_per_block carries stages_per_block * kSmallDepth.
-GemmPlan plan_gemm_small(int M, int N, int K) {
+GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced) {
     GemmPlan p;
     p.mt = M <= 16 ? 1 : 2;
     p.col_tiles = (N + kGemmCols - 1) / kGemmCols;
@@ -635,6 +720,30 @@ GemmPlan plan_gemm_small(int M, int N, int K) {
     const long spb = (stages_total + split - 1) / split;
     p.steps_per_block = (int)(spb * kSmallDepth);
     p.split_k = (int)((stages_total + spb - 1) / spb);
+    // Balanced plan (in-kernel reduction only): the tiles' stages form one walk that
+    // is cut into target_blocks equal ranges, so every CU gets the same number of
+    // stages even where tiles x splits does not divide by the CUs (224 tiles x 2
+    // splits on 256 CUs: 1.75 workgroups per CU, two on most).  A range covers at
+    // most two tiles, and no tile gets more contributors than the caps above allow.
+    // Worth it for long ranges only (measured: 8192x57344, 14 stages per workgroup,
+    // 50.0 -> 48.1 us; 8192x10240, 3 stages, 15.2 -> 16.2 us: the workgroups that
+    // work on two tiles end with two hand-offs), and not with an epilogue in the
+    // reduction or the norm prologue (the same gate|up product with both: 49.7 ->
+    // 54.1 us), which is what allow_balanced says.
+    static const int balance = env_int_gemm("MH_GEMM_BALANCE", 1);
+    if (balance && allow_balanced && M <= kFusedReduceMaxM && p.col_tiles <= kMaxTileCounters) {
+        const long units = (long)p.col_tiles * stages_total;
+        long q = (units + target_blocks - 1) / target_blocks;
+        const long cap = traffic_cap < stages_total ? traffic_cap : stages_total;  // contributors per tile
+        const long q_min = (stages_total + cap - 1) / cap;
+        if (q < q_min) q = q_min;
+        if (q >= 8 && q <= stages_total && stages_total % q != 0) {
+            p.stream_units = (int)stages_total;
+            p.steps_per_block = (int)(q * kSmallDepth);
+            p.blocks = (int)((units + q - 1) / q);
+            p.split_k = (int)((stages_total + q - 1) / q + 1);
+        }
+    }
     return p;
 }
 
@@ -644,8 +753,8 @@ static bool use_small(int M, int group_size) {
     return !off && M <= kSmallMaxM && (spg == 1 || spg == 2 || spg == 4 || spg == 8);
 }
 
-GemmPlan plan_gemm(int M, int N, int K, int group_size) {
-    if (use_small(M, group_size)) return plan_gemm_small(M, N, K);
+GemmPlan plan_gemm(int M, int N, int K, int group_size, bool allow_balanced) {
+    if (use_small(M, group_size)) return plan_gemm_small(M, N, K, allow_balanced);
     GemmPlan p;
     p.mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
     const int bm = 16 * p.mt;
@@ -704,10 +813,12 @@ static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_sm
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)bits;
     if (row_blocked(M, group_size)) M = kSmallMaxM;  // taken 32 rows at a time
-    const GemmPlan p = plan_gemm(M, N, K, group_size);
+    // either plan of the small-M kernel may be the one a launch takes
+    const GemmPlan p = plan_gemm(M, N, K, group_size, false), pb = plan_gemm(M, N, K, group_size, true);
+    const int slots = p.split_k > pb.split_k ? p.split_k : pb.split_k;
     // the small-M kernel may be asked for an epilogue that goes through the partials even unsplit
-    if (p.split_k <= 1 && !use_small(M, group_size)) return 0;
-    return kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float);
+    if (slots <= 1 && !use_small(M, group_size)) return 0;
+    return kTileCounterBytes + (size_t)slots * M * N * sizeof(float);
 }
 
 template <int BITS, int MT>
@@ -732,19 +843,21 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
     unsigned* counters =
         (M <= kFusedReduceMaxM && p.col_tiles <= kMaxTileCounters) ? reinterpret_cast<unsigned*>(workspace) : nullptr;
     float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
-    const dim3 grid(p.col_tiles, p.split_k);
+    const dim3 grid = p.stream_units ? dim3(p.blocks) : dim3(p.col_tiles, p.split_k);
     const bool norm = fuse.ssq_in != nullptr;
-#define MH_LAUNCH_SMALL_N(SPG, NORM)                                                                                \
-    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG, NORM>), grid, dim3(256), 0, stream, (const half_t*)x, \
-                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,      \
-                       partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth, p.split_k,      \
-                       epilogue, fuse)
-#define MH_LAUNCH_SMALL(SPG)                 \
-    do {                                     \
-        if (norm)                            \
-            MH_LAUNCH_SMALL_N(SPG, true);    \
-        else                                 \
-            MH_LAUNCH_SMALL_N(SPG, false);   \
+#define MH_LAUNCH_SMALL_N(SPG, NORM, STREAM)                                                                  \
+    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG, NORM, STREAM>), grid, dim3(256), 0, stream,         \
+                       (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, \
+                       (half_t*)out, partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth,  \
+                       p.split_k, p.stream_units, epilogue, fuse)
+#define MH_LAUNCH_SMALL(SPG)                            \
+    do {                                                \
+        if (norm)                                       \
+            MH_LAUNCH_SMALL_N(SPG, true, false);        \
+        else if (MT == 1 && p.stream_units != 0)        \
+            MH_LAUNCH_SMALL_N(SPG, false, (MT == 1));   \
+        else                                            \
+            MH_LAUNCH_SMALL_N(SPG, false, false);       \
     } while (0)
     switch (group_size / 32) {
         case 1: MH_LAUNCH_SMALL(1); break;
@@ -805,7 +918,7 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
         }
         return MH_OK;
     }
-    const GemmPlan p = plan_gemm(M, N, K, group_size);
+    const GemmPlan p = plan_gemm(M, N, K, group_size, epilogue == kEpilogueNone && fuse.ssq_in == nullptr);
     if ((fuse.ssq_in != nullptr || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
         !gemm_norm_fusion_supported(M, N, K, group_size, bits, epilogue))
         return fail(MH_ERR_INVALID, "gptq gemm: RMSNorm / RoPE fusion needs M <= %d, a group of 32..256 and N %% 256 == 0 "
