@@ -298,19 +298,25 @@ __global__ __launch_bounds__(kI8Threads) void i8_gemm_k128_kernel(
     // thread) and W has 2048 (four per thread); eight threads fetch one row's line.
     int4_t ra[R][2], rb[R][4];
     const int crow = tid >> 3, cchunk = tid & 7;
-    const int8_t* a_src[2];
-    const int8_t* b_src[4];
+    // buffer loads: a fixed 32-bit offset per thread and row, the k offset scalar
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(A), 0, (int)((size_t)M * K), kBufferRsrcFlags);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(W), 0, (int)((size_t)N * K), kBufferRsrcFlags);
+    int a_off[2], b_off[4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) a_src[j] = A + (size_t)min(m0 + crow + 64 * j, M - 1) * K + cchunk * 16;
+    for (int j = 0; j < 2; ++j) a_off[j] = min(m0 + crow + 64 * j, M - 1) * K + cchunk * 16;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b_src[j] = W + (size_t)min(n0 + crow + 64 * j, N - 1) * K + cchunk * 16;
+    for (int j = 0; j < 4; ++j) b_off[j] = min(n0 + crow + 64 * j, N - 1) * K + cchunk * 16;
     const int KT = K / BK;
     auto load_stage = [&](int slot, int kt) {
         const int k0 = min(kt, KT - 1) * BK;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) ra[slot][j] = *reinterpret_cast<const int4_t*>(a_src[j] + k0);
+        for (int j = 0; j < 2; ++j)
+            ra[slot][j] = __builtin_bit_cast(int4_t, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[j], k0, 0));
 #pragma unroll
-        for (int j = 0; j < 4; ++j) rb[slot][j] = *reinterpret_cast<const int4_t*>(b_src[j] + k0);
+        for (int j = 0; j < 4; ++j)
+            rb[slot][j] = __builtin_bit_cast(int4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, b_off[j], k0, 0));
     };
     // LDS rows are 128 bytes; the chunk index is XOR-ed with bits 1..3 of the row, so
     // that the 32 rows a fragment read touches spread over all 16-byte bank groups.
@@ -550,7 +556,9 @@ int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w, const float
     const int group_m = tiles_m < 8 ? tiles_m : 8;
     const int xcd_chunk = (tiles % 8 == 0) ? tiles / 8 : 0;
     static const char* no128 = getenv("MH_I8_NO_K128");
-    if (K % 128 == 0 && !(no128 && *no128 && atoi(no128))) {
+    // the 128-k kernel addresses its operands with 32-bit buffer offsets
+    if (K % 128 == 0 && (size_t)M * K < ((size_t)1 << 31) && (size_t)N * K < ((size_t)1 << 31) &&
+        !(no128 && *no128 && atoi(no128))) {
         const int kt128 = K / 128;
 #define MH_I8_LAUNCH128(R)                                                                                          \
     hipLaunchKernelGGL(i8_gemm_k128_kernel<R>, dim3(tiles), dim3(kI8Threads), 0, as_stream(stream), a, w, a_scale, \
