@@ -27,7 +27,10 @@ def _run(hip, a, w, a_scale, w_scale, want_acc=True, want_out=True):
     (128, 256, 64),       # exactly one tile, one k-step
     (1, 8, 64),           # far smaller than a tile
     (130, 260, 192),      # ragged M and N
-    (257, 1000, 512),
+    (257, 1000, 512),     # 128-k stages, ring of four
+    (100, 300, 768),      # 128-k stages, ring of two
+    (64, 136, 384),       # 128-k stages, ring of one
+    (130, 260, 128),      # a single 128-k stage
     (2048, 4096, 4096),   # config 2
 ])
 def test_i8_gemm_bit_exact(hip, m, n, k):
