@@ -323,16 +323,21 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     // neighbouring row or, past the end of the buffer, zero, and are never stored.
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint32_t*>(qweight), 0, (int)((size_t)(K / P) * N * 4), kBufferRsrcFlags);
-    auto load_q = [&](int tile, int step, uint4_t* dst) {
-        const int s = min(step, last_step);  // the last stage's refills run on into the range that follows
+    // The ring is refilled at a fixed place of the loop body, also in the range's last
+    // stage, where nothing is left to fetch: those loads go through a descriptor of
+    // zero records, so they return zero without touching memory.
+    const __amdgpu_buffer_rsrc_t q_none =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qweight), 0, 0, kBufferRsrcFlags);
+    auto load_q = [&](const __amdgpu_buffer_rsrc_t& rsrc, int tile, int step, uint4_t* dst) {
+        const int s = min(step, last_step);
         const int soff = (s * ROWS_PER_STEP * N + tile * kGemmCols) * 4;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j)
             dst[j] = __builtin_bit_cast(
-                uint4_t, __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (int)lane_off[j], soff, kBufferStreamAgent));
+                uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off[j], soff, kBufferStreamAgent));
     };
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_q(t0, s0 * D + d, qb[d]);
+    for (int d = 0; d < D; ++d) load_q(q_rsrc, t0, s0 * D + d, qb[d]);
 
     // ---- staging of activations and constants: global -> registers -> LDS
     uint4 xr[XL];
@@ -469,6 +474,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     for (int stage = 0; stage < n_stages; ++stage) {
         const int buf = stage & 1;
         const int next_tile = tile_of(stage + 1), next_step = step_of(stage + 1);
+        const __amdgpu_buffer_rsrc_t next_rsrc = stage + 1 < n_stages ? q_rsrc : q_none;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             if (d % SPG == 0) {  // compile-time: a new group starts here
@@ -492,7 +498,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 const uint4_t packed = {as_u32(w[0]), as_u32(w[1]), as_u32(w[2]), as_u32(w[3])};
                 b[t] = __builtin_bit_cast(half8_t, packed);
             }
-            load_q(next_tile, next_step + d, q);
+            load_q(next_rsrc, next_tile, next_step + d, q);
             __builtin_amdgcn_sched_barrier(0);  // keep the reload here (see above)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {

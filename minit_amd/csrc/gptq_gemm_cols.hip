@@ -81,6 +81,7 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     const int end = min(begin + steps_per_wave, steps_total);
     const int last_step = steps_total - 1;
     const int last_stage_step = (last_step / kColsStage) * kColsStage;
+    const int ring_last = max(min(end, steps_total) - 1, 0);
 
     // ---- packed weights
     uint2_t qb[R][LOADS];
@@ -92,7 +93,9 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     const __amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint32_t*>(qweight), 0, (int)((size_t)(K / P) * N * 4), kBufferRsrcFlags);
     auto load_q = [&](int step, uint2_t* dst) {
-        const int s = min(step, last_step);  // past the end of K: re-read the last step, its activations are zero
+        // past the end of the wave's range: re-read its last step (a cache hit; running on
+        // into the next wave's range measured 10 % more HBM traffic), its activations are zero
+        const int s = min(step, ring_last);
         const int soff = s * ROWS_PER_STEP * N * 4;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j)
