@@ -30,13 +30,14 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of the dominant kernel on this workload, measured with two
+# HBM bytes per launch (mean over the four launches of a step, which run the
+# library's two MFMA GPTQ kernels) on this workload, measured with two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, in KiB per
 # dispatch, scaled by what the same counters read for the 1 GiB copy kernel of
 # --calibrate-copy: x2.000 and x1.000); the summary with the commands is kept
 # under profiles/.  A counter cannot be read from inside this process, so the
 # figure is carried here and is only reported for the entry point it was taken on.
-MEASURED_TRAFFIC = {"mh_gptq_matmul": 115_688_243}
+MEASURED_TRAFFIC = {"mh_gptq_matmul": 115_765_709}
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0
 
@@ -263,7 +264,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gptq_gemv_kernel<4,1,8>" if ENTRY == "mh_gptq_gemv" else "gptq_gemm_small_kernel<4,1,4>",
+            "kernel": "gptq_gemv_kernel<4,1,8>" if ENTRY == "mh_gptq_gemv" else "gptq_gemm_small_kernel<4,1,4> (qkv, gate_up) + gptq_gemm_cols_kernel<4,4,1> (o, down)",
             "entry": ENTRY,
             "achieved": round(gbps, 1),
             "peak": HBM_PEAK_GBPS,
