@@ -103,7 +103,9 @@ int mh_gptq_dequant(mh_stream_t stream, const int32_t* qweight, const int32_t* q
  * are ordered on one stream, never by concurrent calls.
  *
  * mh_gptq_gemv   wave64 VALU path, no MFMA; M <= MH_GPTQ_GEMV_MAX_M.
- * mh_gptq_gemm   fp16 MFMA path; any M >= 1.
+ * mh_gptq_gemm   fp16 MFMA path; any M >= 1; the packed weights of one matrix
+ *                (K * N * bits / 8 bytes) must stay below 2 GiB, the kernels
+ *                address them with 32-bit buffer offsets.
  * mh_gptq_matmul picks one of the two (or the act-order path when g_idx is a
  *                non-trivial permutation).
  */
