@@ -214,6 +214,12 @@ int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, si
 int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
                 size_t n, int exact, int dtype);
 
+/* The bias of a quantized linear (QLinearWithBias.forward,
+ * examples/qwen1_5_int8.py:311-317: the product, then `output += bias` with the
+ * bias broadcast over the leading axes): x[r, c] = T(x[r, c] + bias[c]) in
+ * place, one rounding in the storage type like the reference's Add kernel. */
+int mh_add_bias(mh_stream_t stream, void* x, const void* bias, size_t rows, size_t cols, int dtype);
+
 /* ---- Llama-family GPTQ decode loop ------------------------------------------------------
  * The callers around the quantized linears: one greedy decode step per token as
  * the reference's models run it (examples/llama3_70b.py:77-162,215-249;

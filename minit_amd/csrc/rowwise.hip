@@ -372,6 +372,18 @@ static int reduce_t(hipStream_t st, const void* in, void* out, size_t a, size_t 
 
 using namespace mh;
 
+// x[r, c] = T(x[r, c] + bias[c]) in place: the broadcast add that follows the
+// quantized product in a linear with bias (examples/qwen1_5_int8.py:311-317), one
+// rounding in the storage type like the reference's element-wise Add.
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const T* __restrict__ bias, size_t rows, size_t cols) {
+    const size_t n = rows * cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const T sum = Cvt<T>::from_f32(Cvt<T>::to_f32(x[i]) + Cvt<T>::to_f32(bias[i % cols]));
+        x[i] = sum;
+    }
+}
+
 #define MH_DISPATCH_DTYPE(dtype, who, CALL)                                         \
     switch (dtype) {                                                                \
         case MH_F16: { typedef half_t T; CALL; }                                    \
@@ -464,6 +476,19 @@ int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
     return MH_OK;
     MH_DISPATCH_DTYPE(dtype, "mh_silu_mul", MH_SILU_CALL);
 #undef MH_SILU_CALL
+}
+
+int mh_add_bias(mh_stream_t stream, void* x, const void* bias, size_t rows, size_t cols, int dtype) {
+    if (rows * cols == 0) return MH_OK;
+    MH_REQUIRE(x && bias, "mh_add_bias: null pointer");
+    hipStream_t st = as_stream(stream);
+    const unsigned grid = grid_for(rows * cols, 256);
+#define MH_BIAS_CALL                                                                                          \
+    hipLaunchKernelGGL(add_bias_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)x, (const T*)bias, rows, cols); \
+    MH_CHECK_LAUNCH();                                                                                        \
+    return MH_OK;
+    MH_DISPATCH_DTYPE(dtype, "mh_add_bias", MH_BIAS_CALL);
+#undef MH_BIAS_CALL
 }
 
 }  // extern "C"

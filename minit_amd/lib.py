@@ -60,6 +60,7 @@ PROTOTYPES = {
     "mh_sum": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_max": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
+    "mh_add_bias": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_int]),
     "mh_llama_create": (c_int, [POINTER(c_void_p), _P]),
     "mh_llama_destroy": (c_int, [_P]),
     "mh_llama_set_layer": (c_int, [_P, c_int, _P]),
