@@ -147,3 +147,33 @@ def test_llama70b_linear_zero_point_weights_give_zero(hip, name, k, n):
     hip.call("mh_synth_normal", None, x.data_ptr, 4 * k, 0.0, 1.0, 0, 0.0, 5, 0)
     got = _linear(hip, x, lin.qweight, lin.qzeros, lin.scales, 4, n, k).numpy()
     assert not got.any(), f"{name}: {np.count_nonzero(got)} non-zero outputs"
+
+
+@pytest.mark.parametrize("m", [1, 5])
+def test_eight_bit_gate_up_shape_one_hot_rows(hip, m):
+    """8-bit weights at the gate|up shape: the balanced plan of the small-M kernel
+    (a workgroup finishes one tile and begins the next) with two packed rows per
+    8 k; one-hot rows return rows of the dequantized matrix bit for bit."""
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    k, n, bits = 8192, 57344, 8
+    per, groups = 32 // bits, k // GROUP
+    qweight = HIPTensor.allocate((k // per, n), "int32")
+    qzeros = HIPTensor.allocate((groups, n // per), "int32")
+    scales = HIPTensor.allocate((groups, n), "float16")
+    hip.call("mh_synth_u32", None, qweight.data_ptr, (k // per) * n, 97)
+    hip.call("mh_synth_subwords", None, qzeros.data_ptr, groups * (n // per), bits, 0, 255, 98)
+    hip.call("mh_synth_normal", None, scales.data_ptr, groups * n, 0.0, 0.02, 1, 1e-3, 99, 0)
+    rows = np.random.default_rng(m).choice(k, size=m, replace=False)
+    rows[0] = k - 1
+    x = np.zeros((m, k), dtype=np.float16)
+    x[np.arange(m), rows] = 1.0
+    dx = _dev(x)
+    out = HIPTensor.allocate((m, n), "float16")
+    ws = memory.workspace(max(hip.call("mh_gptq_workspace_bytes", m, n, k, GROUP, bits), 256))
+    hip.call("mh_gptq_matmul", None, dx.data_ptr, qweight.data_ptr, qzeros.data_ptr, scales.data_ptr, None,
+             out.data_ptr, m, n, k, GROUP, bits, ws._pointer, ws._size)
+    w = HIPTensor.allocate((k, n), "float16")
+    hip.call("mh_gptq_dequant", None, qweight.data_ptr, qzeros.data_ptr, scales.data_ptr, None, w.data_ptr, n, k,
+             GROUP, bits)
+    np.testing.assert_array_equal(out.numpy().view(np.uint16), w.numpy()[rows].view(np.uint16))
