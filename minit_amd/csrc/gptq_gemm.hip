@@ -681,9 +681,10 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 
 // gptq_gemm_cols.hip
 bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epilogue);
+size_t gemm_cols_workspace_bytes(int M, int N, int K);
 int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                           const void* scales, void* out, int M, int N, int K, int group_size, int bits, int epilogue,
-                          const SmallFuse& fuse);
+                          const SmallFuse& fuse, void* workspace, size_t workspace_bytes);
 
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
@@ -803,7 +804,9 @@ bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits) {
 // (per 1024 columns, so N must be a multiple of that).
 bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
     if (!gemm_supported(M, N, K, group_size, bits) || !use_small(M, group_size)) return false;
-    if (epilogue == kEpilogueResidual && gemm_cols_preferred(M, N, K, group_size, bits, epilogue)) return true;
+    if ((epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
+        gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
+        return true;
     if (M <= kFusedReduceMaxM) return N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
     return N % (epilogue == kEpilogueResidual ? 1024 : kGemmCols) == 0;
 }
@@ -824,7 +827,9 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     const int slots = p.split_k > pb.split_k ? p.split_k : pb.split_k;
     // the small-M kernel may be asked for an epilogue that goes through the partials even unsplit
     if (slots <= 1 && !use_small(M, group_size)) return 0;
-    return kTileCounterBytes + (size_t)slots * M * N * sizeof(float);
+    const size_t small = kTileCounterBytes + (size_t)slots * M * N * sizeof(float);
+    const size_t cols = M <= kFusedReduceMaxM ? gemm_cols_workspace_bytes(M, N, K) : 0;
+    return small > cols ? small : cols;
 }
 
 template <int BITS, int MT>
@@ -905,8 +910,9 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     if ((size_t)K * N * bits / 8 >= ((size_t)1 << 31))
         return fail(MH_ERR_INVALID, "gptq gemm: packed weights of 2 GiB or more are not supported");
     // a narrow output goes to the kernel whose workgroups own their columns over all of K
-    if (fuse.ssq_in == nullptr && gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
-        return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse);
+    if (gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
+        return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse,
+                                     workspace, workspace_bytes);
     if (row_blocked(M, group_size)) {
         // Above kSmallMaxM rows the product is taken 32 rows at a time by the small-M
         // kernel: the packed weights are re-read per block of rows (from the

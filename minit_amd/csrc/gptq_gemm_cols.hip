@@ -25,9 +25,10 @@
 //
 // Measured against the small-M kernel (M = 1, us): 8192x8192 9.8 / 15.3,
 // 4096x4096 5.8 / 9.1, 16384x8192 15.7 / 22.3, 28672x8192 24.5 / 26.2 (at 8 rows
-// 29.8 / 28.2); with more 32-column tiles than CUs (10240 columns: 15.9 / 15.0) or
-// half the CUs idle on a long K (14336x4096: 16.6 / 14.8) it loses, see
-// gemm_cols_preferred.
+// 29.8 / 28.2).  With more 32-column tiles than CUs it loses when the extra tiles
+// make a second round (10240 columns: 15.9 / 15.0) and gains a little when they
+// are cut along K instead (14.1 / 15.0, see the kernel); with half the CUs idle
+// on a long K (14336x4096: 16.6 / 14.8) it loses.  gemm_cols_preferred decides.
 #include "gptq_common.h"
 
 namespace mh {
@@ -53,8 +54,9 @@ __device__ __forceinline__ ColumnConst column_const_from_bits(uint32_t sbits, ui
 template <int BITS, int SPG, int MROWS>
 __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
-    const half_t* __restrict__ scales, half_t* out, int M, int N, int K, int steps_total, int steps_per_wave,
-    int epilogue, SmallFuse fuse) {
+    const half_t* __restrict__ scales, half_t* out, float* partial, unsigned* counters, int M, int N, int K,
+    int steps_total, int steps_per_wave, int full_tiles, int parts, int part_steps_per_wave, int epilogue,
+    SmallFuse fuse) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
     constexpr uint32_t MASK = Packing<BITS>::kMask;
@@ -69,15 +71,29 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
 
     __shared__ uint4 xs[kColsWaves][MROWS * RS];
     __shared__ float red[kColsWaves][MROWS][kColsTile];
+    __shared__ float inv_rms_s[MROWS];
+    __shared__ int is_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 15, kq = lane >> 4;
-    const int tile = blockIdx.x;
+    // Workgroups 0 .. full_tiles - 1 own a tile over all of K.  Where there are a few
+    // more tiles than CUs, the remaining tiles are cut into `parts` K ranges, one
+    // workgroup each, so that every CU gets one whole tile and at most one part; the
+    // parts' sums cross workgroups (see the results section), which ends long
+    // before the whole tiles are through.
+    int tile = blockIdx.x, part = 0, nparts = 1;
+    if (tile >= full_tiles) {
+        const int s = tile - full_tiles;
+        tile = full_tiles + s / parts;
+        part = s % parts;
+        nparts = parts;
+        steps_per_wave = part_steps_per_wave;
+    }
     const int col0 = tile * kColsTile + nl * 2;
 
-    const int begin = wave * steps_per_wave;
+    const int begin = (part * kColsWaves + wave) * steps_per_wave;
     const int end = min(begin + steps_per_wave, steps_total);
     const int last_step = steps_total - 1;
     const int last_stage_step = (last_step / kColsStage) * kColsStage;
@@ -153,6 +169,18 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
         load_q(begin + d, qb[d]);
     }
 
+    if (fuse.ssq_in != nullptr) {
+        // 1 / rms of the rows from the producer's sums of squares (see SmallFuse): 32
+        // lanes per row, folded by shuffles in a fixed order; read after the K loop
+        const int row = tid >> 5, p0 = tid & 31;
+        float ss = 0.f;
+        if (row < M)
+            for (int t = p0; t < fuse.ssq_tiles; t += 32) ss += fuse.ssq_in[(size_t)row * fuse.ssq_tiles + t];
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
+        if (p0 == 0 && row < MROWS) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+    }
+
     DequantRegs regs;
     regs.init(BITS);
     float4_t acc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
@@ -200,16 +228,43 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
         if (m < M) *reinterpret_cast<float2*>(&red[wave][m][nl * 2]) = make_float2(acc[0][r], acc[1][r]);
     }
     __syncthreads();
-    if (tid >= M * (kColsTile / 2)) return;
+    const bool worker = tid < M * (kColsTile / 2);  // one thread per (row, column pair)
     const int m = tid / (kColsTile / 2), c = tid % (kColsTile / 2) * 2;
-    float2 sum = make_float2(0.f, 0.f);
-#pragma unroll
-    for (int w = 0; w < kColsWaves; ++w) {
-        const float2 v = *reinterpret_cast<const float2*>(&red[w][m][c]);
-        sum.x += v.x;
-        sum.y += v.y;
-    }
     const int col = tile * kColsTile + c;
+    float2 sum = make_float2(0.f, 0.f);
+    if (worker) {
+#pragma unroll
+        for (int w = 0; w < kColsWaves; ++w) {
+            const float2 v = *reinterpret_cast<const float2*>(&red[w][m][c]);
+            sum.x += v.x;
+            sum.y += v.y;
+        }
+    }
+    if (nparts > 1) {
+        // a tile cut along K: publish, count in, and the workgroup that arrives last
+        // adds the parts in part order (common.h:arrive_and_check_last)
+        const size_t plane = (size_t)M * N;
+        if (worker) {
+            float* dst = partial + (size_t)part * plane + (size_t)m * N + col;
+            store_agent(dst, sum.x);
+            store_agent(dst + 1, sum.y);
+        }
+        if (!arrive_and_check_last(&counters[tile], (unsigned)nparts, &is_last)) return;
+        if (worker) {
+            sum = make_float2(0.f, 0.f);
+            for (int p = 0; p < nparts; ++p) {
+                const float* src = partial + (size_t)p * plane + (size_t)m * N + col;
+                sum.x += load_agent(src);
+                sum.y += load_agent(src + 1);
+            }
+        }
+    }
+    if (!worker) return;
+    if (fuse.ssq_in != nullptr) {
+        const float inv = inv_rms_s[m];
+        sum.x *= inv;
+        sum.y *= inv;
+    }
     const half2_t y = {(half_t)sum.x, (half_t)sum.y};
     half2_t* op = reinterpret_cast<half2_t*>(out + (size_t)m * N + col);
     if (epilogue == kEpilogueResidual) {
@@ -224,45 +279,97 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
         float ss = (float)h[0] * (float)h[0] + (float)h[1] * (float)h[1];
 #pragma unroll
         for (int off = 1; off < kColsTile / 2; off <<= 1) ss += __shfl_xor(ss, off);
-        if (c == 0) fuse.ssq_out[(size_t)m * gridDim.x + tile] = ss;
+        if (c == 0) fuse.ssq_out[(size_t)m * (N / kColsTile) + tile] = ss;
+        return;
+    }
+    if (epilogue == kEpilogueRopeAppend) {
+        // the two columns are one interleaved pair of a head of 128 dims (gptq_common.h)
+        const int head = col / 128, d = col % 128;
+        const int pos = fuse.positions[m];
+        if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
+            half_t* dst = fuse.vt_cache +
+                          (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;
+            dst[0] = y[0];
+            dst[fuse.max_seq] = y[1];
+            return;
+        }
+        const float cs = fuse.rope_cos[(size_t)pos * 64 + d / 2], sn = fuse.rope_sin[(size_t)pos * 64 + d / 2];
+        const float re = (float)y[0], im = (float)y[1];
+        const half2_t o = {(half_t)(re * cs - im * sn), (half_t)(im * cs + re * sn)};
+        half_t* dst = head < fuse.q_heads
+                          ? fuse.q_out + ((size_t)m * fuse.q_heads + head) * 128 + d
+                          : fuse.k_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads)) * fuse.max_seq + pos) * 128 + d;
+        *reinterpret_cast<half2_t*>(dst) = o;
         return;
     }
     *op = y;
 }
+
+constexpr int kColsParts = 4;  // K ranges of a tile that is cut, when there are more tiles than CUs
 
 bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_COLS");
     if (off && *off && atoi(off)) return false;
     if (bits != 4 || group_size != 128 || M < 1 || M > 8) return false;
     if (N % kColsTile != 0 || K % (32 * kColsStage) != 0) return false;
-    return epilogue == kEpilogueNone || epilogue == kEpilogueResidual;
+    return epilogue == kEpilogueNone || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend;
+}
+
+// Tiles beyond one per CU are cut into kColsParts K ranges, which must not outnumber the CUs.
+static bool cols_cut_plan(int tiles, int K, int cus) {
+    return tiles > cus && (tiles - cus) * kColsParts <= cus && tiles - cus < kMaxTileCounters &&
+           K % (32 * kColsStage * kColsWaves * kColsParts) == 0;
 }
 
 // Where it measured faster than the small-M kernel: every CU gets at most one
-// 32-column tile, and either the tiles cover more than half the CUs or K is short
-// enough for the kernel to be bound by its dependent round trips rather than by
-// the CUs left idle.
+// 32-column tile (plus at most one K range of a cut tile), and either the tiles
+// cover more than half the CUs or K is short enough for the kernel to be bound by
+// its dependent round trips rather than by the CUs left idle.
 bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
     if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue)) return false;
     static const char* force = getenv("MH_GEMM_COLS_FORCE");
     if (force && *force && atoi(force)) return true;
     const int tiles = N / kColsTile, cus = compute_units();
+    static const char* nocut = getenv("MH_GEMM_COLS_NO_CUT");
+    // measured at 8192x10240 (320 tiles on 256 CUs): 14.1 against 15.0 us at M = 1, no gain at M = 8
+    if (cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut))) return K <= 8192 && M <= 2;
     return tiles <= cus && (K <= 8192 || 2 * tiles > cus) && (K <= 16384 || M <= 2);
+}
+
+// Bytes of workspace a launch of this kernel needs for the shape (0: none).
+size_t gemm_cols_workspace_bytes(int M, int N, int K) {
+    return cols_cut_plan(N / kColsTile, K, compute_units()) ? kTileCounterBytes + (size_t)kColsParts * M * N * sizeof(float)
+                                                            : 0;
 }
 
 int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                           const void* scales, void* out, int M, int N, int K, int group_size, int bits, int epilogue,
-                          const SmallFuse& fuse) {
-    if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue) || fuse.ssq_in != nullptr)
+                          const SmallFuse& fuse, void* workspace, size_t workspace_bytes) {
+    if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue))
         return fail(MH_ERR_INVALID, "gptq column-owner kernel: unsupported shape or fusion");
     const int steps_total = K / 32;
     int spw = (steps_total + kColsWaves - 1) / kColsWaves;
     spw = (spw + kColsStage - 1) / kColsStage * kColsStage;  // whole stages, hence whole groups
-    const dim3 grid(N / kColsTile);
+    const int tiles = N / kColsTile, cus = compute_units();
+    int full_tiles = tiles, parts = 1, part_spw = spw;
+    float* partial = nullptr;
+    unsigned* counters = nullptr;
+    if (cols_cut_plan(tiles, K, cus)) {
+        const size_t need = gemm_cols_workspace_bytes(M, N, K);
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
+                        workspace ? workspace_bytes : (size_t)0);
+        full_tiles = cus;
+        parts = kColsParts;
+        part_spw = steps_total / (kColsWaves * kColsParts);
+        counters = reinterpret_cast<unsigned*>(workspace);
+        partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
+    }
+    const dim3 grid(full_tiles + (tiles - full_tiles) * parts);
 #define MH_LAUNCH_COLS(MROWS)                                                                                     \
     hipLaunchKernelGGL((gptq_gemm_cols_kernel<4, 4, MROWS>), grid, dim3(512), 0, stream, (const half_t*)x,         \
-                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out, M, \
-                       N, K, steps_total, spw, epilogue, fuse)
+                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,    \
+                       partial, counters, M, N, K, steps_total, spw, full_tiles, parts, part_spw, epilogue, fuse)
     if (M == 1)
         MH_LAUNCH_COLS(1);
     else if (M == 2)
