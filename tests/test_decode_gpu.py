@@ -130,3 +130,45 @@ def test_attention_split_kv_consistency(hip):
     ref = OD.decode_step(model, tokens, positions, [k_cache[0].copy()], [v_cache[0].copy()])
     g, r = got.astype(np.float64), ref.astype(np.float64)
     assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+
+
+def test_decode_wide_qkv_on_cut_tiles(hip):
+    """The 70B projection widths (q|k|v 8192 -> 10240: 320 column tiles of 32 on 256
+    CUs, at most two rows): the fused q|k|v product then runs on the column-owner
+    kernel with the tiles beyond one per CU cut along K, its norm prologue and
+    RoPE/cache-append epilogue, and o on the same kernel with the residual epilogue.
+    Two layers, so that the second one consumes the first one's sums of squares."""
+    from minit_amd.decode import LlamaDecoder
+    cfg = dict(CFG, n_layers=2, hidden=8192, n_q_heads=64, n_kv_heads=8, ffn=256, vocab=256)
+    batch, context, max_seq = 2, 10, 64
+    model = _host_model(cfg, seed=21)
+    # sums over 8192 terms: keep the projections around unit size, or the fp16 scores of the
+    # reference's attention (q . k before the 1/sqrt(d) scale) overflow
+    for layer in model["layers"]:
+        for name in ("qkv", "o", "gate_up", "down"):
+            qw, qz, sc, g = layer[name]
+            layer[name] = (qw, qz, (sc.astype(np.float32) / 16).astype(np.float16), g)
+    rng = np.random.default_rng(22)
+    shape = (batch, cfg["n_kv_heads"], max_seq, 128)
+    k_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    v_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    for c in k_cache + v_cache:
+        c[:, :, :context] = rng.normal(0, 1, (batch, cfg["n_kv_heads"], context, 128))
+    tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
+    positions = np.asarray([context, context - 3], np.int32)
+    dec = LlamaDecoder(cfg, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+    _, got = dec.decode(tokens, positions, 1, want_logits=True)
+    ref_k, ref_v = [c.copy() for c in k_cache], [c.copy() for c in v_cache]
+    ref = OD.decode_step(model, tokens, positions, ref_k, ref_v)
+    g, r = got.astype(np.float64), ref.astype(np.float64)
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+    assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
+    # the appended keys and values of both layers, each row at its own position
+    for layer in range(cfg["n_layers"]):
+        kc, vc = dec.k_cache[layer].numpy(), dec.v_cache[layer].numpy()  # V is kept [B, KVH, D, T]
+        for b in range(batch):
+            p = int(positions[b])
+            tol = 2e-2 if layer == 0 else 6e-2  # layer 1 sees layer 0's rounding differences
+            assert np.abs(kc[b, :, p].astype(np.float64) - ref_k[layer][b, :, p].astype(np.float64)).max() <= tol
+            assert np.abs(vc[b, :, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max() <= tol
