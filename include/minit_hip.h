@@ -265,6 +265,16 @@ size_t mh_llama_scratch_bytes(void* handle, int batch);
  * receives the last step's fp16 logits [batch, vocab]. */
 int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
                     int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes);
+/* The same, with one step recorded into a HIP graph on first use and replayed
+ * n_steps times (the reference's hook for replaying a recorded operator sequence
+ * is minit/trace/executor.py:49-119, which still dispatches and allocates per
+ * operator; here a step has no host work at all).  Same arguments and results;
+ * `stream` must be a created stream (the null stream cannot record).  The
+ * recorded step is kept in the handle, keyed by (batch, tokens, positions,
+ * out_tokens, scratch), until the model's pointers are set again or it is
+ * destroyed; those buffers must stay allocated while it is kept. */
+int mh_llama_decode_graph(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
+                          int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes);
 
 /* ---- synthetic inputs ------------------------------------------------------------------
  * No counterpart in the reference (it loads checkpoints from disk,

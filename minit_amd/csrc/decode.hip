@@ -154,11 +154,15 @@ __global__ void silu_mul_fused_kernel(const half_t* __restrict__ gu, half_t* __r
 }
 
 // token[b] = argmax_v logits[b, v] (first maximum); appended to the output
-// stream and fed back as the next input; positions[b] += 1.
+// stream and fed back as the next input; positions[b] += 1.  out_tokens points
+// at this step's row of the output, or, when pos_base is given, at the whole
+// [steps, batch] output and the row is positions[b] - pos_base[b]: the same
+// launch, replayed, then fills one row after the other.
 __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __restrict__ logits,
                                                               int32_t* __restrict__ tokens,
                                                               int32_t* __restrict__ out_tokens,
-                                                              int32_t* __restrict__ positions, int vocab) {
+                                                              int32_t* __restrict__ positions,
+                                                              const int32_t* __restrict__ pos_base, int vocab) {
     __shared__ float sval[16];
     __shared__ int sidx[16];
     const int b = blockIdx.x;
@@ -196,8 +200,9 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
         for (int w = 1; w < (int)(blockDim.x >> 6); ++w) consider(sval[w], sidx[w]);
         const int tok = best_i == 0x7fffffff ? 0 : best_i;
         tokens[b] = tok;
-        if (out_tokens) out_tokens[b] = tok;
-        positions[b] += 1;
+        const int pos = positions[b];
+        if (out_tokens) out_tokens[pos_base ? (size_t)(pos - pos_base[b]) * gridDim.x + b : (size_t)b] = tok;
+        positions[b] = pos + 1;
     }
 }
 
@@ -439,12 +444,24 @@ struct Llama {
     const void* final_norm = nullptr;
     const float* cos = nullptr;
     const float* sin = nullptr;
+    // one recorded decode step per set of buffers it was recorded on
+    struct StepGraph {
+        int batch;
+        const void *tokens, *positions, *out_tokens, *scratch;
+        hipGraphExec_t exec;
+    };
+    std::vector<StepGraph> graphs;
+    void drop_graphs() {
+        for (auto& g : graphs) (void)hipGraphExecDestroy(g.exec);
+        graphs.clear();
+    }
 };
 
 struct Scratch {
     half_t *h, *xn, *qkv, *q, *attn, *delta, *gu, *act, *logits;
     float* attn_partial;
     float *ssq_a, *ssq_b;  // per-piece sums of squares of the residual stream, [batch, at most hidden / 32]
+    int32_t* pos_base;     // positions at the start of a call that replays a recorded step
     unsigned* attn_counters;
     void* gptq_ws;
     size_t gptq_ws_bytes;
@@ -496,6 +513,7 @@ static Scratch carve(const Llama& m, int batch, char* base) {
     s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 4) * 4);
     s.ssq_a = (float*)take((size_t)batch * ((c.hidden + 31) / 32) * 4);
     s.ssq_b = (float*)take((size_t)batch * ((c.hidden + 31) / 32) * 4);
+    s.pos_base = (int32_t*)take((size_t)batch * sizeof(int32_t));
     s.total = off;
     return s;
 }
@@ -536,7 +554,9 @@ int mh_llama_create(void** handle, const mh_llama_config* cfg) {
 }
 
 int mh_llama_destroy(void* handle) {
-    delete reinterpret_cast<Llama*>(handle);
+    Llama* m = reinterpret_cast<Llama*>(handle);
+    if (m) m->drop_graphs();
+    delete m;
     return MH_OK;
 }
 
@@ -545,6 +565,7 @@ int mh_llama_set_layer(void* handle, int layer, const mh_llama_layer* l) {
     MH_REQUIRE(m && l, "mh_llama_set_layer: null argument");
     MH_REQUIRE(layer >= 0 && layer < m->cfg.n_layers, "mh_llama_set_layer: layer %d out of range", layer);
     m->layers[layer] = *l;
+    m->drop_graphs();  // recorded steps hold the old pointers
     return MH_OK;
 }
 
@@ -557,6 +578,7 @@ int mh_llama_set_globals(void* handle, const void* embed, const void* lm_head, c
     m->final_norm = final_norm;
     m->cos = freqs_cos;
     m->sin = freqs_sin;
+    m->drop_graphs();
     return MH_OK;
 }
 
@@ -566,8 +588,14 @@ size_t mh_llama_scratch_bytes(void* handle, int batch) {
     return carve(*m, batch, nullptr).total;
 }
 
-int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
-                    int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes) {
+}  // extern "C"
+
+// One decode step is the same sequence of launches on the same buffers for every
+// token (the position and the token travel in device memory), so it can be
+// recorded once into a HIP graph and replayed: `replay` does that, keeping the
+// recorded step in the model for later calls on the same buffers.
+static int decode_impl(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions, int n_steps,
+                       int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes, bool replay) {
     Llama* m = reinterpret_cast<Llama*>(handle);
     MH_REQUIRE(m != nullptr, "mh_llama_decode: null handle");
     MH_REQUIRE(batch > 0 && n_steps >= 0, "mh_llama_decode: bad batch / steps");
@@ -609,7 +637,8 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                                  s.gptq_ws, s.gptq_ws_bytes, epilogue, fuse);
     };
 
-    for (int step = 0; step < n_steps; ++step) {
+    // every launch of one step; out_row / pos_base as for argmax_advance_kernel
+    auto enqueue_step = [&](int32_t* out_row, const int32_t* pos_base) -> int {
         hipLaunchKernelGGL(embed_gather_kernel, dim3(batch), dim3(256), 0, st, tokens, (const half_t*)m->embed, s.h,
                            c.hidden, c.vocab);
         hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, (const half_t*)nullptr,
@@ -695,13 +724,60 @@ int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens
                                (const half_t*)m->final_norm, s.xn, c.hidden, c.rms_eps);
         int rc = mh_f16_matmul_nk(stream, s.xn, m->lm_head, s.logits, batch, c.vocab, c.hidden);
         if (rc) return rc;
-        hipLaunchKernelGGL(argmax_advance_kernel, dim3(batch), dim3(1024), 0, st, s.logits, tokens,
-                           out_tokens ? out_tokens + (size_t)step * batch : nullptr, positions, c.vocab);
+        hipLaunchKernelGGL(argmax_advance_kernel, dim3(batch), dim3(1024), 0, st, s.logits, tokens, out_row, positions,
+                           pos_base, c.vocab);
         MH_CHECK_LAUNCH();
+        return MH_OK;
+    };
+
+    if (!replay) {
+        for (int step = 0; step < n_steps; ++step) {
+            const int rc = enqueue_step(out_tokens ? out_tokens + (size_t)step * batch : nullptr, nullptr);
+            if (rc) return rc;
+        }
+    } else if (n_steps > 0) {
+        MH_REQUIRE(st != nullptr, "mh_llama_decode_graph: needs a stream of its own (the null stream cannot record)");
+        hipGraphExec_t exec = nullptr;
+        for (const auto& g : m->graphs)
+            if (g.batch == batch && g.tokens == tokens && g.positions == positions && g.out_tokens == out_tokens &&
+                g.scratch == scratch)
+                exec = g.exec;
+        if (exec == nullptr) {
+            MH_CHECK_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+            const int rc = enqueue_step(out_tokens, s.pos_base);
+            hipGraph_t graph = nullptr;
+            const hipError_t end = hipStreamEndCapture(st, &graph);  // also leaves capture mode after a failed step
+            if (rc) {
+                if (graph) (void)hipGraphDestroy(graph);
+                return rc;
+            }
+            MH_CHECK_HIP(end);
+            const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(graph);
+            MH_CHECK_HIP(inst);
+            m->graphs.push_back({batch, tokens, positions, out_tokens, scratch, exec});
+        }
+        // row r of the output belongs to the step that starts at pos_base + r
+        MH_CHECK_HIP(hipMemcpyAsync(s.pos_base, positions, (size_t)batch * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+        for (int step = 0; step < n_steps; ++step) MH_CHECK_HIP(hipGraphLaunch(exec, st));
     }
     if (logits_out && n_steps > 0)
         MH_CHECK_HIP(hipMemcpyAsync(logits_out, s.logits, (size_t)batch * c.vocab * 2, hipMemcpyDeviceToDevice, st));
     return MH_OK;
+}
+
+extern "C" {
+
+int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
+                    int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes) {
+    return decode_impl(handle, stream, batch, tokens, positions, n_steps, out_tokens, logits_out, scratch,
+                       scratch_bytes, false);
+}
+
+int mh_llama_decode_graph(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
+                          int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes) {
+    return decode_impl(handle, stream, batch, tokens, positions, n_steps, out_tokens, logits_out, scratch,
+                       scratch_bytes, true);
 }
 
 }  // extern "C"

@@ -72,6 +72,8 @@ class LlamaDecoder:
         self._keep = []          # device tensors referenced by the native model
         self.k_cache, self.v_cache = [], []
         self._scratch = {}
+        self._graph_io = {}      # batch -> (tokens, positions, out_tokens) a recorded step is bound to
+        self._graph_stream = None
         cos, sin = synthetic.rope_tables(c["head_dim"], max_seq, c["rope_theta"])
         self.cos, self.sin = HIPTensor.from_numpy(cos), HIPTensor.from_numpy(sin)
 
@@ -184,22 +186,39 @@ class LlamaDecoder:
             self._scratch[batch] = mem
         return self._scratch[batch]
 
-    def decode(self, tokens, positions, n_steps: int, want_logits: bool = False, stream=None):
+    def decode(self, tokens, positions, n_steps: int, want_logits: bool = False, stream=None, graph: bool = False):
         """Greedy-decodes ``n_steps`` tokens for ``len(tokens)`` rows.
 
+        With ``graph`` one step is recorded into a HIP graph the first time a batch
+        size is seen and replayed per token (``mh_llama_decode_graph``), on a stream
+        and on token / position / output buffers the decoder keeps for that batch size.
         Returns ``(out_tokens [n_steps, B] int32, logits of the last step or None)``.
         """
         batch = len(tokens)
         assert batch <= self.batch_max
         assert int(np.max(positions)) + n_steps <= self.max_seq, "KV cache too short"
-        tok = HIPTensor.from_numpy(np.asarray(tokens, np.int32))
-        pos = HIPTensor.from_numpy(np.asarray(positions, np.int32))
-        out = HIPTensor.allocate((n_steps, batch), "int32")
         logits = HIPTensor.allocate((batch, self.config["vocab"]), "float16") if want_logits else None
         scratch = self._scratch_for(batch)
-        lib.call("mh_llama_decode", self._handle, stream, batch, tok.data_ptr, pos.data_ptr, n_steps,
-                 out.data_ptr, logits.data_ptr if logits else None, scratch._pointer, scratch._size)
-        result = out.numpy()
+        if graph:
+            if batch not in self._graph_io:
+                self._graph_io[batch] = (HIPTensor.allocate((batch,), "int32"), HIPTensor.allocate((batch,), "int32"),
+                                         HIPTensor.allocate((self.max_seq, batch), "int32"))
+            if self._graph_stream is None:
+                self._graph_stream = memory.create_stream()
+            tok, pos, out = self._graph_io[batch]
+            tok.copy_from_numpy(np.asarray(tokens, np.int32))
+            pos.copy_from_numpy(np.asarray(positions, np.int32))
+            lib.call("mh_llama_decode_graph", self._handle, stream or self._graph_stream, batch, tok.data_ptr,
+                     pos.data_ptr, n_steps, out.data_ptr, logits.data_ptr if logits else None, scratch._pointer,
+                     scratch._size)
+            result = out.numpy()[:n_steps].copy()
+        else:
+            tok = HIPTensor.from_numpy(np.asarray(tokens, np.int32))
+            pos = HIPTensor.from_numpy(np.asarray(positions, np.int32))
+            out = HIPTensor.allocate((n_steps, batch), "int32")
+            lib.call("mh_llama_decode", self._handle, stream, batch, tok.data_ptr, pos.data_ptr, n_steps,
+                     out.data_ptr, logits.data_ptr if logits else None, scratch._pointer, scratch._size)
+            result = out.numpy()
         return result, (logits.numpy() if logits else None)
 
     def weight_bytes_per_token(self, batch: int, context: int) -> int:
@@ -215,7 +234,7 @@ class LlamaDecoder:
         return total
 
 
-def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=print, config=None):
+def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=print, config=None, graph=False):
     """Config 4: 70B-shape GPTQ decode, prefilled KV cache, greedy decode."""
     cfg = dict(config or LLAMA3_70B)
     bmax = max(batches)
@@ -227,17 +246,17 @@ def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=pr
     for b in batches:
         toks = np.arange(b, dtype=np.int32) * 17 + 5
         pos = np.full(b, context, np.int32)
-        dec.decode(toks, pos, 2)                       # warm-up
+        dec.decode(toks, pos, 2, graph=graph)          # warm-up (and the recording of the step)
         memory.synchronize()
-        e0, e1 = memory.Event(), memory.Event()
-        e0.record()
-        out, _ = dec.decode(toks, pos, tokens)
-        e1.record()
-        e1.synchronize()
-        ms = e0.elapsed_ms(e1)
+        # host clock around a call that ends in a device synchronisation: the graph
+        # variant runs on the decoder's own stream, where null-stream events do not see it
+        t0 = time.perf_counter()
+        out, _ = dec.decode(toks, pos, tokens, graph=graph)
+        ms = (time.perf_counter() - t0) * 1e3
         tps = b * tokens / (ms * 1e-3)
         gb = dec.weight_bytes_per_token(b, context + tokens // 2) / 1e9
-        results.append({"batch": b, "context": context, "tokens": tokens, "ms_per_token": round(ms / tokens, 3),
+        results.append({"batch": b, "context": context, "tokens": tokens, "graph": bool(graph),
+                        "ms_per_token": round(ms / tokens, 3),
                         "tok_s": round(tps, 1), "algorithmic_gb_per_step": round(gb, 2),
                         "hbm_gbps": round(gb / (ms / tokens * 1e-3), 1)})
         log(f"decode batch {b}: {ms / tokens:.3f} ms/token, {tps:.1f} tok/s")
@@ -251,6 +270,8 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser(description="Llama-3-70B-shape GPTQ decode on one GPU: tokens per second")
     ap.add_argument("--batches", default="1,8,32")
     ap.add_argument("--tokens", type=int, default=64)
+    ap.add_argument("--graph", action="store_true", help="replay one recorded step per token (HIP graph)")
     cli = ap.parse_args()
     print(json.dumps(bench_tokens_per_second(batches=tuple(int(b) for b in cli.batches.split(",")),
-                                             tokens=cli.tokens, log=lambda *a: print(*a, flush=True))))
+                                             tokens=cli.tokens, log=lambda *a: print(*a, flush=True),
+                                             graph=cli.graph)))

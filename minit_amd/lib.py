@@ -67,6 +67,7 @@ PROTOTYPES = {
     "mh_llama_set_globals": (c_int, [_P, _P, _P, _P, _P, _P]),
     "mh_llama_scratch_bytes": (c_size_t, [_P, c_int]),
     "mh_llama_decode": (c_int, [_P, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t]),
+    "mh_llama_decode_graph": (c_int, [_P, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t]),
     "mh_synth_u32": (c_int, [_P, _P, c_size_t, c_uint64]),
     "mh_synth_subwords": (c_int, [_P, _P, c_size_t, c_int, c_uint32, c_uint32, c_uint64]),
     "mh_synth_normal": (c_int, [_P, _P, c_size_t, c_float, c_float, c_int, c_float, c_uint64, c_int]),

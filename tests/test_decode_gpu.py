@@ -172,3 +172,52 @@ def test_decode_wide_qkv_on_cut_tiles(hip):
             tol = 2e-2 if layer == 0 else 6e-2  # layer 1 sees layer 0's rounding differences
             assert np.abs(kc[b, :, p].astype(np.float64) - ref_k[layer][b, :, p].astype(np.float64)).max() <= tol
             assert np.abs(vc[b, :, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max() <= tol
+
+
+@pytest.mark.parametrize("batch", [1, 3, 9])
+def test_recorded_step_replays_like_the_eager_loop(hip, batch):
+    """mh_llama_decode_graph records one step and replays it per token: tokens,
+    logits and the appended cache entries must equal those of the eager loop bit
+    for bit, on the first use (recording), on later calls (replay only), from a
+    different starting position, and with eager work between the calls."""
+    from minit_amd.decode import LlamaDecoder
+    model = _host_model(CFG, seed=40 + batch)
+    rng = np.random.default_rng(400 + batch)
+    max_seq, context, n_steps = 64, 21, 5
+    shape = (batch, CFG["n_kv_heads"], max_seq, CFG["head_dim"])
+    k_cache = [np.zeros(shape, np.float16) for _ in range(CFG["n_layers"])]
+    v_cache = [np.zeros(shape, np.float16) for _ in range(CFG["n_layers"])]
+    for c in k_cache + v_cache:
+        c[:, :, :context] = rng.normal(0, 1, (batch, CFG["n_kv_heads"], context, CFG["head_dim"]))
+    dec = LlamaDecoder(CFG, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+
+    def caches():
+        return [t.numpy() for t in dec.k_cache + dec.v_cache]
+
+    for round_, start in enumerate((context, context, context + 9, context)):
+        tokens = rng.integers(0, CFG["vocab"], batch)
+        positions = np.full(batch, start) + np.arange(batch) % 2   # ragged rows
+        steps = n_steps - round_ % 2                              # the replay count changes too
+        want_tokens, want_logits = dec.decode(tokens, positions, steps, want_logits=True)
+        want_caches = caches()
+        got_tokens, got_logits = dec.decode(tokens, positions, steps, want_logits=True, graph=True)
+        assert got_tokens.shape == (steps, batch)
+        assert np.array_equal(got_tokens, want_tokens), f"call {round_}: tokens differ"
+        assert np.array_equal(got_logits.view(np.uint16), want_logits.view(np.uint16)), f"call {round_}: logits differ"
+        for a, b in zip(caches(), want_caches):
+            assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), f"call {round_}: cache differs"
+
+
+def test_recorded_step_needs_a_stream(hip):
+    from minit_amd import lib
+    from minit_amd.decode import LlamaDecoder
+    from minit_amd.hip.tensor import HIPTensor
+    model = _host_model(CFG, seed=7)
+    dec = LlamaDecoder(CFG, 1, 64)
+    dec.load_host(model)
+    tok, pos = HIPTensor.from_numpy(np.zeros(1, np.int32)), HIPTensor.from_numpy(np.zeros(1, np.int32))
+    scratch = dec._scratch_for(1)
+    with pytest.raises(lib.HipError, match="stream"):
+        lib.call("mh_llama_decode_graph", dec._handle, None, 1, tok.data_ptr, pos.data_ptr, 1, None, None,
+                 scratch._pointer, scratch._size)
