@@ -116,6 +116,29 @@ def bench_int8(lib, HIPTensor, memory, n, iters=20):
             "frac_of_peak": round(tops / INT8_PEAK_TOPS, 4)}
 
 
+def bench_int8_library(n, iters=50):
+    """The vendor library's int8 GEMM (torch._int_mm, int32 output, no scale epilogue)
+    on the W8A8 shapes and operand layout of bench_int8, as a yardstick for what this
+    problem size allows on the part.  Comparison only: nothing of the library's path."""
+    import torch
+    m, k = 2048, 4096
+    a = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda:0")
+    ws = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda:0").t() for _ in range(4)]
+    for w in ws:
+        torch._int_mm(a, w)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        torch._int_mm(a, ws[i % 4])
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / iters
+    tops = 2.0 * m * n * k / us / 1e6
+    return {"M": m, "N": n, "K": k, "us": round(us, 2), "tops": round(tops, 1),
+            "frac_of_peak": round(tops / INT8_PEAK_TOPS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -134,9 +157,14 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
+    ap.add_argument("--int8-library", action="store_true",
+                    help="time the vendor library's int8 GEMM (torch._int_mm) on the W8A8 shapes, then exit")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the W8A8 GEMM lines (M=2048, K=4096, N in {4096, 11008}), then exit")
     args = ap.parse_args()
+    if args.int8_library:  # before this repository's library is loaded: torch brings a HIP runtime of its own
+        print(json.dumps({"int8_gemm_vendor_library": [bench_int8_library(n) for n in (4096, 11008)]}))
+        return
     ENTRY = args.entry
     if args.gpus != 1:
         log(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
