@@ -29,6 +29,11 @@
 // make a second round (10240 columns: 15.9 / 15.0) and gains a little when they
 // are cut along K instead (14.1 / 15.0, see the kernel); with half the CUs idle
 // on a long K (14336x4096: 16.6 / 14.8) it loses.  gemm_cols_preferred decides.
+// A wide output (8192x57344, 1792 tiles) stays with the small-M kernel (48 us): one
+// tile per workgroup here takes 60 us, and a variant whose workgroups walked seven
+// tiles as one stream (activations parked in LDS once, the ring running across tile
+// borders, one barrier per tile) took 53 us with adjacent tiles per workgroup and
+// 60 us with tiles interleaved across workgroups.
 #include "gptq_common.h"
 
 namespace mh {
