@@ -206,6 +206,10 @@ int mh_softmax_causal(mh_stream_t stream, const void* in, void* out,
 /* minit_sum / minit_max (minit/cuda/kernel/cuda/reduce.py:95): [a,b,c] -> [a,1,c]. */
 int mh_sum(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype);
 int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype);
+/* mean along b as the reference composes it (minit/functional/reduce.py:14-18:
+ * sum, then divide by a tensor filled with the axis length, both in T):
+ * out = T( T(sum) / T(b) ), b > 0. */
+int mh_mean(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype);
 
 /* silu(gate) * up in one pass (the models run sigmoid, multiply, multiply as
  * three launches: examples/llama3_70b.py:44-45,126-130,

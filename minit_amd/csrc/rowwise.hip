@@ -190,7 +190,16 @@ __global__ __launch_bounds__(kRowThreads) void softmax_strided_kernel(
 // [a, b, c] -> [a, 1, c], fp32 accumulate, cast at the store
 // (minit/cuda/kernel/cuda/reduce.py:76-92).
 
-template <typename T, bool IS_MAX>
+// MEAN: the sum is rounded to T and divided by T(b), rounded again, which is what the
+// reference's mean composes (minit/functional/reduce.py:14-18: sum, fill, divide).
+template <typename T>
+__device__ __forceinline__ T mean_of_sum(float sum, size_t b) {
+    const float s = Cvt<T>::to_f32(Cvt<T>::from_f32(sum));
+    const float n = Cvt<T>::to_f32(Cvt<T>::from_f32((float)b));
+    return Cvt<T>::from_f32(s / n);
+}
+
+template <typename T, bool IS_MAX, bool MEAN = false>
 __global__ __launch_bounds__(kRowThreads) void reduce_rows_kernel(const T* __restrict__ in,
                                                                  T* __restrict__ out, size_t b) {
     __shared__ float smem[16];
@@ -211,11 +220,11 @@ __global__ __launch_bounds__(kRowThreads) void reduce_rows_kernel(const T* __res
         acc = IS_MAX ? fmaxf(acc, f) : acc + f;
     }
     acc = IS_MAX ? block_max(acc, smem) : block_sum(acc, smem);
-    if (threadIdx.x == 0) out[row] = Cvt<T>::from_f32(acc);
+    if (threadIdx.x == 0) out[row] = MEAN ? mean_of_sum<T>(acc, b) : Cvt<T>::from_f32(acc);
 }
 
 // c > 1: one thread per output element, coalesced across c.
-template <typename T, bool IS_MAX>
+template <typename T, bool IS_MAX, bool MEAN = false>
 __global__ void reduce_strided_kernel(const T* __restrict__ in, T* __restrict__ out, size_t a, size_t b,
                                       size_t c) {
     const size_t total = a * c;
@@ -227,7 +236,7 @@ __global__ void reduce_strided_kernel(const T* __restrict__ in, T* __restrict__ 
             const float f = Cvt<T>::to_f32(in[base + j * c]);
             acc = IS_MAX ? fmaxf(acc, f) : acc + f;
         }
-        out[idx] = Cvt<T>::from_f32(acc);
+        out[idx] = MEAN ? mean_of_sum<T>(acc, b) : Cvt<T>::from_f32(acc);
     }
 }
 
@@ -355,13 +364,13 @@ static int softmax_t(hipStream_t st, const void* in, void* out, size_t a, size_t
     return MH_OK;
 }
 
-template <typename T, bool IS_MAX>
+template <typename T, bool IS_MAX, bool MEAN = false>
 static int reduce_t(hipStream_t st, const void* in, void* out, size_t a, size_t b, size_t c) {
     if (c == 1) {
-        hipLaunchKernelGGL((reduce_rows_kernel<T, IS_MAX>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
+        hipLaunchKernelGGL((reduce_rows_kernel<T, IS_MAX, MEAN>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
                            (const T*)in, (T*)out, b);
     } else {
-        hipLaunchKernelGGL((reduce_strided_kernel<T, IS_MAX>), dim3(grid_for(a * c, 256)), dim3(256), 0, st,
+        hipLaunchKernelGGL((reduce_strided_kernel<T, IS_MAX, MEAN>), dim3(grid_for(a * c, 256)), dim3(256), 0, st,
                            (const T*)in, (T*)out, a, b, c);
     }
     MH_CHECK_LAUNCH();
@@ -433,6 +442,14 @@ int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, si
     MH_REQUIRE(in && out, "mh_max: null pointer");
     MH_REQUIRE(a <= 0x7fffffffu, "mh_max: too many rows");
     MH_DISPATCH_DTYPE(dtype, "mh_max", return (reduce_t<T, true>(as_stream(stream), in, out, a, b, c)));
+}
+
+int mh_mean(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype) {
+    if (a * c == 0) return MH_OK;
+    MH_REQUIRE(in && out, "mh_mean: null pointer");
+    MH_REQUIRE(b > 0, "mh_mean: empty axis");
+    MH_REQUIRE(a <= 0x7fffffffu, "mh_mean: too many rows");
+    MH_DISPATCH_DTYPE(dtype, "mh_mean", return (reduce_t<T, false, true>(as_stream(stream), in, out, a, b, c)));
 }
 
 int mh_rope(mh_stream_t stream, const void* in, const float* freqs_cos, const float* freqs_sin,

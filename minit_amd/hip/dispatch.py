@@ -7,7 +7,7 @@ against the HIP library.
 from ..core.dispatch import register_dispatch
 from ..core.tensor import Tensor
 from ..lib import DTYPE_CODES, call
-from ..operator import MatrixMultiply, Max, RMSNorm, RoPE, Softmax, Sum
+from ..operator import MatrixMultiply, Max, Mean, RMSNorm, RoPE, Softmax, Sum
 from ..quantize.operator import Dequantize
 from ..quantize.tensor import QuantizedTensor, _NoGroup
 from . import memory
@@ -125,3 +125,4 @@ def _register_reduce(op_type, symbol):
 
 _register_reduce(Sum, "mh_sum")
 _register_reduce(Max, "mh_max")
+_register_reduce(Mean, "mh_mean")

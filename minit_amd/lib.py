@@ -59,6 +59,7 @@ PROTOTYPES = {
     "mh_softmax_causal": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_size_t, c_float, c_int]),
     "mh_sum": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_max": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
+    "mh_mean": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
     "mh_add_bias": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_int]),
     "mh_llama_create": (c_int, [POINTER(c_void_p), _P]),

@@ -43,3 +43,11 @@ class Sum(Operator):
 @dataclass
 class Max(Operator):
     axis: int
+
+
+@dataclass
+class Mean(Operator):
+    """Not an operator of the reference, whose ``mean`` dispatches Sum, Fill and
+    Divide (minit/functional/reduce.py:14-18); one operator here so that the three
+    steps are one launch with the same two roundings."""
+    axis: int

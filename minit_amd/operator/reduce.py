@@ -1,1 +1,1 @@
-from . import Max, Sum  # noqa: F401
+from . import Max, Mean, Sum  # noqa: F401

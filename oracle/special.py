@@ -116,6 +116,15 @@ def reduce_sum(x: np.ndarray, axis: int) -> np.ndarray:
     return x.astype(np.float64).sum(axis=axis, keepdims=True).astype(x.dtype)
 
 
+def reduce_mean(x: np.ndarray, axis: int) -> np.ndarray:
+    """minit/functional/reduce.py:14-18: ``sum(x) / fill(size)``, the sum rounded to
+    the storage type, the length as a tensor of that type, and their quotient by the
+    element-wise Divide (minit/cuda/dispatch.py:139, ``{0} / {1}`` in T)."""
+    s = reduce_sum(x, axis)
+    n = np.asarray(x.shape[axis]).astype(x.dtype)
+    return (s.astype(np.float64) / np.float64(n)).astype(x.dtype)
+
+
 def reduce_max(x: np.ndarray, axis: int) -> np.ndarray:
     """Same kernel with init -inf and max."""
     return x.max(axis=axis, keepdims=True)

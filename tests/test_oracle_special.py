@@ -92,3 +92,12 @@ def test_reductions():
     np.testing.assert_allclose(O.reduce_sum(x, 1)[:, 0], x.sum(axis=1), rtol=1e-5, atol=1e-6)
     np.testing.assert_array_equal(O.reduce_max(x, 1)[:, 0], x.max(axis=1))
     assert (O.reduce_sum(np.ones((2, 9), np.float16), 1) == 9).all()
+    # mean = T(T(sum) / T(n)): constant rows give the constant; the sum is rounded
+    # first (2049 ones of fp16 sum to 2048), and so is the length (2049 -> 2048)
+    assert (O.reduce_mean(np.full((2, 9), 0.5, np.float16), 1) == 0.5).all()
+    assert O.reduce_mean(np.ones((1, 2049), np.float16), 1)[0, 0] == 1.0
+    big = np.full((1, 3000), 2.0, np.float16)          # sum 6000 is exact, n = 3000 is exact
+    assert O.reduce_mean(big, 1)[0, 0] == 2.0
+    m = O.reduce_mean(x, 1)
+    assert m.shape == (3, 1, 2)
+    np.testing.assert_allclose(m[:, 0], x.mean(axis=1), rtol=2e-3, atol=1e-6)

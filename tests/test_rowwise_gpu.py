@@ -140,6 +140,11 @@ def test_sum_max(hip, shape, axis):
     np.testing.assert_array_equal(F.max(_t(x), axis).numpy(), O.reduce_max(x, axis))
     ones = np.ones(shape, np.float16)
     assert (F.sum(_t(ones), axis).numpy() == shape[axis]).all()
+    # mean: the rounded sum divided by the rounded length, rounded again
+    s16 = s.astype(np.float64)
+    n16 = np.float64(np.asarray(shape[axis]).astype(np.float16))
+    np.testing.assert_array_equal(F.mean(_t(x), axis).numpy(), (s16 / n16).astype(np.float16))
+    assert (F.mean(_t(ones), axis).numpy() == 1).all()
 
 
 def test_silu_mul(hip):
