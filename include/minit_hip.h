@@ -211,6 +211,13 @@ int mh_max(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, si
  * out = T( T(sum) / T(b) ), b > 0. */
 int mh_mean(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, size_t c, int dtype);
 
+/* The element-wise kernels the models' silu is made of (examples/llama3_70b.py:44-45,
+ * `x * F.sigmoid(x)`): the reference's Sigmoid expression, 1.0 / (1.0 + expf((float)-x))
+ * evaluated in double and rounded once to T (minit/cuda/dispatch.py:143), and the
+ * element-wise product in T (`{0} * {1}`, :137).  n elements, same shape. */
+int mh_sigmoid(mh_stream_t stream, const void* in, void* out, size_t n, int dtype);
+int mh_multiply(mh_stream_t stream, const void* a, const void* b, void* out, size_t n, int dtype);
+
 /* silu(gate) * up in one pass (the models run sigmoid, multiply, multiply as
  * three launches: examples/llama3_70b.py:44-45,126-130,
  * minit/cuda/dispatch.py:137,143).  exact != 0 reproduces the three fp16

@@ -42,6 +42,10 @@ class Tensor(Object):
         from ..functional.special import softmax
         return softmax(self, axis)
 
+    def __mul__(self, other: "Tensor"):
+        from ..functional.arith import multiply
+        return multiply(self, other)
+
     def __matmul__(self, other: "Tensor"):
         from ..functional.linalg import matrix_multiply
         return matrix_multiply(self, other)

@@ -1,3 +1,4 @@
 from .linalg import matrix_multiply
 from .reduce import max, mean, sum
-from .special import rms_norm, rope, softmax
+from .arith import multiply
+from .special import rms_norm, rope, sigmoid, softmax

@@ -6,7 +6,12 @@ from typing import Optional
 
 from ..core.dispatch import dispatch
 from ..core.tensor import Tensor
-from ..operator import RMSNorm, RoPE, Softmax
+from ..operator import RMSNorm, RoPE, Sigmoid, Softmax
+
+
+def sigmoid(x: Tensor):
+    (z,) = dispatch(Sigmoid(), x)
+    return z
 
 
 def rms_norm(x: Tensor, weight: Tensor, axis: int, eps: float) -> Tensor:

@@ -7,7 +7,7 @@ against the HIP library.
 from ..core.dispatch import register_dispatch
 from ..core.tensor import Tensor
 from ..lib import DTYPE_CODES, call
-from ..operator import MatrixMultiply, Max, Mean, RMSNorm, RoPE, Softmax, Sum
+from ..operator import MatrixMultiply, Max, Mean, Multiply, RMSNorm, RoPE, Sigmoid, Softmax, Sum
 from ..quantize.operator import Dequantize
 from ..quantize.tensor import QuantizedTensor, _NoGroup
 from . import memory
@@ -22,6 +22,13 @@ def _abc(shape, axis):
     for dim in shape[axis + 1:]:
         c *= dim
     return a, b, c
+
+
+def _count(shape) -> int:
+    n = 1
+    for dim in shape:
+        n *= dim
+    return n
 
 
 def _code(dtype: str) -> int:
@@ -111,6 +118,24 @@ def register_softmax_operator(op: Softmax, x: HIPTensor):
     z = HIPTensor.allocate(x._shape, x.dtype)
     a, b, c = _abc(x._shape, op.axis)
     call("mh_softmax", None, x.data_ptr, z.data_ptr, a, b, c, _code(x.dtype))
+    return (z,)
+
+
+# The two element-wise rules the models' ``silu`` needs (minit/cuda/dispatch.py:104-117
+# with the expressions of :137 and :143); operands of one shape and dtype.
+@register_dispatch()
+def dispatch_sigmoid(op: Sigmoid, x: HIPTensor):
+    z = HIPTensor.allocate(x._shape, x.dtype)
+    call("mh_sigmoid", None, x.data_ptr, z.data_ptr, _count(x._shape), _code(x.dtype))
+    return (z,)
+
+
+@register_dispatch()
+def dispatch_multiply(op: Multiply, x: HIPTensor, y: HIPTensor):
+    assert x._shape == y._shape, f"multiply: shapes {x._shape} and {y._shape} differ"
+    assert x.dtype == y.dtype
+    z = HIPTensor.allocate(x._shape, x.dtype)
+    call("mh_multiply", None, x.data_ptr, y.data_ptr, z.data_ptr, _count(x._shape), _code(x.dtype))
     return (z,)
 
 

@@ -1,5 +1,5 @@
 """Operator descriptors of the hot path; same names and fields as the reference
-(minit/operator/linalg.py:9-16, special.py:6-23, reduce.py:6-13)."""
+(minit/operator/linalg.py:9-16, special.py:6-23, reduce.py:6-13, arith.py:20-22)."""
 from dataclasses import dataclass
 
 from ..core.operator import Operator
@@ -16,6 +16,12 @@ class BatchMatrixMultiply(Operator):
 
 
 class Sigmoid(Operator):
+    ...
+
+
+@dataclass
+class Multiply(Operator):
+    """minit/operator/arith.py:20-22."""
     ...
 
 

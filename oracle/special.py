@@ -111,6 +111,18 @@ def masked_softmax(scores: np.ndarray, offset: int) -> np.ndarray:
     return softmax(scores + causal_mask(s, offset, scores.dtype)[None, None], 3)
 
 
+def sigmoid(x: np.ndarray) -> np.ndarray:
+    """minit/cuda/dispatch.py:143: ``1.0 / (1.0 + expf((float)-x))``, the sum and the
+    quotient in double (the literals are doubles), one rounding to the storage type."""
+    e = np.exp((-x.astype(np.float32)).astype(np.float32)).astype(np.float32)  # expf: float in, float out
+    return (1.0 / (1.0 + e.astype(np.float64))).astype(x.dtype)
+
+
+def multiply(x: np.ndarray, y: np.ndarray) -> np.ndarray:
+    """minit/cuda/dispatch.py:137: ``{0} * {1}`` in the storage type (one rounding)."""
+    return (x.astype(np.float64) * y.astype(np.float64)).astype(x.dtype)
+
+
 def reduce_sum(x: np.ndarray, axis: int) -> np.ndarray:
     """minit/cuda/kernel/cuda/reduce.py:76-92 with init 0: keepdim sum."""
     return x.astype(np.float64).sum(axis=axis, keepdims=True).astype(x.dtype)

@@ -101,3 +101,24 @@ def test_reductions():
     m = O.reduce_mean(x, 1)
     assert m.shape == (3, 1, 2)
     np.testing.assert_allclose(m[:, 0], x.mean(axis=1), rtol=2e-3, atol=1e-6)
+
+
+def test_sigmoid_and_multiply():
+    """The element-wise expressions of the models' silu (minit/cuda/dispatch.py:137,143)."""
+    x = np.array([0.0, 1.0, -1.0, 20.0, -20.0, 0.5], np.float16)
+    s = O.sigmoid(x)
+    assert s.dtype == np.float16 and s[0] == 0.5
+    assert s[3] == 1.0 and 0 <= s[4] < 1e-7                       # saturation, no NaN
+    assert abs(float(s[1]) + float(s[2]) - 1.0) <= 2 ** -11       # sigmoid(-x) = 1 - sigmoid(x)
+    assert abs(float(s[1]) - 1 / (1 + np.exp(-1.0))) <= 2 ** -12  # half an fp16 step at 0.73
+    # the product is rounded once: 1.001 * 1.001 in fp16
+    a = np.array([1.0009765625, 3.0, -0.5], np.float16)
+    b = np.array([1.0009765625, 0.333251953125, 0.5], np.float16)
+    np.testing.assert_array_equal(O.multiply(a, b), np.array([1.001953125, 1.0, -0.25], np.float16))
+    # and it composes to the three-rounding silu(gate) * up of the quantized-path oracle
+    from oracle import gptq as OG
+    rng = np.random.default_rng(12)
+    g = rng.normal(0, 3, 4096).astype(np.float16)
+    u = rng.normal(0, 3, 4096).astype(np.float16)
+    np.testing.assert_array_equal(O.multiply(O.multiply(g, O.sigmoid(g)), u).view(np.uint16),
+                                  OG.silu_mul(g, u).view(np.uint16))

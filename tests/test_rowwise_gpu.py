@@ -163,6 +163,30 @@ def test_silu_mul(hip):
     _assert_ulp(out.numpy(), OG.silu_mul_f64(g, u).astype(np.float16), what="silu_mul fused")
 
 
+def test_sigmoid_multiply_compose_to_silu(hip):
+    """``x * F.sigmoid(x)`` and ``silu(gate) * up`` through the operator API, as
+    the models spell them (examples/llama3_70b.py:44-45,126-130): the product is
+    bit-exact, sigmoid is the oracle's up to expf against exp, and the composition
+    equals the fused kernel's three-rounding mode bit for bit."""
+    import minit_amd.functional as F
+    from minit_amd.hip.tensor import HIPTensor
+    rng = np.random.default_rng(13)
+    g = rng.normal(0, 3, size=(5, 1031)).astype(np.float16)      # odd width: vector body and scalar tail
+    u = rng.normal(0, 3, size=(5, 1031)).astype(np.float16)
+    dg, du = _t(g), _t(u)
+    np.testing.assert_array_equal(F.multiply(dg, du).numpy().view(np.uint16), O.multiply(g, u).view(np.uint16))
+    sig = F.sigmoid(dg).numpy()
+    _assert_ulp(sig, O.sigmoid(g), ulps=1.0, what="sigmoid")
+    assert (sig.view(np.uint16) != O.sigmoid(g).view(np.uint16)).mean() < 1e-3
+    h = ((dg * F.sigmoid(dg)) * du).numpy()
+    fused = HIPTensor.allocate(g.shape, "float16")
+    hip.call("mh_silu_mul", None, dg.data_ptr, du.data_ptr, fused.data_ptr, g.size, 1, 0)
+    np.testing.assert_array_equal(h.view(np.uint16), fused.numpy().view(np.uint16))
+    _assert_ulp(h, OG.silu_mul(g, u), ulps=1.0, what="silu through operators")
+    with pytest.raises(AssertionError):
+        F.multiply(dg, _t(u[:2]))
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 1000, 512), (8, 128256, 256), (40, 72, 4096), (3, 50, 37)])
 def test_dense_matmul_nk(hip, m, n, k):
     import minit_amd.functional as F
