@@ -116,6 +116,112 @@ def bench_int8(lib, HIPTensor, memory, n, iters=20):
             "frac_of_peak": round(tops / INT8_PEAK_TOPS, 4)}
 
 
+def _time_launches(memory, fn, iters=200, warmup=10):
+    for i in range(warmup):
+        fn(i)
+    memory.synchronize()
+    e0, e1 = memory.Event(), memory.Event()
+    e0.record()
+    for i in range(iters):
+        fn(i)
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_ms(e1) * 1e3 / iters
+
+
+def bench_rowwise(lib, HIPTensor, memory):
+    """Config 3: RMSNorm [16, 4096], RoPE [16, 1, 32, 128] at random positions, softmax
+    and row-sum over [512, ctx]; microseconds per launch and algorithmic GB/s (every
+    operand once).  The working sets are a few MB and stay in cache: these lines show
+    launch latency, not HBM."""
+    import numpy as np
+    from minit_amd import synthetic
+    out = []
+
+    def add(name, us, nbytes):
+        out.append({"kernel": name, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1)})
+
+    f16 = 0
+    x = HIPTensor.allocate((16, 4096), "float16")
+    w = HIPTensor.allocate((4096,), "float16")
+    y = HIPTensor.allocate((16, 4096), "float16")
+    lib.call("mh_synth_normal", None, x.data_ptr, 16 * 4096, 0.0, 1.0, 0, 0.0, 31, 0)
+    lib.call("mh_synth_normal", None, w.data_ptr, 4096, 1.0, 0.1, 0, 0.0, 32, 0)
+    us = _time_launches(memory, lambda i: lib.call("mh_rms_norm", None, x.data_ptr, w.data_ptr, y.data_ptr,
+                                                    16, 4096, 1, 1e-6, f16))
+    add("rms_norm [16,4096]", us, 2 * 16 * 4096 * 2 + 4096 * 2)
+
+    cos, sin = synthetic.rope_tables(128, 4096, 1e6)
+    dcos, dsin = HIPTensor.from_numpy(cos), HIPTensor.from_numpy(sin)
+    pos = HIPTensor.from_numpy(np.random.default_rng(33).integers(0, 4096, size=(16, 1)).astype(np.int32))
+    q = HIPTensor.allocate((16, 1, 32, 128), "float16")
+    qo = HIPTensor.allocate((16, 1, 32, 128), "float16")
+    lib.call("mh_synth_normal", None, q.data_ptr, 16 * 32 * 128, 0.0, 1.0, 0, 0.0, 34, 0)
+    us = _time_launches(memory, lambda i: lib.call("mh_rope", None, q.data_ptr, dcos.data_ptr, dsin.data_ptr,
+                                                    pos.data_ptr, qo.data_ptr, 16, 1, 32, 128, f16))
+    add("rope [16,1,32,128]", us, 2 * 16 * 32 * 128 * 2 + 16 * 64 * 4 * 2)
+
+    for ctx in (1024, 4096):
+        sc = HIPTensor.allocate((512, ctx), "float16")
+        so = HIPTensor.allocate((512, ctx), "float16")
+        rs = HIPTensor.allocate((512, 1), "float16")
+        lib.call("mh_synth_normal", None, sc.data_ptr, 512 * ctx, 0.0, 3.0, 0, 0.0, 35, 0)
+        us = _time_launches(memory, lambda i: lib.call("mh_softmax", None, sc.data_ptr, so.data_ptr, 512, ctx, 1, f16))
+        add(f"softmax [512,{ctx}]", us, 2 * 512 * ctx * 2)
+        us = _time_launches(memory, lambda i: lib.call("mh_sum", None, sc.data_ptr, rs.data_ptr, 512, ctx, 1, f16))
+        add(f"row_sum [512,{ctx}]", us, 512 * ctx * 2 + 512 * 2)
+    return out
+
+
+def bench_small_configs(lib, HIPTensor, memory, ws):
+    """Config 0 (GEMV 4096x4096) and config 1 (Mistral-7B MLP block: gate|up 4096 ->
+    2 x 14336 with the SiLU*up epilogue, down 14336 -> 4096) at M in {1, 8, 32, 128};
+    weight sets rotated over more than the 256 MB Infinity Cache."""
+    res = {}
+    hidden, ffn = 4096, 14336
+    sets = 16  # x 8.7 MB (config 0) / x 91.5 MB (config 1)
+    lin0 = [DeviceLinear(lib, HIPTensor, hidden, hidden, 500 + i) for i in range(32)]
+    x0 = HIPTensor.allocate((1, hidden), "float16")
+    lib.call("mh_synth_normal", None, x0.data_ptr, hidden, 0.0, 1.0, 0, 0.0, 41, 0)
+    y0 = HIPTensor.allocate((1, hidden), "float16")
+    us = _time_launches(memory, lambda i: run_gemv(lib, x0, lin0[i % 32], y0, ws), iters=128, warmup=32)
+    res["gemv_cfg0"] = {"M": 1, "K": hidden, "N": hidden, "us": round(us, 2),
+                        "gbps": round(linear_bytes(1, hidden, hidden) / us / 1e3, 1)}
+    del lin0
+    gate_up = [DeviceLinear(lib, HIPTensor, hidden, 2 * ffn, 600 + i) for i in range(sets // 4)]
+    down = [DeviceLinear(lib, HIPTensor, ffn, hidden, 700 + i) for i in range(sets // 4)]
+    block = []
+    halves = None
+    for m in (1, 8, 32, 128):
+        x = HIPTensor.allocate((m, hidden), "float16")
+        lib.call("mh_synth_normal", None, x.data_ptr, m * hidden, 0.0, 1.0, 0, 0.0, 42, 0)
+        h = HIPTensor.allocate((m, ffn), "float16")
+        y = HIPTensor.allocate((m, hidden), "float16")
+
+        if m <= 32:   # one launch for gate|up with SiLU*up in its reduction
+            def step(i):
+                gu, dn = gate_up[i % len(gate_up)], down[i % len(down)]
+                lib.call("mh_gptq_matmul_silu_pairs", None, x.data_ptr, gu.qweight.data_ptr, gu.qzeros.data_ptr,
+                         gu.scales.data_ptr, h.data_ptr, m, 2 * ffn, hidden, GROUP, BITS, ws._pointer, ws._size)
+                run_gemv(lib, h, dn, y, ws, m=m)
+        else:         # above 32 rows: gate, up, SiLU*up, down as four launches
+            if halves is None:
+                halves = [DeviceLinear(lib, HIPTensor, hidden, ffn, 800 + i) for i in range(8)]
+            g, u = HIPTensor.allocate((m, ffn), "float16"), HIPTensor.allocate((m, ffn), "float16")
+
+            def step(i, g=g, u=u):
+                run_gemv(lib, x, halves[(2 * i) % 8], g, ws, m=m)
+                run_gemv(lib, x, halves[(2 * i + 1) % 8], u, ws, m=m)
+                lib.call("mh_silu_mul", None, g.data_ptr, u.data_ptr, h.data_ptr, m * ffn, 0, 0)
+                run_gemv(lib, h, down[i % len(down)], y, ws, m=m)
+        us = _time_launches(memory, step, iters=40, warmup=4)
+        nbytes = linear_bytes(m, hidden, 2 * ffn) - m * ffn * 2 + linear_bytes(m, ffn, hidden)
+        block.append({"M": m, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                      "tflops": round(2.0 * m * 3 * hidden * ffn / us / 1e6, 2)})
+    res["mlp_block_cfg1"] = block
+    return res
+
+
 def bench_int8_library(n, iters=50):
     """The vendor library's int8 GEMM (torch._int_mm, int32 output, no scale epilogue)
     on the W8A8 shapes and operand layout of bench_int8, as a yardstick for what this
@@ -325,6 +431,13 @@ def main():
                 result["extra"]["int8_gemm"] = [bench_int8(lib, HIPTensor, memory, n) for n in (4096, 11008)]
         except Exception as exc:  # report, do not hide
             result["extra"]["int8_gemm_error"] = str(exc)
+        try:
+            if not args.shapes_only:
+                result["extra"]["rowwise_cfg3"] = bench_rowwise(lib, HIPTensor, memory)
+                big = lib.call("mh_gptq_workspace_bytes", 128, 2 * 14336, 4096, GROUP, BITS)
+                result["extra"].update(bench_small_configs(lib, HIPTensor, memory, memory.workspace(max(big, ws._size))))
+        except Exception as exc:
+            result["extra"]["small_configs_error"] = str(exc)
         try:
             if args.shapes_only:
                 raise RuntimeError("skipped (--shapes-only)")
