@@ -246,10 +246,10 @@ constexpr int kSmallDepth = 8;  // steps per stage = ring depth
 // accumulators), otherwise only the regular one.
 template <int BITS, int MT, int SPG, bool NORM, bool STREAM>
 __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
-    const half_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const half_t* __restrict__ x_all, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
-    half_t* out, float* partial, unsigned* counters,
-    int M, int N, int K, int steps_total, int stages_per_block, int split_k, int stream_units, int epilogue,
+    half_t* out_all, float* partial_all, unsigned* counters,
+    int M_all, int N, int K, int steps_total, int stages_per_block, int split_k, int stream_units, int epilogue,
     SmallFuse fuse) {
     constexpr int P = Packing<BITS>::kPerWord;
     constexpr int PAIRS = Packing<BITS>::kPairs;
@@ -259,6 +259,16 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     constexpr int D = kSmallDepth;
     constexpr int GPS = D / SPG;            // groups per stage
     constexpr int BM = 16 * MT;
+    // More rows than one workgroup takes: blockIdx.z picks a block of BM rows (regular
+    // plan, no in-kernel reduction).  The row blocks read the same packed weights at
+    // the same time, so one of them finds them in a cache; the partial sums of all
+    // blocks form one [split][M_all][N] array for the second stage.
+    const int row0 = blockIdx.z * BM;
+    const int M = min(M_all - row0, BM);
+    const half_t* __restrict__ x = x_all + (size_t)row0 * K;
+    half_t* out = out_all + (size_t)row0 * N;
+    float* partial = partial_all + (size_t)row0 * N;
+    const size_t plane = (size_t)M_all * N;  // one split's partial sums
     constexpr int XCH = D * 4;              // 16-byte activation chunks per row per stage
     constexpr int RS = XCH + 1;             // padded row stride
     constexpr int XL = BM * XCH / 256;      // chunks each thread stages: 2 (MT=1) or 4 (MT=2)
@@ -555,7 +565,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                     const half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
                 } else {
-                    float* dst = partial + ((size_t)slot * M + m) * N + col;
+                    float* dst = partial + (size_t)slot * plane + (size_t)m * N + col;
                     if (counters)
                         store_agent4(dst, v);
                     else
@@ -585,7 +595,6 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 
     auto reduce_tile = [&](int tile, int nseg) {
         constexpr int BATCH = 16;  // partial loads in flight per thread
-        const size_t plane = (size_t)M * N;
         auto sum_splits = [&](const float* p) {
             float4_t s = {0.f, 0.f, 0.f, 0.f};
             for (int sp = 0; sp < nseg; sp += BATCH) {
@@ -703,25 +712,31 @@ static int env_int_gemm(const char* name, int fallback) {
     return atoi(v);
 }
 
-constexpr int kSmallMaxM = 32;
+constexpr int kSmallMaxM = 32;     // rows of one launch with epilogues / norm fusion
+constexpr int kSmallBlockM = 64;   // rows per pass of a plain product above kSmallMaxM rows
 constexpr int kFusedReduceMaxM = 8;
 
 // Plan of the small-M kernel: column tiles x K splits sized so the GPU holds
 // about MH_GEMM_SMALL_WAVES_PER_CU waves per CU; a block walks whole stages.
 // GemmPlan::steps_per_block carries stages_per_block * kSmallDepth.
-GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced) {
+GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_blocks = 1) {
     GemmPlan p;
-    p.mt = M <= 16 ? 1 : 2;
+    p.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     p.col_tiles = (N + kGemmCols - 1) / kGemmCols;
-    p.m_blocks = 1;
+    p.m_blocks = row_blocks;
     p.steps_total = K / 32;
     const long stages_total = (p.steps_total + kSmallDepth - 1) / kSmallDepth;
     static const int waves_per_cu = env_int_gemm("MH_GEMM_SMALL_WAVES_PER_CU", 8);
     const long target_blocks = (long)compute_units() * waves_per_cu / 4;
-    long split = target_blocks / p.col_tiles;
+    long split = target_blocks / ((long)p.col_tiles * row_blocks);
     if (split > stages_total) split = stages_total;
     // fp32 partials cost 8*M*N bytes per split against K*N/2 bytes of weights
-    const long traffic_cap = K / (32L * M) > 1 ? K / (32L * M) : 1;
+    // (a single block of more than 32 rows is bound by instruction issue and by the
+    // CUs left idle, and more splits are worth twice the partial-sum traffic:
+    // 4096x14336 at 64 rows 32.8 -> 26.6 us; with two or more row blocks side by
+    // side the CUs are taken and the looser cap loses, 38.5 -> 42.1 us at 128 rows)
+    const long cap_unit = M > 32 && row_blocks == 1 ? 16L * M : 32L * M;
+    const long traffic_cap = K / cap_unit > 1 ? K / cap_unit : 1;
     if (split > traffic_cap) split = traffic_cap;
     if (split < 1) split = 1;
     const long spb = (stages_total + split - 1) / split;
@@ -821,7 +836,11 @@ static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_sm
 
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     (void)bits;
-    if (row_blocked(M, group_size)) M = kSmallMaxM;  // taken 32 rows at a time
+    if (row_blocked(M, group_size)) {
+        // blocks of kSmallBlockM rows in one launch; partial sums [split][M][N]
+        const GemmPlan p = plan_gemm_small(kSmallBlockM, N, K, false, (M + kSmallBlockM - 1) / kSmallBlockM);
+        return kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float);
+    }
     // either plan of the small-M kernel may be the one a launch takes
     const GemmPlan p = plan_gemm(M, N, K, group_size, false), pb = plan_gemm(M, N, K, group_size, true);
     const int slots = p.split_k > pb.split_k ? p.split_k : pb.split_k;
@@ -854,21 +873,26 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
     unsigned* counters =
         (M <= kFusedReduceMaxM && p.col_tiles <= kMaxTileCounters) ? reinterpret_cast<unsigned*>(workspace) : nullptr;
     float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
-    const dim3 grid = p.stream_units ? dim3(p.blocks) : dim3(p.col_tiles, p.split_k);
+    const dim3 grid = p.stream_units ? dim3(p.blocks) : dim3(p.col_tiles, p.split_k, p.m_blocks);
     const bool norm = fuse.ssq_in != nullptr;
 #define MH_LAUNCH_SMALL_N(SPG, NORM, STREAM)                                                                  \
     hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG, NORM, STREAM>), grid, dim3(256), 0, stream,         \
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, \
                        (half_t*)out, partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth,  \
                        p.split_k, p.stream_units, epilogue, fuse)
-#define MH_LAUNCH_SMALL(SPG)                            \
-    do {                                                \
-        if (norm)                                       \
-            MH_LAUNCH_SMALL_N(SPG, true, false);        \
-        else if (MT == 1 && p.stream_units != 0)        \
-            MH_LAUNCH_SMALL_N(SPG, false, (MT == 1));   \
-        else                                            \
-            MH_LAUNCH_SMALL_N(SPG, false, false);       \
+#define MH_LAUNCH_SMALL(SPG)                                     \
+    do {                                                         \
+        if constexpr (MT <= 2) {                                 \
+            if (norm) {                                          \
+                MH_LAUNCH_SMALL_N(SPG, true, false);             \
+                break;                                           \
+            }                                                    \
+            if (MT == 1 && p.stream_units != 0) {                \
+                MH_LAUNCH_SMALL_N(SPG, false, (MT == 1));        \
+                break;                                           \
+            }                                                    \
+        }                                                        \
+        MH_LAUNCH_SMALL_N(SPG, false, false);                    \
     } while (0)
     switch (group_size / 32) {
         case 1: MH_LAUNCH_SMALL(1); break;
@@ -914,20 +938,28 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
         return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse,
                                      workspace, workspace_bytes);
     if (row_blocked(M, group_size)) {
-        // Above kSmallMaxM rows the product is taken 32 rows at a time by the small-M
-        // kernel: the packed weights are re-read per block of rows (from the
-        // Infinity Cache when they fit), which measured 2-5x faster at M = 64..128
-        // than the staged kernel, whose few large workgroups leave most CUs idle.
+        // Above kSmallMaxM rows the small-M kernel takes blocks of 64 rows (four 16-row
+        // tiles per workgroup) side by side in one launch: the packed weights are read
+        // once per block of rows, the second reader mostly from a cache.  Measured
+        // 2-5x faster at M = 64..128 than the staged kernel, whose few large
+        // workgroups leave most CUs idle.
         if (epilogue != kEpilogueNone || fuse.ssq_in != nullptr)
             return fail(MH_ERR_INVALID, "gptq gemm: epilogues and norm fusion need M <= %d", kSmallMaxM);
-        const size_t esz = sizeof(half_t);
-        for (int m0 = 0; m0 < M; m0 += kSmallMaxM) {
-            const int rows = M - m0 < kSmallMaxM ? M - m0 : kSmallMaxM;
-            const int rc = gptq_gemm_launch(stream, (const char*)x + (size_t)m0 * K * esz, qweight, qzeros, scales,
-                                            (char*)out + (size_t)m0 * N * esz, rows, N, K, group_size, bits, workspace,
-                                            workspace_bytes, kEpilogueNone, fuse);
-            if (rc) return rc;
-        }
+        const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
+                        workspace ? workspace_bytes : (size_t)0);
+        if ((uintptr_t)workspace % 256 != 0)
+            return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace must be 256-byte aligned");
+        // one launch: blockIdx.z walks the blocks of kSmallBlockM rows
+        const GemmPlan p = plan_gemm_small(kSmallBlockM, N, K, false, (M + kSmallBlockM - 1) / kSmallBlockM);
+        if (bits == 4)
+            launch_gemm_small<4, 4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size,
+                                    kEpilogueNone, fuse);
+        else
+            launch_gemm_small<8, 4>(stream, p, x, qweight, qzeros, scales, out, workspace, M, N, K, group_size,
+                                    kEpilogueNone, fuse);
+        MH_CHECK_LAUNCH();
         return MH_OK;
     }
     const GemmPlan p = plan_gemm(M, N, K, group_size, epilogue == kEpilogueNone && fuse.ssq_in == nullptr);
