@@ -131,6 +131,18 @@ def special_cases():
         "x": t,
         "sum": [[[8, 0, 18]], [[2.5, 4.25, 8]]],
         "max": [[[10, 8, 12]], [[2, 4, 8]]],
+        # mean = sum / 4 (the reference divides the rounded sum by the rounded length: both exact here)
+        "mean": [[[2, 0, 4.5]], [[0.625, 1.0625, 2]]],
+    }
+    # mean where the roundings show: 2049 ones sum to 2049, which fp16 rounds to 2048 (ties to even), and the
+    # length 2049 rounds to 2048 as well: 2048 / 2048 = 1; 2050 halves: sum 1025, length 2050 -> 0.5
+    cases["mean_roundings"] = {"ones": 2049, "ones_mean": 1.0, "halves": 2050, "halves_mean": 0.5}
+    # the two element-wise kernels of the models' silu: sigmoid(0) = 1 / (1 + 1) = 0.5; products rounded once:
+    # (1 + 2^-10)^2 = 1 + 2^-9 + 2^-20 -> 1 + 2^-9; 3 * 0.333251953125 = 0.999755859375 -> 1.0 (tie to even)
+    cases["elementwise"] = {
+        "sigmoid_in": [0.0], "sigmoid_out": [0.5],
+        "a": [1.0009765625, 3.0, -0.5, 0.0], "b": [1.0009765625, 0.333251953125, 0.5, -7.0],
+        "product": [1.001953125, 1.0, -0.25, -0.0],
     }
     # silu(g) * u with the three fp16 roundings of the models (sigmoid, g * sigmoid, * u) at g = 0: 0 * 0.5 = 0
     cases["silu_mul_zero_gate"] = {"gate": [0.0, 0.0], "up": [3.0, -2.0], "out": [0.0, -0.0]}

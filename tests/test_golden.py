@@ -79,6 +79,14 @@ def test_oracle_special_known_answers():
     x = np.asarray(c["x"], np.float16)
     np.testing.assert_array_equal(OS.reduce_sum(x, 1), np.asarray(c["sum"], np.float16))
     np.testing.assert_array_equal(OS.reduce_max(x, 1), np.asarray(c["max"], np.float16))
+    np.testing.assert_array_equal(OS.reduce_mean(x, 1), np.asarray(c["mean"], np.float16))
+    c = s["mean_roundings"]
+    assert OS.reduce_mean(np.ones((1, c["ones"]), np.float16), 1)[0, 0] == c["ones_mean"]
+    assert OS.reduce_mean(np.full((1, c["halves"]), 0.5, np.float16), 1)[0, 0] == c["halves_mean"]
+    c = s["elementwise"]
+    np.testing.assert_array_equal(OS.sigmoid(np.asarray(c["sigmoid_in"], np.float16)), np.asarray(c["sigmoid_out"], np.float16))
+    got = OS.multiply(np.asarray(c["a"], np.float16), np.asarray(c["b"], np.float16))
+    np.testing.assert_array_equal(got.view(np.uint16), np.asarray(c["product"], np.float16).view(np.uint16))
     c = s["silu_mul_zero_gate"]
     got = OG.silu_mul(np.asarray(c["gate"], np.float16), np.asarray(c["up"], np.float16))
     np.testing.assert_array_equal(got.view(np.uint16), np.asarray(c["out"], np.float16).view(np.uint16))
@@ -152,6 +160,15 @@ def test_hip_special_known_answers(hip):
     x = _t(np.asarray(c["x"], np.float16))
     np.testing.assert_array_equal(F.sum(x, 1).numpy(), np.asarray(c["sum"], np.float16))
     np.testing.assert_array_equal(F.max(x, 1).numpy(), np.asarray(c["max"], np.float16))
+    np.testing.assert_array_equal(F.mean(x, 1).numpy(), np.asarray(c["mean"], np.float16))
+    c = s["mean_roundings"]
+    assert F.mean(_t(np.ones((1, c["ones"]), np.float16)), 1).numpy()[0, 0] == c["ones_mean"]
+    assert F.mean(_t(np.full((1, c["halves"]), 0.5, np.float16)), 1).numpy()[0, 0] == c["halves_mean"]
+    c = s["elementwise"]
+    np.testing.assert_array_equal(F.sigmoid(_t(np.asarray(c["sigmoid_in"], np.float16))).numpy(),
+                                  np.asarray(c["sigmoid_out"], np.float16))
+    got = F.multiply(_t(np.asarray(c["a"], np.float16)), _t(np.asarray(c["b"], np.float16))).numpy()
+    np.testing.assert_array_equal(got.view(np.uint16), np.asarray(c["product"], np.float16).view(np.uint16))
     c = s["silu_mul_zero_gate"]
     g, u = _t(np.asarray(c["gate"], np.float16)), _t(np.asarray(c["up"], np.float16))
     out = HIPTensor.allocate((2,), "float16")
