@@ -273,7 +273,10 @@ size_t mh_llama_scratch_bytes(void* handle, int batch);
  * first step and the last sampled token on return; positions [batch] int32 is
  * where each row's next K/V entry goes and is advanced by one per step;
  * out_tokens (optional) receives [n_steps, batch]; logits_out (optional)
- * receives the last step's fp16 logits [batch, vocab]. */
+ * receives the last step's fp16 logits [batch, vocab].  The caller keeps
+ * positions[b] + n_steps <= max_seq; the kernels clamp a position to
+ * [0, max_seq - 1], so a cache that is full overwrites its last slot (wrong
+ * tokens, no access outside the cache). */
 int mh_llama_decode(void* handle, mh_stream_t stream, int batch, int32_t* tokens, int32_t* positions,
                     int n_steps, int32_t* out_tokens, void* logits_out, void* scratch, size_t scratch_bytes);
 /* The same, with one step recorded into a HIP graph on first use and replayed

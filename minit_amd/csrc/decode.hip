@@ -111,7 +111,7 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(
     half_t* __restrict__ v_cache, int qh, int kvh, int head_dim, int max_seq) {
     const int head = blockIdx.x, b = blockIdx.y;
     const int half_dim = head_dim / 2;
-    const int pos = positions[b];
+    const int pos = min(max(positions[b], 0), max_seq - 1);  // a full cache overwrites its last slot rather than its neighbour
     const half_t* src = qkv + ((size_t)b * (qh + 2 * kvh) + head) * head_dim;
     for (int i = threadIdx.x; i < half_dim; i += blockDim.x) {
         const float re = (float)src[2 * i], im = (float)src[2 * i + 1];
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i16 = lane & 15, kq = lane >> 4;
-    const int len = positions[b] + 1;  // the new token has been appended
+    const int len = min(max(positions[b], 0), max_seq - 1) + 1;  // the new token has been appended
     // chunk starts stay multiples of 64 so that the transposed V reads are 16-byte aligned
     const int span = ((len + splits - 1) / splits + 63) / 64 * 64;
     const int t0 = split * span, t1 = min(len, t0 + span);

@@ -629,7 +629,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 const float4_t sum = sum_splits(partial + (size_t)m * N + c);
                 const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
                 const int head = c / 128, d = c % 128;
-                const int pos = fuse.positions[m];
+                const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
                 if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
                     half_t* dst = fuse.vt_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) *
                                                       fuse.max_seq + pos;

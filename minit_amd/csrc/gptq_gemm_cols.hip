@@ -290,7 +290,7 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     if (epilogue == kEpilogueRopeAppend) {
         // the two columns are one interleaved pair of a head of 128 dims (gptq_common.h)
         const int head = col / 128, d = col % 128;
-        const int pos = fuse.positions[m];
+        const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
         if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
             half_t* dst = fuse.vt_cache +
                           (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void splitk_finalize_rope_kernel(const float* 
     const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
     const int m = (int)(i / N), c = (int)(i % N);
     const int head = c / 128, d = c % 128;
-    const int pos = fuse.positions[m];
+    const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
     if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
         half_t* dst = fuse.vt_cache +
                       (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;

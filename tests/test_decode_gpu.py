@@ -221,3 +221,43 @@ def test_recorded_step_needs_a_stream(hip):
     with pytest.raises(lib.HipError, match="stream"):
         lib.call("mh_llama_decode_graph", dec._handle, None, 1, tok.data_ptr, pos.data_ptr, 1, None, None,
                  scratch._pointer, scratch._size)
+
+
+def test_positions_are_kept_inside_the_cache(hip):
+    """The last slot is usable (positions = max_seq - 1, one step, against the
+    oracle), and a caller that runs past it gets its position clamped: the step
+    completes and the neighbouring head's cache rows keep their contents."""
+    from minit_amd import lib
+    from minit_amd.decode import LlamaDecoder
+    from minit_amd.hip.tensor import HIPTensor
+    batch, max_seq = 2, 64
+    model = _host_model(CFG, seed=77)
+    rng = np.random.default_rng(770)
+    shape = (batch, CFG["n_kv_heads"], max_seq, CFG["head_dim"])
+    k_cache = [rng.normal(0, 1, shape).astype(np.float16) for _ in range(CFG["n_layers"])]
+    v_cache = [rng.normal(0, 1, shape).astype(np.float16) for _ in range(CFG["n_layers"])]
+    tokens = rng.integers(0, CFG["vocab"], batch)
+    positions = np.full(batch, max_seq - 1)
+    dec = LlamaDecoder(CFG, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+    got_tokens, got_logits = dec.decode(tokens, positions, 1, want_logits=True)
+    ref_tokens, ref_logits = OD.greedy(model, tokens, positions, [c.copy() for c in k_cache],
+                                       [c.copy() for c in v_cache], 1)
+    g, r = got_logits.astype(np.float64), ref_logits[-1].astype(np.float64)
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+
+    # two more steps through the C ABI from the last slot: positions 64 and 65 do not exist
+    before = [t.numpy() for t in dec.k_cache + dec.v_cache]
+    tok = HIPTensor.from_numpy(np.asarray(tokens, np.int32))
+    pos = HIPTensor.from_numpy(np.full(batch, max_seq - 1, np.int32))
+    out = HIPTensor.allocate((3, batch), "int32")
+    scratch = dec._scratch_for(batch)
+    lib.call("mh_llama_decode", dec._handle, None, batch, tok.data_ptr, pos.data_ptr, 3, out.data_ptr, None,
+             scratch._pointer, scratch._size)
+    assert ((out.numpy() >= 0) & (out.numpy() < CFG["vocab"])).all()
+    after = [t.numpy() for t in dec.k_cache + dec.v_cache]
+    for l in range(CFG["n_layers"]):
+        kb, ka = before[l], after[l]                      # [B, KVH, T, D]
+        assert np.array_equal(kb[:, :, :max_seq - 1].view(np.uint16), ka[:, :, :max_seq - 1].view(np.uint16))
+        vb, va = before[CFG["n_layers"] + l], after[CFG["n_layers"] + l]   # [B, KVH, D, T]
+        assert np.array_equal(vb[..., :max_seq - 1].view(np.uint16), va[..., :max_seq - 1].view(np.uint16))
