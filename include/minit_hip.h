@@ -77,7 +77,8 @@ int mh_gptq_unpack(mh_stream_t stream, const int32_t* packed, uint8_t* out,
 /* ---- GPTQ dequantize --------------------------------------------------------
  * Replaces dispatch_dequantize (minit/quantize/dispatch.py:14-20) applied to
  * the packed checkpoint tensors: out[k, n] = fp16((q[k,n] - (z[g,n] + 1)) * s[g,n]),
- * g = g_idx[k] (g_idx == NULL means g = k / group_size).
+ * g = g_idx[k] (g_idx == NULL means g = k / group_size; an entry outside
+ * [0, K / group_size) is clamped into it).
  *   qweight int32 [K/P, N] (packed along K), qzeros int32 [G, N/P] (packed
  *   along N), scales fp16 [G, N], g_idx int32 [K] or NULL, out fp16 [K, N];
  *   P = 32 / bits, G = K / group_size.

@@ -52,7 +52,7 @@ __global__ void dequant_kernel(const uint32_t* __restrict__ qweight, const uint3
 #pragma unroll
         for (int i = 0; i < P; ++i) {
             const int k = r * P + i;
-            const int g = g_idx ? g_idx[k] : k / group_size;
+            const int g = g_idx ? min(max(g_idx[k], 0), K / group_size - 1) : k / group_size;  // a bad index reads a wrong group, not outside the tables
             const uint32_t z = (qzeros[(size_t)g * (N / P) + n / P] >> ((n % P) * BITS)) & MASK;
             const half_t s = scales[(size_t)g * N + n];
             out[(size_t)k * N + n] = dequant_one((q >> (i * BITS)) & MASK, z, s);
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void gptq_matmul_generic_kernel(
 #pragma unroll
         for (int i = 0; i < P; ++i) {
             const int k = r * P + i;
-            const int g = g_idx ? g_idx[k] : k / group_size;
+            const int g = g_idx ? min(max(g_idx[k], 0), K / group_size - 1) : k / group_size;  // a bad index reads a wrong group, not outside the tables
             const uint32_t z = (qzeros[(size_t)g * (N / P) + n / P] >> ((n % P) * BITS)) & MASK;
             const half_t w = dequant_one((q >> (i * BITS)) & MASK, z, scales[(size_t)g * N + n]);
             acc = __builtin_fmaf((float)xr[k], (float)w, acc);
