@@ -232,6 +232,14 @@ int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
  * place, one rounding in the storage type like the reference's Add kernel. */
 int mh_add_bias(mh_stream_t stream, void* x, const void* bias, size_t rows, size_t cols, int dtype);
 
+/* Activations in the row order of an act-order weight that was sorted by group
+ * once at load time (the reference gathers scale and zero point per element of K
+ * through g_idx instead, minit/quantize/dispatch.py:16-19; with W_sorted[j] =
+ * W[index[j]] the product x W equals gather(x) W_sorted and W_sorted has
+ * sequential groups): out[r, j] = x[r, index[j]], index int32 [cols], not in place. */
+int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, void* out, size_t rows, size_t cols,
+                      int dtype);
+
 /* ---- Llama-family GPTQ decode loop ------------------------------------------------------
  * The callers around the quantized linears: one greedy decode step per token as
  * the reference's models run it (examples/llama3_70b.py:77-162,215-249;

@@ -420,6 +420,19 @@ __global__ void add_bias_kernel(T* __restrict__ x, const T* __restrict__ bias, s
     }
 }
 
+// out[r, j] = x[r, index[j]]: the activations in the row order of a weight that was
+// sorted by group at load time.  An index outside [0, cols) is clamped.
+template <typename T>
+__global__ void gather_columns_kernel(const T* __restrict__ x, const int32_t* __restrict__ index, T* __restrict__ out,
+                                      size_t rows, size_t cols) {
+    const size_t n = rows * cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / cols, j = i % cols;
+        const int src = min(max(index[j], 0), (int)cols - 1);
+        out[i] = x[r * cols + src];
+    }
+}
+
 #define MH_DISPATCH_DTYPE(dtype, who, CALL)                                         \
     switch (dtype) {                                                                \
         case MH_F16: { typedef half_t T; CALL; }                                    \
@@ -520,6 +533,22 @@ int mh_silu_mul(mh_stream_t stream, const void* gate, const void* up, void* out,
     return MH_OK;
     MH_DISPATCH_DTYPE(dtype, "mh_silu_mul", MH_SILU_CALL);
 #undef MH_SILU_CALL
+}
+
+int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, void* out, size_t rows, size_t cols,
+                      int dtype) {
+    if (rows * cols == 0) return MH_OK;
+    MH_REQUIRE(x && index && out, "mh_gather_columns: null pointer");
+    MH_REQUIRE(x != out, "mh_gather_columns: not in place");
+    MH_REQUIRE(cols <= 0x7fffffffu, "mh_gather_columns: too many columns");
+    const unsigned grid = grid_for(rows * cols, 256);
+#define MH_GATHER_CALL                                                                                          \
+    hipLaunchKernelGGL(gather_columns_kernel<T>, dim3(grid), dim3(256), 0, as_stream(stream), (const T*)x, index, \
+                       (T*)out, rows, cols);                                                                    \
+    MH_CHECK_LAUNCH();                                                                                          \
+    return MH_OK;
+    MH_DISPATCH_DTYPE(dtype, "mh_gather_columns", MH_GATHER_CALL);
+#undef MH_GATHER_CALL
 }
 
 int mh_sigmoid(mh_stream_t stream, const void* in, void* out, size_t n, int dtype) {

@@ -61,6 +61,7 @@ PROTOTYPES = {
     "mh_max": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_mean": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_sigmoid": (c_int, [_P, _P, _P, c_size_t, c_int]),
+    "mh_gather_columns": (c_int, [_P, _P, _P, _P, c_size_t, c_size_t, c_int]),
     "mh_multiply": (c_int, [_P, _P, _P, _P, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
     "mh_add_bias": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_int]),

@@ -27,6 +27,35 @@ def pack_subwords(values: numpy.ndarray, axis: int, bits: int) -> numpy.ndarray:
     return numpy.ascontiguousarray(numpy.moveaxis(out, -1, axis)).view(numpy.int32)
 
 
+def unpack_subwords(packed: numpy.ndarray, axis: int, bits: int) -> numpy.ndarray:
+    """Inverse of :func:`pack_subwords` (examples/qwen1_5_int8.py:40-50): uint8 sub-words."""
+    per_word = 32 // bits
+    w = numpy.moveaxis(numpy.asarray(packed).view(numpy.uint32), axis, -1)
+    shifts = (numpy.arange(per_word, dtype=numpy.uint32) * bits)[None, None, :]
+    v = (w[:, :, None] >> shifts) & numpy.uint32((1 << bits) - 1)
+    v = v.reshape(w.shape[0], w.shape[1] * per_word).astype(numpy.uint8)
+    return numpy.ascontiguousarray(numpy.moveaxis(v, -1, axis))
+
+
+def sort_rows_by_group(qweight: numpy.ndarray, g_idx: numpy.ndarray, bits: int, group_size: int):
+    """One-time repack of an act-order weight: rows of ``W`` stably sorted by their group.
+
+    Returns ``(qweight_sorted, perm)`` with ``W_sorted[j] = W[perm[j]]`` and
+    ``g_idx[perm[j]] == j // group_size``, so ``x @ W == x[:, perm] @ W_sorted``
+    and ``W_sorted`` has sequential groups (the layout the MFMA kernels read).
+    ``None`` when some group does not hold exactly ``group_size`` rows: such a
+    weight stays on the per-element path.
+    """
+    g = numpy.asarray(g_idx, dtype=numpy.int64)
+    k = g.shape[0]
+    counts = numpy.bincount(g, minlength=k // group_size)
+    if counts.shape[0] != k // group_size or (counts != group_size).any():
+        return None
+    perm = numpy.argsort(g, kind="stable").astype(numpy.int32)
+    rows = unpack_subwords(qweight, 0, bits)          # [K, N] uint8
+    return pack_subwords(rows[perm], 0, bits), perm
+
+
 def quantized_tensor_from_host(qweight, qzeros, scales, g_idx=None) -> QuantizedTensor:
     return QuantizedTensor(
         HIPTensor.from_numpy(numpy.ascontiguousarray(qweight)),

@@ -12,25 +12,53 @@ from typing import Optional
 from ..functional.linalg import matrix_multiply
 from ..lib import DTYPE_CODES, call
 from ..hip.tensor import HIPTensor
-from .gptq import quantized_tensor_from_host
+from .gptq import quantized_tensor_from_host, sort_rows_by_group
 from .tensor import QuantizedTensor
 
 
 class QLinear:
-    def __init__(self, weight: QuantizedTensor, bias: Optional[HIPTensor] = None) -> None:
+    def __init__(self, weight: QuantizedTensor, bias: Optional[HIPTensor] = None,
+                 input_order: Optional[HIPTensor] = None) -> None:
+        """``input_order`` (int32 ``[K]``): the activations' columns are gathered in
+        this order before the product (a weight whose rows were sorted by group)."""
         if bias is not None:
             assert tuple(bias._shape) == (weight.out_features,), "bias must have N entries"
             assert bias.dtype == weight._scale.dtype, "bias and scales share one dtype"
+        if input_order is not None:
+            assert tuple(input_order._shape) == (weight.in_features,) and input_order.dtype == "int32"
         self.weight = weight
         self.bias = bias
+        self.input_order = input_order
 
     @classmethod
-    def from_host(cls, w) -> "QLinear":
-        """From :class:`minit_amd.quantize.checkpoint.GPTQLinearWeights`."""
-        weight = quantized_tensor_from_host(w.qweight, w.qzeros, w.scales, w.g_idx)
-        return cls(weight, None if w.bias is None else HIPTensor.from_numpy(w.bias))
+    def from_host(cls, w, reorder: bool = True) -> "QLinear":
+        """From :class:`minit_amd.quantize.checkpoint.GPTQLinearWeights`.
+
+        An act-order weight (``g_idx`` not sequential) is repacked once, rows sorted
+        by group, so that the product runs on the MFMA kernels with the activations
+        gathered to match; ``reorder=False`` (or groups of uneven size) keeps the
+        checkpoint layout and the per-element kernel.
+        """
+        bias = None if w.bias is None else HIPTensor.from_numpy(w.bias)
+        if w.g_idx is not None and reorder:
+            geo = w.geometry
+            packed = sort_rows_by_group(w.qweight, w.g_idx, geo.bits, geo.group_size)
+            if packed is not None:
+                qweight, perm = packed
+                return cls(quantized_tensor_from_host(qweight, w.qzeros, w.scales, None), bias,
+                           HIPTensor.from_numpy(perm))
+        return cls(quantized_tensor_from_host(w.qweight, w.qzeros, w.scales, w.g_idx), bias)
 
     def forward(self, x):
+        if self.input_order is not None:
+            k = self.weight.in_features
+            rows = 1
+            for d in x._shape[:-1]:
+                rows *= d
+            gathered = HIPTensor.allocate(x._shape, x.dtype)
+            call("mh_gather_columns", None, x.data_ptr, self.input_order.data_ptr, gathered.data_ptr, rows, k,
+                 DTYPE_CODES[x.dtype])
+            x = gathered
         out = matrix_multiply(x, self.weight)
         if self.bias is not None:
             n = self.weight.out_features

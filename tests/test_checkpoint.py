@@ -110,7 +110,8 @@ def test_safetensors_files_and_index(tmp_path):
                                                   (1024, 256, 128, 4, True)])
 def test_linear_from_checkpoint_matches_oracle(hip, tmp_path, k, n, g, bits, act_order):
     """File -> QLinear -> forward, bias included, leading axes folded; the act-order
-    checkpoint keeps its g_idx and takes the per-element path."""
+    checkpoint is repacked once (rows sorted by group) and runs on the MFMA kernels
+    with gathered activations."""
     from safetensors.numpy import save_file
     from minit_amd import synthetic
     from minit_amd.hip.tensor import HIPTensor
@@ -119,7 +120,8 @@ def test_linear_from_checkpoint_matches_oracle(hip, tmp_path, k, n, g, bits, act
     path = os.path.join(tmp_path, "w.safetensors")
     save_file(_named("layer.proj", t), path)
     lin = ck.quantized_linear(ck.load_safetensors([path]), "layer.proj")
-    assert (lin.weight._group is not None) == act_order and lin.weight.bits == bits and lin.weight.group_size == g
+    assert lin.weight._group is None and (lin.input_order is not None) == act_order
+    assert lin.weight.bits == bits and lin.weight.group_size == g
     x = synthetic.activations("ckpt", f"x{k}", (2, 3, k))
     y = lin(HIPTensor.from_numpy(x)).numpy()
     assert y.shape == (2, 3, n)
@@ -128,6 +130,53 @@ def test_linear_from_checkpoint_matches_oracle(hip, tmp_path, k, n, g, bits, act
     # the reference adds the bias to the fp16 product, in fp16
     ref = (prod.astype(np.float16).astype(np.float64) + t["bias"].astype(np.float64)).reshape(2, 3, n)
     assert_fp16_close(y, ref, what="checkpoint linear")
+
+
+def test_sort_rows_by_group_is_a_row_permutation_with_sequential_groups():
+    """W_sorted[j] = W[perm[j]] bit for bit (the oracle's act-order dequantization
+    against its sequential one on the repacked words), groups become sequential,
+    and a weight whose groups are of uneven size is left alone."""
+    from minit_amd.quantize.gptq import sort_rows_by_group, unpack_subwords
+    rng = np.random.default_rng(5)
+    for k, n, g, bits in ((512, 24, 128, 4), (256, 16, 64, 8)):
+        t = _linear(rng, k, n, g, bits, act_order=True)
+        qsorted, perm = sort_rows_by_group(t["qweight"], t["g_idx"], bits, g)
+        assert sorted(perm.tolist()) == list(range(k))
+        assert (t["g_idx"][perm] == np.arange(k) // g).all()
+        np.testing.assert_array_equal(unpack_subwords(qsorted, 0, bits), O.unpack(t["qweight"], 0, bits)[perm])
+        w_act = O.dequantize_packed(t["qweight"], t["qzeros"], t["scales"], t["g_idx"], bits, g)
+        w_seq = O.dequantize_packed(qsorted, t["qzeros"], t["scales"], None, bits, g)
+        np.testing.assert_array_equal(w_seq.view(np.uint16), w_act[perm].view(np.uint16))
+    uneven = t["g_idx"].copy()
+    uneven[np.flatnonzero(uneven == 0)[0]] = 1
+    assert sort_rows_by_group(t["qweight"], uneven, bits, g) is None
+
+
+@pytest.mark.gpu
+def test_act_order_repacked_and_per_element_paths_agree(hip):
+    """The same act-order checkpoint with and without the one-time repack, against
+    the oracle; one-hot activations return rows of the dequantized matrix bit for
+    bit on both paths."""
+    from minit_amd import synthetic
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.quantize.linear import QLinear
+    k, n, g, bits = 2048, 1024, 128, 4
+    t = _linear(np.random.default_rng(21), k, n, g, bits, act_order=True, bias=False)
+    w = ck.read_linear(_named("p", t), "p")
+    fast, slow = QLinear.from_host(w), QLinear.from_host(w, reorder=False)
+    assert fast.input_order is not None and slow.input_order is None and slow.weight._group is not None
+    x = synthetic.activations("ckpt", "act", (5, k))
+    ref = O.matmul_f64(x, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], bits, g)
+    dx = HIPTensor.from_numpy(x)
+    assert_fp16_close(fast(dx).numpy(), ref, what="repacked act-order")
+    assert_fp16_close(slow(dx).numpy(), ref, what="per-element act-order")
+    dense = O.dequantize_packed(t["qweight"], t["qzeros"], t["scales"], t["g_idx"], bits, g)
+    rows = [0, 1, k // 2 + 3, k - 2, k - 1]
+    onehot = np.zeros((5, k), np.float16)
+    onehot[np.arange(5), rows] = 1.0
+    dh = HIPTensor.from_numpy(onehot)
+    np.testing.assert_array_equal(fast(dh).numpy().view(np.uint16), dense[rows].view(np.uint16))
+    np.testing.assert_array_equal(slow(dh).numpy().view(np.uint16), dense[rows].view(np.uint16))
 
 
 @pytest.mark.gpu
