@@ -271,3 +271,37 @@ def test_silu_pairs_epilogue(hip, m, k, ffn):
     assert (np.abs(got.astype(np.float64) - ref) <= 1.0 * ulp + slack + 1e-7).all()
     # and the product itself is the oracle's
     assert_fp16_close(y.reshape(m, 2 * ffn), O.matmul_f64(x, qweight, qzeros, scales, None, 4, g), what="gate|up")
+
+
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        bits = int(rng.choice([4, 4, 4, 8]))
+        g = int(rng.choice([32, 64, 128, 128, 256]))
+        k = g * int(rng.integers(1, 9)) * int(rng.choice([1, 2, 4]))
+        n = 8 * int(rng.integers(1, 160))
+        m = int(rng.choice([1, 2, 3, 5, 8, 9, 16, 17, 31, 32, 33, 48, 64, 65, 100, 130]))
+        cases.append((m, k, n, g, bits))
+    return cases
+
+
+@pytest.mark.parametrize("m,k,n,group_size,bits", _random_cases(28, seed=2024))
+def test_random_shapes_match_oracle(hip, m, k, n, group_size, bits):
+    """Seeded sweep over row counts, ragged widths, depths, group sizes and bit
+    widths: whichever kernel the dispatcher picks must agree with the oracle, and
+    one-hot rows must come back as rows of the dequantized matrix bit for bit."""
+    from minit_amd import synthetic
+    qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=1000 + m + k + n,
+                                       zero_range=(0, (1 << bits) - 1))
+    x = synthetic.activations("sweep", f"x{m}_{k}_{n}", (m, k))
+    got = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, group_size, bits)
+    assert_fp16_close(got, O.matmul_f64(x, qweight, qzeros, scales, None, bits, group_size),
+                      what=f"sweep {m}x{k}x{n} g{group_size} b{bits}")
+    rows = np.random.default_rng(m * k + n).integers(0, k, size=m)
+    rows[0] = k - 1
+    onehot = np.zeros((m, k), dtype=np.float16)
+    onehot[np.arange(m), rows] = 1.0
+    got = _run_linear(hip, "mh_gptq_matmul", onehot, qweight, qzeros, scales, group_size, bits)
+    w = O.dequantize_packed(qweight, qzeros, scales, None, bits, group_size)
+    np.testing.assert_array_equal(got.view(np.uint16), w[rows].view(np.uint16))
