@@ -42,6 +42,25 @@ def test_i8_gemm_bit_exact(hip, m, n, k):
     np.testing.assert_array_equal(out.view(np.uint16), ref_out.view(np.uint16))
 
 
+def _sweep(count, seed):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, 400)), int(rng.integers(1, 700)), 64 * int(rng.integers(1, 13)))
+            for _ in range(count)]
+
+
+@pytest.mark.parametrize("m,n,k", _sweep(16, seed=77))
+def test_i8_gemm_random_shapes(hip, m, n, k):
+    """Seeded sweep over ragged M and N (any value, not only multiples of the
+    tile) and over K in both kernels' ranges (64-k and 128-k stages): int32
+    accumulators and the scaled fp16 output bit for bit."""
+    from minit_amd import synthetic
+    a, w, a_scale, w_scale = synthetic.int8_operands(f"i8-sweep-{m}-{n}-{k}", m, n, k)
+    out, acc = _run(hip, a, w, a_scale, w_scale)
+    ref_out, ref_acc = O.gemm(a, w, a_scale, w_scale)
+    np.testing.assert_array_equal(acc, ref_acc)
+    np.testing.assert_array_equal(out.view(np.uint16), ref_out.view(np.uint16))
+
+
 def test_i8_gemm_extreme_values(hip):
     """All operands at +-127 / -128: the largest accumulators the type allows."""
     m, n, k = 64, 64, 4096
