@@ -29,6 +29,8 @@
 // make a second round (10240 columns: 15.9 / 15.0) and gains a little when they
 // are cut along K instead (14.1 / 15.0, see the kernel); with half the CUs idle
 // on a long K (14336x4096: 16.6 / 14.8) it loses.  gemm_cols_preferred decides.
+// 8-bit weights (two packed rows per lane and step): 8192x8192 14.6 / 18.1,
+// 4096x4096 8.4 / 9.9.
 // A wide output (8192x57344, 1792 tiles) stays with the small-M kernel (48 us): one
 // tile per workgroup here takes 60 us, and a variant whose workgroups walked seven
 // tiles as one stream (activations parked in LDS once, the ring running across tile
@@ -315,7 +317,8 @@ constexpr int kColsParts = 4;  // K ranges of a tile that is cut, when there are
 bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_COLS");
     if (off && *off && atoi(off)) return false;
-    if (bits != 4 || group_size != 128 || M < 1 || M > 8) return false;
+    if ((bits != 4 && bits != 8) || M < 1 || M > 8) return false;
+    if (group_size != 32 && group_size != 64 && group_size != 128 && group_size != 256) return false;
     if (N % kColsTile != 0 || K % (32 * kColsStage) != 0) return false;
     return epilogue == kEpilogueNone || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend;
 }
@@ -336,9 +339,11 @@ bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epil
     if (force && *force && atoi(force)) return true;
     const int tiles = N / kColsTile, cus = compute_units();
     static const char* nocut = getenv("MH_GEMM_COLS_NO_CUT");
+    // the thresholds were measured on 4-bit weights; 8-bit rows carry twice the bytes per k
+    const long kb = (long)K * bits / 4;
     // measured at 8192x10240 (320 tiles on 256 CUs): 14.1 against 15.0 us at M = 1, no gain at M = 8
-    if (cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut))) return K <= 8192 && M <= 2;
-    return tiles <= cus && (K <= 8192 || 2 * tiles > cus) && (K <= 16384 || M <= 2);
+    if (cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut))) return kb <= 8192 && M <= 2;
+    return tiles <= cus && (kb <= 8192 || 2 * tiles > cus) && (kb <= 16384 || M <= 2);
 }
 
 // Bytes of workspace a launch of this kernel needs for the shape (0: none).
@@ -371,10 +376,25 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
         partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     }
     const dim3 grid(full_tiles + (tiles - full_tiles) * parts);
-#define MH_LAUNCH_COLS(MROWS)                                                                                     \
-    hipLaunchKernelGGL((gptq_gemm_cols_kernel<4, 4, MROWS>), grid, dim3(512), 0, stream, (const half_t*)x,         \
+#define MH_LAUNCH_COLS_B(BITS, SPG, MROWS)                                                                        \
+    hipLaunchKernelGGL((gptq_gemm_cols_kernel<BITS, SPG, MROWS>), grid, dim3(512), 0, stream, (const half_t*)x,    \
                        (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,    \
                        partial, counters, M, N, K, steps_total, spw, full_tiles, parts, part_spw, epilogue, fuse)
+#define MH_LAUNCH_COLS_S(BITS, MROWS)                        \
+    switch (group_size / 32) {                               \
+        case 1: MH_LAUNCH_COLS_B(BITS, 1, MROWS); break;     \
+        case 2: MH_LAUNCH_COLS_B(BITS, 2, MROWS); break;     \
+        case 4: MH_LAUNCH_COLS_B(BITS, 4, MROWS); break;     \
+        default: MH_LAUNCH_COLS_B(BITS, 8, MROWS); break;    \
+    }
+#define MH_LAUNCH_COLS(MROWS)           \
+    do {                                \
+        if (bits == 4) {                \
+            MH_LAUNCH_COLS_S(4, MROWS)  \
+        } else {                        \
+            MH_LAUNCH_COLS_S(8, MROWS)  \
+        }                               \
+    } while (0)
     if (M == 1)
         MH_LAUNCH_COLS(1);
     else if (M == 2)
@@ -383,6 +403,8 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
         MH_LAUNCH_COLS(4);
     else
         MH_LAUNCH_COLS(8);
+#undef MH_LAUNCH_COLS_B
+#undef MH_LAUNCH_COLS_S
 #undef MH_LAUNCH_COLS
     MH_CHECK_LAUNCH();
     return MH_OK;

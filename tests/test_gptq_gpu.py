@@ -123,24 +123,28 @@ def test_one_hot_rows_are_exact(hip, entry, m, bits):
     np.testing.assert_array_equal(got.view(np.uint16), w[rows].view(np.uint16))
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (1, 4096, 4096), (2, 768, 96), (3, 2304, 160), (5, 1280, 8192),
-                                   (8, 8192, 64), (8, 512, 1024)])
-def test_narrow_outputs_match_oracle(hip, m, k, n):
+@pytest.mark.parametrize("m,k,n,g,bits", [
+    (1, 256, 32, 128, 4), (1, 4096, 4096, 128, 4), (2, 768, 96, 128, 4), (3, 2304, 160, 128, 4),
+    (5, 1280, 8192, 128, 4), (8, 8192, 64, 128, 4), (8, 512, 1024, 128, 4),
+    # 8-bit words (two packed rows per lane and step) and the other group sizes
+    (1, 4096, 4096, 128, 8), (2, 768, 96, 64, 8), (8, 1024, 1024, 256, 8), (4, 512, 2048, 32, 8),
+    (1, 2048, 4096, 32, 4), (3, 2304, 160, 64, 4), (5, 1280, 8192, 256, 4), (8, 768, 512, 64, 4),
+])
+def test_narrow_outputs_match_oracle(hip, m, k, n, g, bits):
     """Shapes served by the kernel whose workgroups own 32 columns over all of K
-    (4 bits, groups of 128, at most 8 rows, K a multiple of 256, N of 32): K ranges
+    (groups of 32 to 256, at most 8 rows, K a multiple of 256, N of 32): K ranges
     that leave waves idle or half used, every zero point, one-hot rows bit for bit."""
     from minit_amd import synthetic
-    g = 128
-    qweight, qzeros, scales = _weights(k, n, g, 4, seed=31, zero_range=(0, 15))
+    qweight, qzeros, scales = _weights(k, n, g, bits, seed=31, zero_range=(0, (1 << bits) - 1))
     x = synthetic.activations("test31", f"x{m}_{k}", (m, k))
-    got = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, 4)
-    assert_fp16_close(got, O.matmul_f64(x, qweight, qzeros, scales, None, 4, g), what=f"narrow {m}x{k}x{n}")
+    got = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, bits)
+    assert_fp16_close(got, O.matmul_f64(x, qweight, qzeros, scales, None, bits, g), what=f"narrow {m}x{k}x{n}")
     rows = np.random.default_rng(32).choice(k, size=m, replace=False)
     rows[0] = k - 1
     onehot = np.zeros((m, k), dtype=np.float16)
     onehot[np.arange(m), rows] = 1.0
-    got = _run_linear(hip, "mh_gptq_matmul", onehot, qweight, qzeros, scales, g, 4)
-    w = O.dequantize_packed(qweight, qzeros, scales, None, 4, g)
+    got = _run_linear(hip, "mh_gptq_matmul", onehot, qweight, qzeros, scales, g, bits)
+    w = O.dequantize_packed(qweight, qzeros, scales, None, bits, g)
     np.testing.assert_array_equal(got.view(np.uint16), w[rows].view(np.uint16))
 
 
