@@ -17,10 +17,10 @@ import numpy as np
 from . import gptq, special
 
 
-def _linear(x, w):
+def _linear(x, w, bits=4):
     """``w`` is ``(qweight, qzeros, scales, group_size)``."""
     qweight, qzeros, scales, group_size = w
-    return gptq.matmul(x, qweight, qzeros, scales, None, 4, group_size)
+    return gptq.matmul(x, qweight, qzeros, scales, None, bits, group_size)
 
 
 def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache: list, v_cache: list):
@@ -29,13 +29,14 @@ def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache:
     qh, kvh, d = cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     rep = qh // kvh
     eps = cfg["rms_eps"]
+    bits = cfg.get("bits", 4)
     b = len(tokens)
     h = model["embed"][tokens].astype(np.float16)                      # [B, H]
     cos, sin = model["cos"], model["sin"]
     inv_sqrt_d = np.float16(np.sqrt(np.float64(d)))
     for l, layer in enumerate(model["layers"]):
         xn = special.rms_norm(h, layer["input_norm"], 1, eps)
-        qkv = _linear(xn, layer["qkv"])
+        qkv = _linear(xn, layer["qkv"], bits)
         q = qkv[:, :qh * d].reshape(b, 1, qh, d)
         k = qkv[:, qh * d:(qh + kvh) * d].reshape(b, 1, kvh, d)
         v = qkv[:, (qh + kvh) * d:].reshape(b, kvh, d)
@@ -55,13 +56,13 @@ def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache:
                 scores = (scores / inv_sqrt_d).astype(np.float16)      # fp16 division
                 probs = special.softmax(scores[None, :], 1)[0]
                 attn[i, j] = (probs.astype(np.float64) @ vv[g]).astype(np.float16)
-        o = _linear(attn.reshape(b, qh * d), layer["o"])
+        o = _linear(attn.reshape(b, qh * d), layer["o"], bits)
         h = h + o                                                      # fp16 add
         xn = special.rms_norm(h, layer["post_norm"], 1, eps)
-        gu = _linear(xn, layer["gate_up"])
+        gu = _linear(xn, layer["gate_up"], bits)
         f = gu.shape[1] // 2
         act = gptq.silu_mul(gu[:, :f], gu[:, f:])
-        h = h + _linear(act, layer["down"])
+        h = h + _linear(act, layer["down"], bits)
     xn = special.rms_norm(h, model["final_norm"], 1, eps)
     return gptq.dense_matmul(xn, model["lm_head"].T.astype(np.float16))
 
