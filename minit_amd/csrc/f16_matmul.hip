@@ -21,32 +21,40 @@ constexpr int kDenseDepth = 8;
 // the a fragment fetched at its point of use, every step waited for the load it
 // had just issued.)  Steps past the end of K re-read the last step and multiply
 // it by a zeroed a fragment.
-template <int MT>
+template <int MT, int NT>
 __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __restrict__ a,
                                                             const half_t* __restrict__ b,
                                                             half_t* __restrict__ out, int M, int N, int K) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i16 = lane & 15, kq = lane >> 4;
-    const int n0 = (blockIdx.x * 4 + wave) * 16;
+    // a wave owns NT groups of 16 output columns: above 16 rows two groups share every
+    // a fragment, which halves the a traffic per byte of b (a comes from the caches,
+    // but through the same vector memory path as b)
+    const int n0 = (blockIdx.x * 4 + wave) * (16 * NT);
     const int m0 = blockIdx.y * (16 * MT);
     if (n0 >= N) return;
-    const int n = min(n0 + i16, N - 1);
-    const half_t* brow = b + (size_t)n * K + kq * 8;
+    const half_t* brow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) brow[nt] = b + (size_t)min(n0 + nt * 16 + i16, N - 1) * K + kq * 8;
     const half_t* arow[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) arow[mt] = a + (size_t)min(m0 + mt * 16 + i16, M - 1) * K + kq * 8;
 
-    float4_t acc[MT];
+    float4_t acc[MT][NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int steps = K / 32;
     const int last = steps - 1;
     constexpr int D = kDenseDepth;
-    uint4_t bq[D], aq[D][MT];
+    uint4_t bq[D][NT], aq[D][MT];
     auto load = [&](int slot, int s) {
         const size_t off = (size_t)min(s, last) * 32;
-        bq[slot] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow + off));
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            bq[slot][nt] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow[nt] + off));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) aq[slot][mt] = *reinterpret_cast<const uint4_t*>(arow[mt] + off);
     };
@@ -56,8 +64,9 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const bool live = s0 + d <= last;
-            const half8_t bf = __builtin_bit_cast(half8_t, bq[d]);
-            half8_t af[MT];
+            half8_t bf[NT], af[MT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) bf[nt] = __builtin_bit_cast(half8_t, bq[d][nt]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 af[mt] = __builtin_bit_cast(half8_t, live ? aq[d][mt] : uint4_t{0u, 0u, 0u, 0u});
@@ -65,17 +74,22 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)  // rows of the result are m (operand A), columns are n (operand B)
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt], bf, acc[mt], 0, 0, 0);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt], bf[nt], acc[mt][nt], 0, 0, 0);
         }
     }
-    // acc[mt][r] is row m0 + mt*16 + kq*4 + r, column n0 + i16
-    if (n0 + i16 < N) {
+    // acc[mt][nt][r] is row m0 + mt*16 + kq*4 + r, column n0 + nt*16 + i16
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n = n0 + nt * 16 + i16;
+        if (n >= N) continue;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = m0 + mt * 16 + kq * 4 + r;
-                if (m < M) out[(size_t)m * N + n0 + i16] = (half_t)acc[mt][r];
+                if (m < M) out[(size_t)m * N + n] = (half_t)acc[mt][nt][r];
             }
     }
 }
@@ -114,12 +128,17 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
         return MH_OK;
     }
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-    dim3 grid((N + 63) / 64, (M + 16 * mt - 1) / (16 * mt));
+    const int nt = mt == 1 ? 1 : 2;  // columns per wave: 16 or 32
+    dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt));
+#define MH_DENSE(MT, NT)                                                                                            \
+    hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT>), grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, \
+                       (half_t*)out, M, N, K)
     switch (mt) {
-        case 1: hipLaunchKernelGGL(f16_matmul_nk_kernel<1>, grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K); break;
-        case 2: hipLaunchKernelGGL(f16_matmul_nk_kernel<2>, grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K); break;
-        default: hipLaunchKernelGGL(f16_matmul_nk_kernel<4>, grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K); break;
+        case 1: MH_DENSE(1, 1); break;
+        case 2: MH_DENSE(2, 2); break;
+        default: MH_DENSE(4, 2); break;
     }
+#undef MH_DENSE
     MH_CHECK_LAUNCH();
     return MH_OK;
 }
