@@ -58,19 +58,30 @@ def _compile_one(hipcc: str, src: str, force: bool, verbose: bool) -> str:
     obj = os.path.join(OBJ_DIR, f"{os.path.splitext(src)[0]}.{_digest(src)}.o")
     if os.path.exists(obj) and not force:
         return obj
-    cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    tmp = obj + ".tmp"
+    cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", tmp]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, obj)  # a cached object is either absent or complete
     return obj
 
 
 def build(force: bool = False, verbose: bool = True, jobs: int = 4) -> str:
-    """Compiles every ``csrc/*.hip`` for gfx950 and links ``libminit_hip.so``."""
-    hipcc = find_hipcc()
+    """Compiles every ``csrc/*.hip`` for gfx950 and links ``libminit_hip.so``.
+
+    One builder at a time (a file lock on the object directory, as the reference
+    guards its kernel cache, minit/compiler/cache.py:8-28)."""
     os.makedirs(OBJ_DIR, exist_ok=True)
+    from filelock import FileLock
+    with FileLock(os.path.join(OBJ_DIR, ".lock")):
+        return _build_locked(force, verbose, jobs)
+
+
+def _build_locked(force: bool, verbose: bool, jobs: int) -> str:
+    hipcc = find_hipcc()
     srcs = sources()
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
         objs = list(pool.map(lambda s: _compile_one(hipcc, s, force, verbose), srcs))
