@@ -65,21 +65,22 @@ def linear_bytes(m, k, n, group=GROUP, bits=BITS):
 class DeviceLinear:
     """One GPTQ weight set generated on the device."""
 
-    def __init__(self, lib, HIPTensor, k, n, seed):
-        per = 32 // BITS
+    def __init__(self, lib, HIPTensor, k, n, seed, bits=BITS):
+        per = 32 // bits
         groups = k // GROUP
-        self.k, self.n = k, n
+        self.k, self.n, self.bits = k, n, bits
         self.qweight = HIPTensor.allocate((k // per, n), "int32")
         self.qzeros = HIPTensor.allocate((groups, n // per), "int32")
         self.scales = HIPTensor.allocate((groups, n), "float16")
+        zlo, zhi = (6, 9) if bits == 4 else (120, 135)
         lib.call("mh_synth_u32", None, self.qweight.data_ptr, (k // per) * n, seed * 3 + 0)
-        lib.call("mh_synth_subwords", None, self.qzeros.data_ptr, groups * (n // per), BITS, 6, 9, seed * 3 + 1)
+        lib.call("mh_synth_subwords", None, self.qzeros.data_ptr, groups * (n // per), bits, zlo, zhi, seed * 3 + 1)
         lib.call("mh_synth_normal", None, self.scales.data_ptr, groups * n, 0.0, 0.02, 1, 1e-3, seed * 3 + 2, 0)
 
 
 def run_gemv(lib, x, lin, out, ws, m=1, entry="mh_gptq_matmul"):
     lib.call(entry, None, x.data_ptr, lin.qweight.data_ptr, lin.qzeros.data_ptr, lin.scales.data_ptr, None,
-             out.data_ptr, m, lin.n, lin.k, GROUP, BITS, ws._pointer, ws._size)
+             out.data_ptr, m, lin.n, lin.k, GROUP, getattr(lin, "bits", BITS), ws._pointer, ws._size)
 
 
 def bench_int8(lib, HIPTensor, memory, n, iters=20):
@@ -433,6 +434,17 @@ def main():
             cached[name] = {"us": round(us, 2), "gbps": round(linear_bytes(1, k, n) / us / 1e3, 1),
                             "weight_mb": round(linear_bytes(1, k, n) / 1e6, 1)}
         result["extra"] = {"gemv_per_shape": per_shape, "gemv_per_shape_cache_resident": cached}
+        if not args.shapes_only:
+            # the same four shapes on 8-bit weights (the bit width the reference's own example ships,
+            # examples/qwen1_5_int8.py): half the arithmetic per byte
+            w8 = {}
+            for j, (name, k, n) in enumerate(LINEARS):
+                sets = [DeviceLinear(lib, HIPTensor, k, n, 900 + 10 * j + i, bits=8) for i in range(3)]
+                ws8 = memory.workspace(max(lib.call("mh_gptq_workspace_bytes", 1, n, k, GROUP, 8), ws._size))
+                us = _time_launches(memory, lambda i: run_gemv(lib, xs[k], sets[i % 3], outs[n], ws8), iters=30, warmup=3)
+                w8[name] = {"us": round(us, 2), "gbps": round(linear_bytes(1, k, n, bits=8) / us / 1e3, 1)}
+                del sets
+            result["extra"]["gemv_w8a16_per_shape"] = w8
         try:
             if not args.shapes_only:
                 result["extra"]["int8_gemm"] = [bench_int8(lib, HIPTensor, memory, n) for n in (4096, 11008)]
