@@ -309,3 +309,47 @@ def test_random_shapes_match_oracle(hip, m, k, n, group_size, bits):
     got = _run_linear(hip, "mh_gptq_matmul", onehot, qweight, qzeros, scales, group_size, bits)
     w = O.dequantize_packed(qweight, qzeros, scales, None, bits, group_size)
     np.testing.assert_array_equal(got.view(np.uint16), w[rows].view(np.uint16))
+
+
+def test_two_streams_with_their_own_workspaces(hip):
+    """Launchers keep no mutable state of their own: products enqueued on two
+    created streams, each with its own workspace, interleaved from one host
+    thread, give the bits of the same calls made one after the other on the null
+    stream (split-K shapes, so the workspaces are in use)."""
+    from minit_amd import synthetic
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    shapes = [(1, 2048, 768, 128, 4), (8, 1024, 1536, 128, 4)]
+    jobs = []
+    for i, (m, k, n, g, bits) in enumerate(shapes):
+        qweight, qzeros, scales = _weights(k, n, g, bits, seed=90 + i)
+        x = synthetic.activations("streams", f"x{i}", (m, k))
+        dev = [_dev(hip, t) for t in (x, qweight, qzeros, scales)]
+        nbytes = max(hip.call("mh_gptq_workspace_bytes", m, n, k, g, bits), 256)
+        ws = HIPTensor.allocate((nbytes,), "int8")
+        ws._memory.reset()
+        jobs.append(dict(m=m, k=k, n=n, g=g, bits=bits, dev=dev, ws=ws, nbytes=nbytes,
+                         out=HIPTensor.allocate((m, n), "float16"), stream=memory.create_stream()))
+    memory.synchronize()
+
+    def launch(job, stream):
+        x, qw, qz, sc = job["dev"]
+        hip.call("mh_gptq_matmul", stream, x.data_ptr, qw.data_ptr, qz.data_ptr, sc.data_ptr, None,
+                 job["out"].data_ptr, job["m"], job["n"], job["k"], job["g"], job["bits"],
+                 job["ws"].data_ptr, job["nbytes"])
+
+    want = []
+    for job in jobs:
+        launch(job, None)
+        memory.synchronize()
+        want.append(job["out"].numpy().copy())
+        job["out"]._memory.reset()
+    memory.synchronize()
+    for _ in range(10):
+        for job in jobs:
+            launch(job, job["stream"])
+    for job in jobs:
+        memory.synchronize(job["stream"])
+    for job, ref in zip(jobs, want):
+        np.testing.assert_array_equal(job["out"].numpy().view(np.uint16), ref.view(np.uint16))
+        hip.call("mh_stream_destroy", job["stream"])
