@@ -157,3 +157,13 @@ def test_prototypes_match_header_argument_counts():
         assert n == len(argtypes), f"{name}: header has {n} parameters, prototype lists {len(argtypes)}"
     for name in decls:
         assert name in lib.PROTOTYPES, f"{name} has no ctypes prototype"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N above 1 exits with a message that says so."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                          text=True, timeout=120)
+    assert proc.returncode != 0 and "one GPU" in proc.stderr and proc.stdout.strip() == ""
