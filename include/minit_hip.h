@@ -254,6 +254,28 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  *   embed, lm_head     fp16 [vocab, hidden]; norms fp16 [hidden]
  *   freqs_cos / sin    fp32 [max_seq, D / 2]
  */
+/* The attention core of one decode step on its own (examples/llama3_70b.py:77-113
+ * for one new token per row: cache append, q.k^T, / sqrt(d), the causal mask --
+ * identically zero here --, softmax, P.V), grouped-query heads sharing one read of
+ * their KV head's cache instead of the reference's 8x head-expanded copies.
+ *   mh_rope_kv_append   qkv fp16 [batch, (QH + 2 KVH) * D] (q heads, then k heads, then
+ *                       v heads): q and k rotated at positions[b] with the interleaved
+ *                       pairs of mh_rope, q to q_out [batch, QH, D], k into k_cache
+ *                       [batch, KVH, max_seq, D] and v into vt_cache [batch, KVH, D,
+ *                       max_seq] at that position (clamped to the cache)
+ *   mh_attn_decode      out[b, h] = softmax(q[b, h] . K[b, h / (QH / KVH), 0..positions[b]] / sqrt(D)) . V,
+ *                       fp32 inside, one rounding; D == 128, QH / KVH in {1, 2, 4, 8};
+ *                       positions[b] is the index of the newest cache entry.  The
+ *                       workspace is zero-filled once by the caller and left with its
+ *                       counters at zero. */
+size_t mh_attn_decode_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int head_dim, int max_seq);
+int mh_attn_decode(mh_stream_t stream, const void* q, const void* k_cache, const void* vt_cache,
+                   const int32_t* positions, void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                   int max_seq, void* workspace, size_t workspace_bytes);
+int mh_rope_kv_append(mh_stream_t stream, const void* qkv, const float* freqs_cos, const float* freqs_sin,
+                      const int32_t* positions, void* q_out, void* k_cache, void* vt_cache, int batch, int n_q_heads,
+                      int n_kv_heads, int head_dim, int max_seq);
+
 typedef struct {
     int n_layers, hidden, n_q_heads, n_kv_heads, head_dim, ffn, vocab;
     int group_size, bits, max_seq;

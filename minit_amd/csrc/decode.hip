@@ -472,15 +472,32 @@ struct Scratch {
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
 
-static int attn_splits(const Llama& m, int batch) {
-    const int pairs = batch * m.cfg.n_kv_heads;
+static int attn_splits(int n_kv_heads, int max_seq, int batch) {
+    const int pairs = batch * n_kv_heads;
     // two blocks per CU: 0.5, 1, 1.5, 4 and 8 measured no faster at any batch size (context 2048)
     int splits = (2 * compute_units() + pairs - 1) / pairs;
     // a block walks 256 positions per pass of its four waves
-    const int max_splits = (m.cfg.max_seq + 255) / 256;
+    const int max_splits = (max_seq + 255) / 256;
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
     return splits < 1 ? 1 : splits;
+}
+static int attn_splits(const Llama& m, int batch) { return attn_splits(m.cfg.n_kv_heads, m.cfg.max_seq, batch); }
+
+// Workspace of a stand-alone attention call: arrival counters (one per row and KV
+// head, zero between calls), then the per-split records.
+static size_t attn_counter_bytes(int batch, int n_kv_heads) { return align_up((size_t)batch * n_kv_heads * sizeof(unsigned)); }
+static size_t attn_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int head_dim, int max_seq) {
+    return attn_counter_bytes(batch, n_kv_heads) +
+           align_up((size_t)batch * n_q_heads * attn_splits(n_kv_heads, max_seq, batch) * (head_dim + 4) * sizeof(float));
+}
+
+template <int G>
+static void launch_attn_raw(hipStream_t st, const half_t* q, const half_t* k_cache, const half_t* vt_cache,
+                            const int32_t* positions, half_t* out, float* partial, unsigned* counters, int batch,
+                            int n_kv_heads, int max_seq, int splits) {
+    hipLaunchKernelGGL((attn_decode_kernel<G, 128>), dim3(splits, n_kv_heads, batch), dim3(256), 0, st, q, k_cache,
+                       vt_cache, positions, out, partial, counters, n_kv_heads, max_seq, 1.0f / sqrtf(128.f), splits);
 }
 
 static Scratch carve(const Llama& m, int batch, char* base) {
@@ -525,10 +542,8 @@ template <int G>
 static void launch_attn(hipStream_t st, const Llama& m, const Scratch& s, const mh_llama_layer& L,
                         const int32_t* positions, int batch, int splits) {
     const mh_llama_config& c = m.cfg;
-    hipLaunchKernelGGL((attn_decode_kernel<G, 128>), dim3(splits, c.n_kv_heads, batch), dim3(256), 0, st,
-                       s.q, (const half_t*)L.k_cache, (const half_t*)L.v_cache, positions, s.attn,
-                       s.attn_partial, s.attn_counters, c.n_kv_heads, c.max_seq,
-                       1.0f / sqrtf((float)c.head_dim), splits);
+    launch_attn_raw<G>(st, s.q, (const half_t*)L.k_cache, (const half_t*)L.v_cache, positions, s.attn, s.attn_partial,
+                       s.attn_counters, batch, c.n_kv_heads, c.max_seq, splits);
 }
 
 }  // namespace mh
@@ -536,6 +551,64 @@ static void launch_attn(hipStream_t st, const Llama& m, const Scratch& s, const 
 using namespace mh;
 
 extern "C" {
+
+size_t mh_attn_decode_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int head_dim, int max_seq) {
+    if (batch <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || head_dim != 128 || max_seq <= 0) return 0;
+    return attn_workspace_bytes(batch, n_q_heads, n_kv_heads, head_dim, max_seq);
+}
+
+int mh_attn_decode(mh_stream_t stream, const void* q, const void* k_cache, const void* vt_cache,
+                   const int32_t* positions, void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                   int max_seq, void* workspace, size_t workspace_bytes) {
+    MH_REQUIRE(batch >= 0, "mh_attn_decode: bad batch %d", batch);
+    if (batch == 0) return MH_OK;
+    MH_REQUIRE(q && k_cache && vt_cache && positions && out, "mh_attn_decode: null pointer");
+    MH_REQUIRE(head_dim == 128, "mh_attn_decode: head_dim must be 128, got %d", head_dim);
+    MH_REQUIRE(n_kv_heads > 0 && n_q_heads % n_kv_heads == 0, "mh_attn_decode: bad head counts %d / %d", n_q_heads,
+               n_kv_heads);
+    const int g = n_q_heads / n_kv_heads;
+    MH_REQUIRE(g == 1 || g == 2 || g == 4 || g == 8, "mh_attn_decode: %d query heads per KV head unsupported", g);
+    MH_REQUIRE(max_seq >= 8 && max_seq % 8 == 0, "mh_attn_decode: max_seq must be a multiple of 8, got %d", max_seq);
+    MH_REQUIRE(((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)vt_cache | (uintptr_t)out) % 16 == 0,
+               "mh_attn_decode: operands must be 16-byte aligned");
+    const size_t need = attn_workspace_bytes(batch, n_q_heads, n_kv_heads, head_dim, max_seq);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(MH_ERR_WORKSPACE, "mh_attn_decode: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    MH_REQUIRE((uintptr_t)workspace % 256 == 0, "mh_attn_decode: workspace must be 256-byte aligned");
+    unsigned* counters = reinterpret_cast<unsigned*>(workspace);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + attn_counter_bytes(batch, n_kv_heads));
+    const int splits = attn_splits(n_kv_heads, max_seq, batch);
+    hipStream_t st = as_stream(stream);
+#define MH_ATTN(G)                                                                                                 \
+    launch_attn_raw<G>(st, (const half_t*)q, (const half_t*)k_cache, (const half_t*)vt_cache, positions, (half_t*)out, \
+                       partial, counters, batch, n_kv_heads, max_seq, splits)
+    switch (g) {
+        case 1: MH_ATTN(1); break;
+        case 2: MH_ATTN(2); break;
+        case 4: MH_ATTN(4); break;
+        default: MH_ATTN(8); break;
+    }
+#undef MH_ATTN
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+int mh_rope_kv_append(mh_stream_t stream, const void* qkv, const float* freqs_cos, const float* freqs_sin,
+                      const int32_t* positions, void* q_out, void* k_cache, void* vt_cache, int batch, int n_q_heads,
+                      int n_kv_heads, int head_dim, int max_seq) {
+    MH_REQUIRE(batch >= 0, "mh_rope_kv_append: bad batch %d", batch);
+    if (batch == 0) return MH_OK;
+    MH_REQUIRE(qkv && freqs_cos && freqs_sin && positions && q_out && k_cache && vt_cache,
+               "mh_rope_kv_append: null pointer");
+    MH_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && n_q_heads > 0 && n_kv_heads > 0 && max_seq > 0,
+               "mh_rope_kv_append: bad sizes");
+    hipLaunchKernelGGL(rope_kv_append_kernel, dim3(n_q_heads + 2 * n_kv_heads, batch), dim3(64), 0, as_stream(stream),
+                       (const half_t*)qkv, freqs_cos, freqs_sin, positions, (half_t*)q_out, (half_t*)k_cache,
+                       (half_t*)vt_cache, n_q_heads, n_kv_heads, head_dim, max_seq);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
 
 int mh_llama_create(void** handle, const mh_llama_config* cfg) {
     MH_REQUIRE(handle && cfg, "mh_llama_create: null argument");

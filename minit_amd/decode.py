@@ -55,6 +55,38 @@ def interleave_gate_up(qweight, qzeros, scales, bits=4):
     return qweight[:, cols], qzeros[:, words], scales[:, cols]
 
 
+def decode_attention(q, k_cache, vt_cache, positions, max_seq: int):
+    """Attention of one new token per row over a preallocated cache (the core of
+    examples/llama3_70b.py:77-113 for a decode step) through ``mh_attn_decode``.
+
+    ``q [B, QH, 128]``, ``k_cache [B, KVH, max_seq, 128]``, ``vt_cache [B, KVH, 128,
+    max_seq]`` (V transposed), ``positions [B]`` int32 = index of the newest entry;
+    all :class:`HIPTensor`.  Returns ``[B, QH, 128]``.
+    """
+    batch, qh, d = q._shape
+    kvh = k_cache._shape[1]
+    nbytes = lib.call("mh_attn_decode_workspace_bytes", batch, qh, kvh, d, max_seq)
+    ws = _attention_workspace(nbytes)
+    out = HIPTensor.allocate((batch, qh, d), q.dtype)
+    lib.call("mh_attn_decode", None, q.data_ptr, k_cache.data_ptr, vt_cache.data_ptr, positions.data_ptr,
+             out.data_ptr, batch, qh, kvh, d, max_seq, ws._pointer, ws._size)
+    return out
+
+
+_ATTN_WS = None
+
+
+def _attention_workspace(nbytes: int):
+    """Zero-filled once; the kernel leaves its counters at zero."""
+    global _ATTN_WS
+    if _ATTN_WS is None or _ATTN_WS._size < nbytes:
+        memory.synchronize()
+        _ATTN_WS = memory.HIPMemory(max(nbytes, 1 << 20))
+        _ATTN_WS.reset()
+        memory.synchronize()
+    return _ATTN_WS
+
+
 class LlamaDecoder:
     """Owns the device tensors of one model and its KV cache."""
 

@@ -65,6 +65,9 @@ PROTOTYPES = {
     "mh_multiply": (c_int, [_P, _P, _P, _P, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
     "mh_add_bias": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_int]),
+    "mh_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "mh_attn_decode": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
+    "mh_rope_kv_append": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int]),
     "mh_llama_create": (c_int, [POINTER(c_void_p), _P]),
     "mh_llama_destroy": (c_int, [_P]),
     "mh_llama_set_layer": (c_int, [_P, c_int, _P]),
@@ -79,7 +82,8 @@ PROTOTYPES = {
 }
 
 # functions whose return value is not a status code
-_NOT_STATUS = {"mh_abi_version", "mh_last_error", "mh_gptq_workspace_bytes", "mh_llama_scratch_bytes"}
+_NOT_STATUS = {"mh_abi_version", "mh_last_error", "mh_gptq_workspace_bytes", "mh_llama_scratch_bytes",
+               "mh_attn_decode_workspace_bytes"}
 
 DTYPE_CODES = {"float16": 0, "bfloat16": 1, "float32": 2}
 

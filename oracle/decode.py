@@ -23,6 +23,32 @@ def _linear(x, w, bits=4):
     return gptq.matmul(x, qweight, qzeros, scales, None, bits, group_size)
 
 
+def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, positions: np.ndarray) -> np.ndarray:
+    """Attention of one new token per row over its cache, examples/llama3_70b.py:95-113.
+
+    ``q [B, QH, D]``, caches ``[B, KVH, T, D]`` with the newest entry at
+    ``positions[b]``; query head j reads KV head ``j // (QH / KVH)``.  Rounded to
+    fp16 where the reference holds an fp16 tensor: the scores, their division by
+    ``sqrt(D)``, the probabilities and the result.  The additive causal mask is zero
+    for a single new token.
+    """
+    b, qh, d = q.shape
+    rep = qh // k_cache.shape[1]
+    sqrt_d = np.float16(np.sqrt(np.float64(d)))
+    out = np.zeros((b, qh, d), np.float16)
+    for i in range(b):
+        p = int(positions[i])
+        kk = k_cache[i, :, :p + 1].astype(np.float64)                  # [KVH, T, D]
+        vv = v_cache[i, :, :p + 1].astype(np.float64)
+        for j in range(qh):
+            g = j // rep
+            scores = (kk[g] @ q[i, j].astype(np.float64)).astype(np.float16)
+            scores = (scores / sqrt_d).astype(np.float16)              # fp16 division
+            probs = special.softmax(scores[None, :], 1)[0]
+            out[i, j] = (probs.astype(np.float64) @ vv[g]).astype(np.float16)
+    return out
+
+
 def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache: list, v_cache: list):
     """Returns fp16 logits ``[B, vocab]``; caches ``[B, KVH, T, D]`` are updated in place."""
     cfg = model["config"]
@@ -43,19 +69,11 @@ def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache:
         pos = positions.reshape(b, 1)
         q = special.rope(q, cos, sin, pos)[:, 0]                       # [B, QH, D]
         k = special.rope(k, cos, sin, pos)[:, 0]                       # [B, KVH, D]
-        attn = np.zeros((b, qh, d), np.float16)
         for i in range(b):
             p = int(positions[i])
             k_cache[l][i, :, p] = k[i]
             v_cache[l][i, :, p] = v[i]
-            kk = k_cache[l][i, :, :p + 1].astype(np.float64)           # [KVH, T, D]
-            vv = v_cache[l][i, :, :p + 1].astype(np.float64)
-            for j in range(qh):
-                g = j // rep
-                scores = (kk[g] @ q[i, j].astype(np.float64)).astype(np.float16)
-                scores = (scores / inv_sqrt_d).astype(np.float16)      # fp16 division
-                probs = special.softmax(scores[None, :], 1)[0]
-                attn[i, j] = (probs.astype(np.float64) @ vv[g]).astype(np.float16)
+        attn = attention(q, k_cache[l], v_cache[l], positions)
         o = _linear(attn.reshape(b, qh * d), layer["o"], bits)
         h = h + o                                                      # fp16 add
         xn = special.rms_norm(h, layer["post_norm"], 1, eps)

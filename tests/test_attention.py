@@ -1,0 +1,117 @@
+"""Decode attention on its own: the restatement is pinned on the CPU by what the
+mathematics fixes, and the HIP entry points (mh_rope_kv_append, mh_attn_decode)
+are checked against it on the GPU.  The device keeps fp32 where the reference
+rounds scores and probabilities to fp16, so outputs are compared under an
+absolute bound of 4e-3 (values are averages of N(0, 1) entries) and a relative
+L2 bound of 5e-3."""
+import numpy as np
+import pytest
+
+from oracle import decode as OD
+from oracle import special as OS
+
+
+def test_oracle_attention_closed_forms():
+    rng = np.random.default_rng(1)
+    b, qh, kvh, t, d = 2, 4, 2, 9, 128
+    q = rng.normal(0, 1, (b, qh, d)).astype(np.float16)
+    k = rng.normal(0, 1, (b, kvh, t, d)).astype(np.float16)
+    v = rng.normal(0, 1, (b, kvh, t, d)).astype(np.float16)
+    pos = np.array([8, 3])
+    out = OD.attention(q, k, v, pos)
+    assert out.shape == (b, qh, d) and out.dtype == np.float16
+    # a single visible entry: the output is that value row, whatever q is
+    one = OD.attention(q, k, v, np.array([0, 0]))
+    for h in range(qh):
+        np.testing.assert_array_equal(one[:, h], v[:, h // 2, 0])
+    # q = 0: uniform weights, the mean of the visible value rows
+    zero = OD.attention(np.zeros_like(q), k, v, pos)
+    for i in range(b):
+        mean = v[i, :, :pos[i] + 1].astype(np.float64).mean(axis=1)
+        np.testing.assert_allclose(zero[i, 0].astype(np.float64), mean[0], atol=2e-3)
+        np.testing.assert_allclose(zero[i, 3].astype(np.float64), mean[1], atol=2e-3)
+    # entries past positions[b] are not read
+    k2, v2 = k.copy(), v.copy()
+    k2[1, :, 4:] = 77
+    v2[1, :, 4:] = -55
+    np.testing.assert_array_equal(OD.attention(q, k2, v2, pos)[1], out[1])
+    # against the float64 form without intermediate rounding
+    for i, h in ((0, 0), (1, 3)):
+        g = h // 2
+        s = k[i, g, :pos[i] + 1].astype(np.float64) @ q[i, h].astype(np.float64) / np.sqrt(d)
+        p = np.exp(s - s.max())
+        ref = (p / p.sum()) @ v[i, g, :pos[i] + 1].astype(np.float64)
+        np.testing.assert_allclose(out[i, h].astype(np.float64), ref, atol=4e-3)
+
+
+def _t(arr):
+    from minit_amd.hip.tensor import HIPTensor
+    return HIPTensor.from_numpy(np.ascontiguousarray(arr))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch,qh,kvh,max_seq,positions", [
+    (1, 8, 1, 64, [0]),                     # one visible entry
+    (3, 8, 2, 320, [5, 255, 319]),          # ragged rows, a chunk boundary, the last slot
+    (2, 64, 8, 2112, [2047, 1000]),         # the 70B head geometry, several splits
+    (5, 4, 4, 128, [17, 64, 63, 127, 1]),   # one query head per KV head
+    (2, 4, 2, 576, [300, 575]),             # two query heads per KV head
+])
+def test_attention_entry_points_match_oracle(hip, batch, qh, kvh, max_seq, positions):
+    from minit_amd.hip.tensor import HIPTensor
+    d = 128
+    rng = np.random.default_rng(batch * 100 + qh)
+    pos = np.asarray(positions, np.int32)
+    k_cache = rng.normal(0, 1, (batch, kvh, max_seq, d)).astype(np.float16)
+    v_cache = rng.normal(0, 1, (batch, kvh, max_seq, d)).astype(np.float16)
+    qkv = rng.normal(0, 1, (batch, (qh + 2 * kvh) * d)).astype(np.float16)
+    cos, sin = OS.rope_tables(d, max_seq, 5e5)
+
+    # oracle: rotate q and k, append k and v at positions[b], attend
+    q_ref = OS.rope(qkv[:, :qh * d].reshape(batch, 1, qh, d), cos, sin, pos.reshape(batch, 1))[:, 0]
+    k_new = OS.rope(qkv[:, qh * d:(qh + kvh) * d].reshape(batch, 1, kvh, d), cos, sin, pos.reshape(batch, 1))[:, 0]
+    v_new = qkv[:, (qh + kvh) * d:].reshape(batch, kvh, d)
+    k_ref, v_ref = k_cache.copy(), v_cache.copy()
+    for i in range(batch):
+        k_ref[i, :, pos[i]] = k_new[i]
+        v_ref[i, :, pos[i]] = v_new[i]
+    ref = OD.attention(q_ref, k_ref, v_ref, pos)
+
+    dk, dvt = _t(k_cache), _t(np.transpose(v_cache, (0, 1, 3, 2)))
+    dq = HIPTensor.allocate((batch, qh, d), "float16")
+    dpos, dqkv, dcos, dsin = _t(pos), _t(qkv), _t(cos), _t(sin)   # named: the buffers must outlive the launch
+    hip.call("mh_rope_kv_append", None, dqkv.data_ptr, dcos.data_ptr, dsin.data_ptr, dpos.data_ptr,
+             dq.data_ptr, dk.data_ptr, dvt.data_ptr, batch, qh, kvh, d, max_seq)
+    # the copy of v is exact; the rotation is fp32 on the device against float64 here, one
+    # rounding each: equal except where the fp32 value sits on a rounding boundary (one step)
+    np.testing.assert_array_equal(dvt.numpy().view(np.uint16), np.transpose(v_ref, (0, 1, 3, 2)).view(np.uint16))
+    for got, want in ((dq.numpy(), q_ref), (dk.numpy(), k_ref)):
+        step = np.spacing(np.abs(want)).astype(np.float64)
+        assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= step).all()
+        assert (got.view(np.uint16) != want.view(np.uint16)).mean() < 1e-3
+
+    nbytes = hip.call("mh_attn_decode_workspace_bytes", batch, qh, kvh, d, max_seq)
+    ws = HIPTensor.allocate((nbytes,), "int8")
+    ws._memory.reset()
+    out = HIPTensor.allocate((batch, qh, d), "float16")
+    for _ in range(2):   # the second call finds the counters as the first one left them
+        hip.call("mh_attn_decode", None, dq.data_ptr, dk.data_ptr, dvt.data_ptr, dpos.data_ptr, out.data_ptr,
+                 batch, qh, kvh, d, max_seq, ws.data_ptr, nbytes)
+    got = out.numpy().astype(np.float64)
+    r = ref.astype(np.float64)
+    assert np.abs(got - r).max() <= 4e-3, np.abs(got - r).max()
+    assert np.linalg.norm(got - r) / np.linalg.norm(r) <= 5e-3
+
+
+@pytest.mark.gpu
+def test_attention_arguments_are_checked(hip):
+    from minit_amd import lib
+    from minit_amd.hip.tensor import HIPTensor
+    t = HIPTensor.allocate((4096,), "float16")
+    with pytest.raises(lib.HipError, match="head_dim"):
+        hip.call("mh_attn_decode", None, t.data_ptr, t.data_ptr, t.data_ptr, t.data_ptr, t.data_ptr, 1, 8, 1, 64, 64,
+                 t.data_ptr, 8192)
+    with pytest.raises(lib.HipError, match="workspace"):
+        hip.call("mh_attn_decode", None, t.data_ptr, t.data_ptr, t.data_ptr, t.data_ptr, t.data_ptr, 1, 8, 1, 128, 64,
+                 None, 0)
+    assert hip.call("mh_attn_decode_workspace_bytes", 1, 8, 1, 64, 64) == 0
