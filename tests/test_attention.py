@@ -97,6 +97,9 @@ def test_attention_entry_points_match_oracle(hip, batch, qh, kvh, max_seq, posit
     for _ in range(2):   # the second call finds the counters as the first one left them
         hip.call("mh_attn_decode", None, dq.data_ptr, dk.data_ptr, dvt.data_ptr, dpos.data_ptr, out.data_ptr,
                  batch, qh, kvh, d, max_seq, ws.data_ptr, nbytes)
+    from minit_amd.decode import decode_attention
+    bound = decode_attention(dq, dk, dvt, dpos, max_seq)      # the Python binding, its own workspace
+    np.testing.assert_array_equal(bound.numpy().view(np.uint16), out.numpy().view(np.uint16))
     got = out.numpy().astype(np.float64)
     r = ref.astype(np.float64)
     assert np.abs(got - r).max() <= 4e-3, np.abs(got - r).max()
