@@ -268,6 +268,10 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  *                       positions[b] is the index of the newest cache entry.  The
  *                       workspace is zero-filled once by the caller and left with its
  *                       counters at zero. */
+/* Greedy sampling on the device: out[r] = index of the first maximum of the fp16
+ * row logits[r, 0..cols) (Top1Sampler, minit/chat/sample.py:11-14, which copies the
+ * row to the host for numpy's argmax); NaN entries are never selected. */
+int mh_argmax(mh_stream_t stream, const void* logits, int32_t* out, int rows, int cols);
 size_t mh_attn_decode_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int head_dim, int max_seq);
 int mh_attn_decode(mh_stream_t stream, const void* q, const void* k_cache, const void* vt_cache,
                    const int32_t* positions, void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,

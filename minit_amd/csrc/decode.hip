@@ -200,9 +200,9 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
         for (int w = 1; w < (int)(blockDim.x >> 6); ++w) consider(sval[w], sidx[w]);
         const int tok = best_i == 0x7fffffff ? 0 : best_i;
         tokens[b] = tok;
-        const int pos = positions[b];
+        const int pos = positions ? positions[b] : 0;  // no positions: a plain row-wise argmax
         if (out_tokens) out_tokens[pos_base ? (size_t)(pos - pos_base[b]) * gridDim.x + b : (size_t)b] = tok;
-        positions[b] = pos + 1;
+        if (positions) positions[b] = pos + 1;
     }
 }
 
@@ -590,6 +590,16 @@ int mh_attn_decode(mh_stream_t stream, const void* q, const void* k_cache, const
         default: MH_ATTN(8); break;
     }
 #undef MH_ATTN
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+int mh_argmax(mh_stream_t stream, const void* logits, int32_t* out, int rows, int cols) {
+    MH_REQUIRE(rows >= 0 && cols > 0, "mh_argmax: bad shape %d x %d", rows, cols);
+    if (rows == 0) return MH_OK;
+    MH_REQUIRE(logits && out, "mh_argmax: null pointer");
+    hipLaunchKernelGGL(argmax_advance_kernel, dim3(rows), dim3(1024), 0, as_stream(stream), (const half_t*)logits, out,
+                       (int32_t*)nullptr, (int32_t*)nullptr, (const int32_t*)nullptr, cols);
     MH_CHECK_LAUNCH();
     return MH_OK;
 }

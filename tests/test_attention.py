@@ -118,3 +118,21 @@ def test_attention_arguments_are_checked(hip):
         hip.call("mh_attn_decode", None, t.data_ptr, t.data_ptr, t.data_ptr, t.data_ptr, t.data_ptr, 1, 8, 1, 128, 64,
                  None, 0)
     assert hip.call("mh_attn_decode_workspace_bytes", 1, 8, 1, 64, 64) == 0
+
+
+@pytest.mark.gpu
+def test_argmax_rows_first_maximum(hip):
+    """mh_argmax against numpy's argmax (first maximum), ties and a vocabulary-sized
+    row with an odd width included."""
+    from minit_amd.hip.tensor import HIPTensor
+    rng = np.random.default_rng(4)
+    for rows, cols in ((1, 7), (3, 1000), (2, 128257), (4, 4096)):
+        x = rng.normal(0, 2, (rows, cols)).astype(np.float16)
+        x[0, cols // 2] = x.max() + 1            # a clear winner
+        if rows > 1:
+            x[1, :] = 0.5                        # all tied: the first index wins
+            x[-1, [cols - 1, cols // 3]] = 60.0  # a two-way tie
+        dx = _t(x)
+        out = HIPTensor.allocate((rows,), "int32")
+        hip.call("mh_argmax", None, dx.data_ptr, out.data_ptr, rows, cols)
+        np.testing.assert_array_equal(out.numpy(), x.argmax(axis=-1).astype(np.int32))
