@@ -268,6 +268,12 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  *                       positions[b] is the index of the newest cache entry.  The
  *                       workspace is zero-filled once by the caller and left with its
  *                       counters at zero. */
+/* The residual add and the norm that follows it in one pass over the row
+ * (examples/llama3_70b.py:159-162: `x = x + attn(...)`, then `norm(x)`): h[r, :] =
+ * fp16(h + delta) in place (skipped when delta is NULL), out[r, :] = RMSNorm(h) *
+ * weight with mh_rms_norm's arithmetic.  fp16, hidden a multiple of 8 up to 8192. */
+int mh_add_rms_norm(mh_stream_t stream, void* h, const void* delta, const void* weight, void* out, int rows,
+                    int hidden, float eps);
 /* Greedy sampling on the device: out[r] = index of the first maximum of the fp16
  * row logits[r, 0..cols) (Top1Sampler, minit/chat/sample.py:11-14, which copies the
  * row to the host for numpy's argmax); NaN entries are never selected. */

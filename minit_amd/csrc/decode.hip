@@ -594,6 +594,21 @@ int mh_attn_decode(mh_stream_t stream, const void* q, const void* k_cache, const
     return MH_OK;
 }
 
+int mh_add_rms_norm(mh_stream_t stream, void* h, const void* delta, const void* weight, void* out, int rows,
+                    int hidden, float eps) {
+    MH_REQUIRE(rows >= 0 && hidden > 0, "mh_add_rms_norm: bad shape %d x %d", rows, hidden);
+    if (rows == 0) return MH_OK;
+    MH_REQUIRE(h && weight && out, "mh_add_rms_norm: null pointer");
+    MH_REQUIRE(hidden % 8 == 0 && hidden <= 8192, "mh_add_rms_norm: hidden must be a multiple of 8 up to 8192, got %d",
+               hidden);
+    MH_REQUIRE(((uintptr_t)h | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) % 16 == 0,
+               "mh_add_rms_norm: operands must be 16-byte aligned");
+    hipLaunchKernelGGL(add_rms_norm_kernel, dim3(rows), dim3(256), 0, as_stream(stream), (half_t*)h, (const half_t*)delta,
+                       (const half_t*)weight, (half_t*)out, hidden, eps);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
 int mh_argmax(mh_stream_t stream, const void* logits, int32_t* out, int rows, int cols) {
     MH_REQUIRE(rows >= 0 && cols > 0, "mh_argmax: bad shape %d x %d", rows, cols);
     if (rows == 0) return MH_OK;

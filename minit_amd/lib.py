@@ -65,6 +65,7 @@ PROTOTYPES = {
     "mh_multiply": (c_int, [_P, _P, _P, _P, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
     "mh_add_bias": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_int]),
+    "mh_add_rms_norm": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_float]),
     "mh_argmax": (c_int, [_P, _P, _P, c_int, c_int]),
     "mh_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "mh_attn_decode": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),

@@ -1,4 +1,5 @@
-"""Decode attention on its own: the restatement is pinned on the CPU by what the
+"""The parts of a decode step as entry points of their own (attention, RoPE and
+cache append, residual add + RMSNorm, greedy sampling).  Decode attention: the restatement is pinned on the CPU by what the
 mathematics fixes, and the HIP entry points (mh_rope_kv_append, mh_attn_decode)
 are checked against it on the GPU.  The device keeps fp32 where the reference
 rounds scores and probabilities to fp16, so outputs are compared under an
@@ -136,3 +137,28 @@ def test_argmax_rows_first_maximum(hip):
         out = HIPTensor.allocate((rows,), "int32")
         hip.call("mh_argmax", None, dx.data_ptr, out.data_ptr, rows, cols)
         np.testing.assert_array_equal(out.numpy(), x.argmax(axis=-1).astype(np.int32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,hidden", [(1, 8192), (5, 4096), (3, 264)])
+def test_add_rms_norm_matches_add_then_norm(hip, rows, hidden):
+    """h + delta rounded to fp16 first (bit for bit against the fp16 sum), then the
+    norm of that sum within one fp16 step of the float64 closed form; delta = NULL
+    leaves h alone."""
+    from minit_amd.hip.tensor import HIPTensor
+    rng = np.random.default_rng(rows + hidden)
+    h = rng.normal(0, 1, (rows, hidden)).astype(np.float16)
+    delta = rng.normal(0, 1, (rows, hidden)).astype(np.float16)
+    w = rng.normal(1, 0.1, hidden).astype(np.float16)
+    dh, dd, dw = _t(h), _t(delta), _t(w)
+    out = HIPTensor.allocate((rows, hidden), "float16")
+    hip.call("mh_add_rms_norm", None, dh.data_ptr, dd.data_ptr, dw.data_ptr, out.data_ptr, rows, hidden, 1e-5)
+    summed = h + delta                                      # numpy fp16 add: one rounding
+    np.testing.assert_array_equal(dh.numpy().view(np.uint16), summed.view(np.uint16))
+    ref = OS.rms_norm(summed, w, 1, 1e-5).astype(np.float64)
+    err = np.abs(out.numpy().astype(np.float64) - ref)
+    assert (err <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + 1e-6).all()
+    hip.call("mh_add_rms_norm", None, dh.data_ptr, None, dw.data_ptr, out.data_ptr, rows, hidden, 1e-5)
+    np.testing.assert_array_equal(dh.numpy().view(np.uint16), summed.view(np.uint16))
+    err = np.abs(out.numpy().astype(np.float64) - ref)
+    assert (err <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + 1e-6).all()
