@@ -63,3 +63,18 @@ def quantized_tensor_from_host(qweight, qzeros, scales, g_idx=None) -> Quantized
         HIPTensor.from_numpy(numpy.ascontiguousarray(qzeros)),
         HIPTensor.from_numpy(numpy.ascontiguousarray(scales)),
     )
+
+
+def quantized_tensor_from_unpacked(data, zero, scales, g_idx=None, bits: int = 8) -> QuantizedTensor:
+    """From the *unpacked* form the reference's ``QuantizedTensor`` holds
+    (examples/qwen1_5_int8.py:276-285: ``data`` uint8 ``[K, N]``, ``zero`` uint8
+    ``[G, N]``, one sub-word per element): packed once on the host into the
+    checkpoint layout the kernels read.  ``data`` / ``zero`` are numpy arrays or
+    device tensors with a ``numpy()`` method.
+    """
+    def host(t):
+        return t.numpy() if hasattr(t, "numpy") else numpy.asarray(t)
+    d, z = host(data), host(zero)
+    assert d.ndim == 2 and z.ndim == 2 and d.shape[1] == z.shape[1], "data [K, N] and zero [G, N] expected"
+    return quantized_tensor_from_host(pack_subwords(d, 0, bits), pack_subwords(z, 1, bits), host(scales),
+                                      None if g_idx is None else host(g_idx))

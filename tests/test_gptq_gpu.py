@@ -353,3 +353,27 @@ def test_two_streams_with_their_own_workspaces(hip):
     for job, ref in zip(jobs, want):
         np.testing.assert_array_equal(job["out"].numpy().view(np.uint16), ref.view(np.uint16))
         hip.call("mh_stream_destroy", job["stream"])
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_quantized_tensor_from_the_reference_s_unpacked_form(hip, bits):
+    """A weight held the way the reference's QuantizedTensor holds it (one uint8
+    per sub-word) is packed once and then behaves like the checkpoint tensors:
+    same product, same dequantized matrix, bit for bit."""
+    import minit_amd.functional as F
+    from minit_amd import synthetic
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.quantize.gptq import quantized_tensor_from_host, quantized_tensor_from_unpacked
+    k, n, g = 512, 264, 128
+    qweight, qzeros, scales = _weights(k, n, g, bits, seed=70 + bits, zero_range=(0, (1 << bits) - 1))
+    data, zero = O.unpack(qweight, 0, bits), O.unpack(qzeros, 1, bits)          # uint8 [K, N], [G, N]
+    a = quantized_tensor_from_unpacked(HIPTensor.from_numpy(data), HIPTensor.from_numpy(zero), scales, bits=bits)
+    b = quantized_tensor_from_host(qweight, qzeros, scales)
+    assert (a.bits, a.group_size, a.in_features, a.out_features) == (bits, g, k, n)
+    np.testing.assert_array_equal(a._data.numpy(), qweight)
+    np.testing.assert_array_equal(a._zero.numpy(), qzeros)
+    x = HIPTensor.from_numpy(synthetic.activations("unpacked", "x", (3, k)))
+    np.testing.assert_array_equal(F.matrix_multiply(x, a).numpy().view(np.uint16),
+                                  F.matrix_multiply(x, b).numpy().view(np.uint16))
+    np.testing.assert_array_equal(a.dequantize().numpy().view(np.uint16),
+                                  O.dequantize_packed(qweight, qzeros, scales, None, bits, g).view(np.uint16))
