@@ -162,3 +162,73 @@ def test_add_rms_norm_matches_add_then_norm(hip, rows, hidden):
     np.testing.assert_array_equal(dh.numpy().view(np.uint16), summed.view(np.uint16))
     err = np.abs(out.numpy().astype(np.float64) - ref)
     assert (err <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + 1e-6).all()
+
+
+@pytest.mark.gpu
+def test_one_step_composed_from_the_operator_api(hip):
+    """One decode step written the way the reference's model code is written -- norm,
+    quantized linears, rotary embedding and cache append, attention, silu(gate) * up
+    as ``x * F.sigmoid(x)``, residual adds, lm_head, argmax -- from the operator API
+    and the stand-alone entry points, against the oracle's step and against the
+    native loop's logits."""
+    import minit_amd.functional as F
+    from minit_amd.decode import LlamaDecoder, decode_attention
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.quantize.gptq import quantized_tensor_from_host
+    from test_decode_gpu import CFG, _host_model
+    cfg = CFG
+    batch, max_seq, context = 3, 64, 23
+    qh, kvh, d, ffn, hidden = cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["ffn"], cfg["hidden"]
+    model = _host_model(cfg, seed=91)
+    rng = np.random.default_rng(910)
+    shape = (batch, kvh, max_seq, d)
+    k_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    v_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    for c in k_cache + v_cache:
+        c[:, :, :context] = rng.normal(0, 1, (batch, kvh, context, d))
+    tokens = rng.integers(0, cfg["vocab"], batch)
+    positions = np.array([context, context - 4, context - 9])
+    ref_logits = OD.decode_step(model, tokens, positions, [c.copy() for c in k_cache], [c.copy() for c in v_cache])
+
+    def qt(w, cols=None):
+        qweight, qzeros, scales, _ = w
+        if cols is not None:
+            lo, hi = cols
+            qweight, qzeros, scales = qweight[:, lo:hi], qzeros[:, lo // 8:hi // 8], scales[:, lo:hi]
+        return quantized_tensor_from_host(*(np.ascontiguousarray(t) for t in (qweight, qzeros, scales)))
+
+    cos, sin = _t(model["cos"]), _t(model["sin"])
+    pos = _t(positions.astype(np.int32))
+    eps = cfg["rms_eps"]
+    h = _t(model["embed"][tokens])
+    xn = F.rms_norm(h, _t(model["layers"][0]["input_norm"]), 1, eps)
+    for l, layer in enumerate(model["layers"]):
+        kc, vt = _t(k_cache[l]), _t(np.transpose(v_cache[l], (0, 1, 3, 2)))
+        qkv = F.matrix_multiply(xn, qt(layer["qkv"]))
+        q = HIPTensor.allocate((batch, qh, d), "float16")
+        hip.call("mh_rope_kv_append", None, qkv.data_ptr, cos.data_ptr, sin.data_ptr, pos.data_ptr, q.data_ptr,
+                 kc.data_ptr, vt.data_ptr, batch, qh, kvh, d, max_seq)
+        attn = decode_attention(q, kc, vt, pos, max_seq)
+        o = F.matrix_multiply(attn.reshape((batch, qh * d)), qt(layer["o"]))
+        post = _t(layer["post_norm"])
+        hip.call("mh_add_rms_norm", None, h.data_ptr, o.data_ptr, post.data_ptr, xn.data_ptr, batch, hidden, eps)
+        gate = F.matrix_multiply(xn, qt(layer["gate_up"], (0, ffn)))
+        up = F.matrix_multiply(xn, qt(layer["gate_up"], (ffn, 2 * ffn)))
+        act = (gate * F.sigmoid(gate)) * up                       # silu(gate) * up as the models spell it
+        down = F.matrix_multiply(act, qt(layer["down"]))
+        nxt = _t(model["layers"][l + 1]["input_norm"] if l + 1 < cfg["n_layers"] else model["final_norm"])
+        hip.call("mh_add_rms_norm", None, h.data_ptr, down.data_ptr, nxt.data_ptr, xn.data_ptr, batch, hidden, eps)
+    logits = F.matrix_multiply(xn, _t(model["lm_head"]))          # dense rule: weight [vocab, hidden]
+    token = HIPTensor.allocate((batch,), "int32")
+    hip.call("mh_argmax", None, logits.data_ptr, token.data_ptr, batch, cfg["vocab"])
+
+    g, r = logits.numpy().astype(np.float64), ref_logits.astype(np.float64)
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+    assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
+    np.testing.assert_array_equal(token.numpy(), logits.numpy().astype(np.float32).argmax(axis=-1))
+
+    dec = LlamaDecoder(cfg, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+    _, native = dec.decode(tokens, positions, 1, want_logits=True)
+    n = native.astype(np.float64)
+    assert np.linalg.norm(g - n) / np.linalg.norm(n) <= 1e-2
