@@ -218,6 +218,9 @@ int mh_mean(mh_stream_t stream, const void* in, void* out, size_t a, size_t b, s
  * element-wise product in T (`{0} * {1}`, :137).  n elements, same shape. */
 int mh_sigmoid(mh_stream_t stream, const void* in, void* out, size_t n, int dtype);
 int mh_multiply(mh_stream_t stream, const void* a, const void* b, void* out, size_t n, int dtype);
+/* The residual add of the models (`x = x + attn(...)`, examples/llama3_70b.py:159-162;
+ * `{0} + {1}` in T, minit/cuda/dispatch.py:135): out = T(a + b), same shape. */
+int mh_add(mh_stream_t stream, const void* a, const void* b, void* out, size_t n, int dtype);
 
 /* silu(gate) * up in one pass (the models run sigmoid, multiply, multiply as
  * three launches: examples/llama3_70b.py:44-45,126-130,

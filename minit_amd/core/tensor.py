@@ -42,6 +42,10 @@ class Tensor(Object):
         from ..functional.special import softmax
         return softmax(self, axis)
 
+    def __add__(self, other: "Tensor"):
+        from ..functional.arith import add
+        return add(self, other)
+
     def __mul__(self, other: "Tensor"):
         from ..functional.arith import multiply
         return multiply(self, other)

@@ -326,10 +326,11 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict_
 // The two element-wise kernels the models' silu uses on its own (examples/llama3_70b.py:
 // 44-45): sigmoid with the reference's expression, 1.0 / (1.0 + expf((float)-x)) in
 // double and one rounding (minit/cuda/dispatch.py:143), and the product in T (:137).
-// OP 0: sigmoid(a); OP 1: a * b.
+// OP 0: sigmoid(a); OP 1: a * b; OP 2: a + b (the residual add, `{0} + {1}`, :135).
 template <typename T, int OP>
 __device__ __forceinline__ float elementwise_one(float a, float b) {
     if (OP == 0) return (float)(1.0 / (1.0 + (double)expf(-a)));  // double -> float -> T rounds like double -> T: 24 >= 2 * 11 + 2
+    if (OP == 2) return a + b;  // fp32 sum of two 16-bit values, rounded to T at the store: the result of a half add
     return a * b;
 }
 
@@ -341,13 +342,13 @@ __global__ void elementwise_kernel(const T* __restrict__ a, const T* __restrict_
     for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
         float x[8], y[8];
         unpack8<T>(reinterpret_cast<const uint4*>(a)[v], x);
-        if (OP == 1) unpack8<T>(reinterpret_cast<const uint4*>(b)[v], y);
+        if (OP != 0) unpack8<T>(reinterpret_cast<const uint4*>(b)[v], y);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = elementwise_one<T, OP>(x[i], OP == 1 ? y[i] : 0.f);
+        for (int i = 0; i < 8; ++i) x[i] = elementwise_one<T, OP>(x[i], OP != 0 ? y[i] : 0.f);
         reinterpret_cast<uint4*>(out)[v] = pack8<T>(x);
     }
     for (size_t j = nvec * 8 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += stride)
-        out[j] = Cvt<T>::from_f32(elementwise_one<T, OP>(Cvt<T>::to_f32(a[j]), OP == 1 ? Cvt<T>::to_f32(b[j]) : 0.f));
+        out[j] = Cvt<T>::from_f32(elementwise_one<T, OP>(Cvt<T>::to_f32(a[j]), OP != 0 ? Cvt<T>::to_f32(b[j]) : 0.f));
 }
 
 static unsigned grid_for(size_t work_items, int per_block) {
@@ -561,6 +562,19 @@ int mh_sigmoid(mh_stream_t stream, const void* in, void* out, size_t n, int dtyp
     MH_CHECK_LAUNCH();                                                                                       \
     return MH_OK;
     MH_DISPATCH_DTYPE(dtype, "mh_sigmoid", MH_EW_CALL);
+#undef MH_EW_CALL
+}
+
+int mh_add(mh_stream_t stream, const void* a, const void* b, void* out, size_t n, int dtype) {
+    if (n == 0) return MH_OK;
+    MH_REQUIRE(a && b && out, "mh_add: null pointer");
+    const unsigned grid = grid_for(n / 8 + 1, 256);
+#define MH_EW_CALL                                                                                          \
+    hipLaunchKernelGGL((elementwise_kernel<T, 2>), dim3(grid), dim3(256), 0, as_stream(stream), (const T*)a, \
+                       (const T*)b, (T*)out, n);                                                            \
+    MH_CHECK_LAUNCH();                                                                                      \
+    return MH_OK;
+    MH_DISPATCH_DTYPE(dtype, "mh_add", MH_EW_CALL);
 #undef MH_EW_CALL
 }
 

@@ -1,4 +1,4 @@
 from .linalg import matrix_multiply
 from .reduce import max, mean, sum
-from .arith import multiply
+from .arith import add, multiply
 from .special import rms_norm, rope, sigmoid, softmax

@@ -7,7 +7,7 @@ against the HIP library.
 from ..core.dispatch import register_dispatch
 from ..core.tensor import Tensor
 from ..lib import DTYPE_CODES, call
-from ..operator import MatrixMultiply, Max, Mean, Multiply, RMSNorm, RoPE, Sigmoid, Softmax, Sum
+from ..operator import Add, MatrixMultiply, Max, Mean, Multiply, RMSNorm, RoPE, Sigmoid, Softmax, Sum
 from ..quantize.operator import Dequantize
 from ..quantize.tensor import QuantizedTensor, _NoGroup
 from . import memory
@@ -136,6 +136,15 @@ def dispatch_multiply(op: Multiply, x: HIPTensor, y: HIPTensor):
     assert x.dtype == y.dtype
     z = HIPTensor.allocate(x._shape, x.dtype)
     call("mh_multiply", None, x.data_ptr, y.data_ptr, z.data_ptr, _count(x._shape), _code(x.dtype))
+    return (z,)
+
+
+@register_dispatch()
+def dispatch_add(op: Add, x: HIPTensor, y: HIPTensor):
+    assert x._shape == y._shape, f"add: shapes {x._shape} and {y._shape} differ"
+    assert x.dtype == y.dtype
+    z = HIPTensor.allocate(x._shape, x.dtype)
+    call("mh_add", None, x.data_ptr, y.data_ptr, z.data_ptr, _count(x._shape), _code(x.dtype))
     return (z,)
 
 

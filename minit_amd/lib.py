@@ -63,6 +63,7 @@ PROTOTYPES = {
     "mh_sigmoid": (c_int, [_P, _P, _P, c_size_t, c_int]),
     "mh_gather_columns": (c_int, [_P, _P, _P, _P, c_size_t, c_size_t, c_int]),
     "mh_multiply": (c_int, [_P, _P, _P, _P, c_size_t, c_int]),
+    "mh_add": (c_int, [_P, _P, _P, _P, c_size_t, c_int]),
     "mh_silu_mul": (c_int, [_P, _P, _P, _P, c_size_t, c_int, c_int]),
     "mh_add_bias": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_int]),
     "mh_add_rms_norm": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_float]),

@@ -26,6 +26,12 @@ class Multiply(Operator):
 
 
 @dataclass
+class Add(Operator):
+    """minit/operator/arith.py (the residual add of the models)."""
+    ...
+
+
+@dataclass
 class RMSNorm(Operator):
     axis: int
     eps: float

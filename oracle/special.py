@@ -118,6 +118,11 @@ def sigmoid(x: np.ndarray) -> np.ndarray:
     return (1.0 / (1.0 + e.astype(np.float64))).astype(x.dtype)
 
 
+def add(x: np.ndarray, y: np.ndarray) -> np.ndarray:
+    """minit/cuda/dispatch.py:135: ``{0} + {1}`` in the storage type (one rounding)."""
+    return (x.astype(np.float64) + y.astype(np.float64)).astype(x.dtype)
+
+
 def multiply(x: np.ndarray, y: np.ndarray) -> np.ndarray:
     """minit/cuda/dispatch.py:137: ``{0} * {1}`` in the storage type (one rounding)."""
     return (x.astype(np.float64) * y.astype(np.float64)).astype(x.dtype)

@@ -218,6 +218,8 @@ def test_one_step_composed_from_the_operator_api(hip):
         down = F.matrix_multiply(act, qt(layer["down"]))
         nxt = _t(model["layers"][l + 1]["input_norm"] if l + 1 < cfg["n_layers"] else model["final_norm"])
         hip.call("mh_add_rms_norm", None, h.data_ptr, down.data_ptr, nxt.data_ptr, xn.data_ptr, batch, hidden, eps)
+    # the residual add also exists as an operator of its own (`x = x + ...` in the models)
+    np.testing.assert_array_equal((h + down).numpy().view(np.uint16), (h.numpy() + down.numpy()).view(np.uint16))
     logits = F.matrix_multiply(xn, _t(model["lm_head"]))          # dense rule: weight [vocab, hidden]
     token = HIPTensor.allocate((batch,), "int32")
     hip.call("mh_argmax", None, logits.data_ptr, token.data_ptr, batch, cfg["vocab"])

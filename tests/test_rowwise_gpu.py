@@ -185,6 +185,9 @@ def test_sigmoid_multiply_compose_to_silu(hip):
     _assert_ulp(h, OG.silu_mul(g, u), ulps=1.0, what="silu through operators")
     with pytest.raises(AssertionError):
         F.multiply(dg, _t(u[:2]))
+    # the residual add: one fp16 rounding, equal to numpy's half add bit for bit
+    np.testing.assert_array_equal((dg + du).numpy().view(np.uint16), (g + u).view(np.uint16))
+    np.testing.assert_array_equal(F.add(dg, du).numpy().view(np.uint16), O.add(g, u).view(np.uint16))
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1000, 512), (8, 128256, 256), (40, 72, 4096), (3, 50, 37)])
