@@ -47,7 +47,7 @@ def _host_model(cfg, seed=0):
             "final_norm": rng.normal(1, 0.1, cfg["hidden"]).astype(np.float16), "cos": cos, "sin": sin}
 
 
-@pytest.mark.parametrize("batch,context", [(1, 17), (3, 40), (9, 12)])  # 9 rows: the unfused path
+@pytest.mark.parametrize("batch,context", [(1, 17), (3, 40), (9, 12), (33, 20)])  # 9 rows: the unfused path; 33: row blocks
 def test_greedy_decode_matches_oracle(hip, batch, context):
     from minit_amd.decode import LlamaDecoder
     model = _host_model(CFG, seed=batch)
