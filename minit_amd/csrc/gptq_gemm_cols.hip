@@ -43,7 +43,8 @@ namespace mh {
 #pragma clang fp contract(off)
 
 constexpr int kColsTile = 32;   // columns per workgroup
-constexpr int kColsWaves = 8;   // K ranges per workgroup (16 measured slower: 8192x8192 10.5 against 10.0 us, 28672x8192 25.0 against 24.5)
+constexpr int kColsWaves = 8;     // K ranges per workgroup (16 measured slower: 8192x8192 10.5 against 10.0 us, 28672x8192 25.0 against 24.5)
+constexpr int kColsCutWaves = 4;  // on the cut plan, where a CU holds a whole tile and a part: plain 8192x10240 12.3 against 14.3 us with 8
 constexpr int kColsStage = 8;   // steps per activation stage
 constexpr int kColsRing = 8;    // steps in flight per wave
 
@@ -58,8 +59,8 @@ __device__ __forceinline__ ColumnConst column_const_from_bits(uint32_t sbits, ui
     return c;
 }
 
-template <int BITS, int SPG, int MROWS>
-__global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
+template <int BITS, int SPG, int MROWS, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* out, float* partial, unsigned* counters, int M, int N, int K,
     int steps_total, int steps_per_wave, int full_tiles, int parts, int part_steps_per_wave, int epilogue,
@@ -76,8 +77,8 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     constexpr int RS = 33;                               // padded row stride of the staging area
     static_assert(R % kColsStage == 0 && R % SPG == 0, "slots must divide the ring");
 
-    __shared__ uint4 xs[kColsWaves][MROWS * RS];
-    __shared__ float red[kColsWaves][MROWS][kColsTile];
+    __shared__ uint4 xs[WAVES][MROWS * RS];
+    __shared__ float red[WAVES][MROWS][kColsTile];
     __shared__ float inv_rms_s[MROWS];
     __shared__ int is_last;
 
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     }
     const int col0 = tile * kColsTile + nl * 2;
 
-    const int begin = (part * kColsWaves + wave) * steps_per_wave;
+    const int begin = (part * WAVES + wave) * steps_per_wave;
     const int end = min(begin + steps_per_wave, steps_total);
     const int last_step = steps_total - 1;
     const int last_stage_step = (last_step / kColsStage) * kColsStage;
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(512) void gptq_gemm_cols_kernel(
     float2 sum = make_float2(0.f, 0.f);
     if (worker) {
 #pragma unroll
-        for (int w = 0; w < kColsWaves; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             const float2 v = *reinterpret_cast<const float2*>(&red[w][m][c]);
             sum.x += v.x;
             sum.y += v.y;
@@ -326,7 +327,12 @@ bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epil
 // Tiles beyond one per CU are cut into kColsParts K ranges, which must not outnumber the CUs.
 static bool cols_cut_plan(int tiles, int K, int cus) {
     return tiles > cus && (tiles - cus) * kColsParts <= cus && tiles - cus < kMaxTileCounters &&
-           K % (32 * kColsStage * kColsWaves * kColsParts) == 0;
+           K % (32 * kColsStage * kColsCutWaves * kColsParts) == 0;
+}
+// The cut plan is taken for one or two rows (measured: no gain at 8 rows).
+static bool cols_use_cut(int M, int tiles, int K, int cus) {
+    static const char* nocut = getenv("MH_GEMM_COLS_NO_CUT");
+    return M <= 2 && cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut));
 }
 
 // Where it measured faster than the small-M kernel: every CU gets at most one
@@ -338,11 +344,10 @@ bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epil
     static const char* force = getenv("MH_GEMM_COLS_FORCE");
     if (force && *force && atoi(force)) return true;
     const int tiles = N / kColsTile, cus = compute_units();
-    static const char* nocut = getenv("MH_GEMM_COLS_NO_CUT");
     // the thresholds were measured on 4-bit weights; 8-bit rows carry twice the bytes per k
     const long kb = (long)K * bits / 4;
-    // measured at 8192x10240 (320 tiles on 256 CUs): 14.1 against 15.0 us at M = 1, no gain at M = 8
-    if (cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut))) return kb <= 8192 && M <= 2;
+    // measured at 8192x10240 (320 tiles on 256 CUs): 12.7 against 15.0 us at M = 1
+    if (cols_use_cut(M, tiles, K, cus)) return kb <= 8192;
     return tiles <= cus && (kb <= 8192 || 2 * tiles > cus) && (kb <= 16384 || M <= 2);
 }
 
@@ -358,28 +363,46 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
     if (!gemm_cols_supported(M, N, K, group_size, bits, epilogue))
         return fail(MH_ERR_INVALID, "gptq column-owner kernel: unsupported shape or fusion");
     const int steps_total = K / 32;
-    int spw = (steps_total + kColsWaves - 1) / kColsWaves;
-    spw = (spw + kColsStage - 1) / kColsStage * kColsStage;  // whole stages, hence whole groups
     const int tiles = N / kColsTile, cus = compute_units();
+    const bool cut = cols_use_cut(M, tiles, K, cus);
+    // four waves for the plain product; with the norm prologue and an epilogue in the reduction (the
+    // decode loop's q|k|v) eight measured faster, 15.0 against 15.4 us
+    const bool cut_w8 = cut && (epilogue != kEpilogueNone || fuse.ssq_in != nullptr) &&
+                        K % (32 * kColsStage * kColsWaves * kColsParts) == 0;
+    const int waves = cut && !cut_w8 ? kColsCutWaves : kColsWaves;
+    int spw = (steps_total + waves - 1) / waves;
+    spw = (spw + kColsStage - 1) / kColsStage * kColsStage;  // whole stages, hence whole groups
     int full_tiles = tiles, parts = 1, part_spw = spw;
     float* partial = nullptr;
     unsigned* counters = nullptr;
-    if (cols_cut_plan(tiles, K, cus)) {
+    if (cut) {
         const size_t need = gemm_cols_workspace_bytes(M, N, K);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
                         workspace ? workspace_bytes : (size_t)0);
         full_tiles = cus;
         parts = kColsParts;
-        part_spw = steps_total / (kColsWaves * kColsParts);
+        part_spw = steps_total / (waves * kColsParts);
         counters = reinterpret_cast<unsigned*>(workspace);
         partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     }
     const dim3 grid(full_tiles + (tiles - full_tiles) * parts);
-#define MH_LAUNCH_COLS_B(BITS, SPG, MROWS)                                                                        \
-    hipLaunchKernelGGL((gptq_gemm_cols_kernel<BITS, SPG, MROWS>), grid, dim3(512), 0, stream, (const half_t*)x,    \
-                       (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, (half_t*)out,    \
-                       partial, counters, M, N, K, steps_total, spw, full_tiles, parts, part_spw, epilogue, fuse)
+#define MH_LAUNCH_COLS_W(BITS, SPG, MROWS, WAVES)                                                                  \
+    hipLaunchKernelGGL((gptq_gemm_cols_kernel<BITS, SPG, MROWS, WAVES>), grid, dim3(WAVES * 64), 0, stream,        \
+                       (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, \
+                       (half_t*)out, partial, counters, M, N, K, steps_total, spw, full_tiles, parts, part_spw,    \
+                       epilogue, fuse)
+// the cut plan runs with one or two rows only
+#define MH_LAUNCH_COLS_B(BITS, SPG, MROWS)                               \
+    do {                                                                 \
+        if constexpr (MROWS <= 2) {                                      \
+            if (cut && !cut_w8) {                                        \
+                MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsCutWaves);       \
+                break;                                                   \
+            }                                                            \
+        }                                                                \
+        MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsWaves);                  \
+    } while (0)
 #define MH_LAUNCH_COLS_S(BITS, MROWS)                        \
     switch (group_size / 32) {                               \
         case 1: MH_LAUNCH_COLS_B(BITS, 1, MROWS); break;     \
@@ -403,6 +426,7 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
         MH_LAUNCH_COLS(4);
     else
         MH_LAUNCH_COLS(8);
+#undef MH_LAUNCH_COLS_W
 #undef MH_LAUNCH_COLS_B
 #undef MH_LAUNCH_COLS_S
 #undef MH_LAUNCH_COLS
