@@ -172,6 +172,31 @@ __device__ __forceinline__ half_t silu_pair(half_t gate, half_t up) {
 // The workspace of the split-K kernels starts with one arrival counter per
 // 256-column tile.  The caller zero-fills the workspace once; every launch
 // leaves the counters at zero again.
+// Sums of squares per piece -> the share of one lane of a 32-lane row group (pieces
+// p0, p0 + 32, ...), added in that order.  The first 256 pieces are requested
+// together (ssq_lane_load) -- a loop that loads and adds per iteration costs one
+// memory round trip per 32 pieces, eight for the 256 pieces a hidden size of 8192
+// leaves -- and may be requested ahead of other loads and summed after them.
+struct SsqLane {
+    float v[8];
+};
+__device__ __forceinline__ SsqLane ssq_lane_load(const float* __restrict__ row, int pieces, int p0) {
+    SsqLane s;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int t = p0 + 32 * j;
+        s.v[j] = t < pieces ? row[t] : 0.f;
+    }
+    return s;
+}
+__device__ __forceinline__ float ssq_lane_sum(const SsqLane& s, const float* __restrict__ row, int pieces, int p0) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += s.v[j];
+    for (int t = p0 + 256; t < pieces; t += 32) ss += row[t];
+    return ss;
+}
+
 constexpr int kMaxTileCounters = 16384;
 constexpr size_t kTileCounterBytes = kMaxTileCounters * sizeof(unsigned);
 

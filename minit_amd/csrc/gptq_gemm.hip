@@ -456,8 +456,10 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         for (int pass = 0; pass < (BM * 32 + 255) / 256; ++pass) {
             const int row = pass * 8 + (tid >> 5), p0 = tid & 31;
             float ss = 0.f;
-            if (row < M)
-                for (int t = p0; t < fuse.ssq_tiles; t += 32) ss += fuse.ssq_in[(size_t)row * fuse.ssq_tiles + t];
+            if (row < M) {
+                const float* pieces = fuse.ssq_in + (size_t)row * fuse.ssq_tiles;
+                ss = ssq_lane_sum(ssq_lane_load(pieces, fuse.ssq_tiles, p0), pieces, fuse.ssq_tiles, p0);
+            }
 #pragma unroll
             for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
             if (p0 == 0 && row < BM) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);

@@ -44,7 +44,8 @@ namespace mh {
 
 constexpr int kColsTile = 32;   // columns per workgroup
 constexpr int kColsWaves = 8;     // K ranges per workgroup (16 measured slower: 8192x8192 10.5 against 10.0 us, 28672x8192 25.0 against 24.5)
-constexpr int kColsCutWaves = 4;  // on the cut plan, where a CU holds a whole tile and a part: plain 8192x10240 12.3 against 14.3 us with 8
+constexpr int kColsCutWaves = 4;  // on the cut plan, where a CU holds a whole tile and a part: 8192x10240 12.3 against 14.3 us with 8
+                                  // (with the norm prologue, RoPE and cache append of the decode loop: 12.1 against 13.6)
 constexpr int kColsStage = 8;   // steps per activation stage
 constexpr int kColsRing = 8;    // steps in flight per wave
 
@@ -169,6 +170,14 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         }
     };
 
+    // the producer's sums of squares (norm prologue) are requested ahead of everything
+    // else, so that waiting for them below leaves the ring in flight
+    const int ssq_row = tid >> 5, ssq_p0 = tid & 31;
+    const bool ssq_mine = fuse.ssq_in != nullptr && ssq_row < M;
+    const float* ssq_pieces = fuse.ssq_in + (size_t)(ssq_mine ? ssq_row : 0) * fuse.ssq_tiles;
+    SsqLane ssq_part = {};
+    if (ssq_mine) ssq_part = ssq_lane_load(ssq_pieces, fuse.ssq_tiles, ssq_p0);
+
     // requests in the order of use
 #pragma unroll
     for (int d = 0; d < R; ++d) {
@@ -180,13 +189,11 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     if (fuse.ssq_in != nullptr) {
         // 1 / rms of the rows from the producer's sums of squares (see SmallFuse): 32
         // lanes per row, folded by shuffles in a fixed order; read after the K loop
-        const int row = tid >> 5, p0 = tid & 31;
         float ss = 0.f;
-        if (row < M)
-            for (int t = p0; t < fuse.ssq_tiles; t += 32) ss += fuse.ssq_in[(size_t)row * fuse.ssq_tiles + t];
+        if (ssq_mine) ss = ssq_lane_sum(ssq_part, ssq_pieces, fuse.ssq_tiles, ssq_p0);
 #pragma unroll
         for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
-        if (p0 == 0 && row < MROWS) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+        if (ssq_p0 == 0 && ssq_row < MROWS) inv_rms_s[ssq_row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
     }
 
     DequantRegs regs;
@@ -365,11 +372,7 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
     const int steps_total = K / 32;
     const int tiles = N / kColsTile, cus = compute_units();
     const bool cut = cols_use_cut(M, tiles, K, cus);
-    // four waves for the plain product; with the norm prologue and an epilogue in the reduction (the
-    // decode loop's q|k|v) eight measured faster, 15.0 against 15.4 us
-    const bool cut_w8 = cut && (epilogue != kEpilogueNone || fuse.ssq_in != nullptr) &&
-                        K % (32 * kColsStage * kColsWaves * kColsParts) == 0;
-    const int waves = cut && !cut_w8 ? kColsCutWaves : kColsWaves;
+    const int waves = cut ? kColsCutWaves : kColsWaves;
     int spw = (steps_total + waves - 1) / waves;
     spw = (spw + kColsStage - 1) / kColsStage * kColsStage;  // whole stages, hence whole groups
     int full_tiles = tiles, parts = 1, part_spw = spw;
@@ -396,7 +399,7 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
 #define MH_LAUNCH_COLS_B(BITS, SPG, MROWS)                               \
     do {                                                                 \
         if constexpr (MROWS <= 2) {                                      \
-            if (cut && !cut_w8) {                                        \
+            if (cut) {                                                   \
                 MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsCutWaves);       \
                 break;                                                   \
             }                                                            \
