@@ -48,6 +48,7 @@ constexpr int kColsCutWaves = 4;  // on the cut plan, where a CU holds a whole t
                                   // (with the norm prologue, RoPE and cache append of the decode loop: 12.1 against 13.6)
 constexpr int kColsStage = 8;   // steps per activation stage
 constexpr int kColsRing = 8;    // steps in flight per wave
+constexpr int kColsParts = 4;  // K ranges of a tile that is cut, when there are more tiles than CUs
 
 // (s, s), (1024 + z + 1) twice, (64 + z + 1) twice from the bits of s and the
 // zero point: below 2048 an fp16 integer n + 1024 is the bit pattern 0x6400 + n,
@@ -178,12 +179,33 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     SsqLane ssq_part = {};
     if (ssq_mine) ssq_part = ssq_lane_load(ssq_pieces, fuse.ssq_tiles, ssq_p0);
 
+    // Operands of the epilogue that do not depend on the product are requested here as
+    // well (the row's position now, what hangs on it after the ring): at the end of
+    // the kernel each would be a dependent round trip on the critical path.
+    const bool ep_worker = tid < M * (kColsTile / 2);  // one thread per (row, column pair) of the tile
+    const int ep_m = tid / (kColsTile / 2), ep_col = tile * kColsTile + tid % (kColsTile / 2) * 2;
+    int ep_pos = 0;
+    if (epilogue == kEpilogueRopeAppend && ep_worker) ep_pos = fuse.positions[ep_m];
+
     // requests in the order of use
 #pragma unroll
     for (int d = 0; d < R; ++d) {
         if (d % kColsStage == 0) load_x(begin + d, d / kColsStage);
         if (d % SPG == 0) load_c(begin + d, d / SPG);
         load_q(begin + d, qb[d]);
+    }
+
+    half2_t ep_h = {(half_t)0.f, (half_t)0.f}, ep_w = {(half_t)0.f, (half_t)0.f};
+    float ep_cos = 0.f, ep_sin = 0.f;
+    if (ep_worker) {
+        if (epilogue == kEpilogueResidual) {
+            ep_h = *reinterpret_cast<const half2_t*>(out + (size_t)ep_m * N + ep_col);
+            if (fuse.xw_out) ep_w = *reinterpret_cast<const half2_t*>(fuse.next_norm_w + ep_col);
+        } else if (epilogue == kEpilogueRopeAppend) {
+            ep_pos = min(max(ep_pos, 0), fuse.max_seq - 1);
+            ep_cos = fuse.rope_cos[(size_t)ep_pos * 64 + ep_col % 128 / 2];
+            ep_sin = fuse.rope_sin[(size_t)ep_pos * 64 + ep_col % 128 / 2];
+        }
     }
 
     if (fuse.ssq_in != nullptr) {
@@ -266,12 +288,20 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         }
         if (!arrive_and_check_last(&counters[tile], (unsigned)nparts, &is_last)) return;
         if (worker) {
-            sum = make_float2(0.f, 0.f);
-            for (int p = 0; p < nparts; ++p) {
-                const float* src = partial + (size_t)p * plane + (size_t)m * N + col;
-                sum.x += load_agent(src);
-                sum.y += load_agent(src + 1);
+            // the parts are requested together and added in part order (nparts is kColsParts here)
+            float2 v[kColsParts];
+#pragma unroll
+            for (int p = 0; p < kColsParts; ++p) {
+                const float* src = partial + (size_t)min(p, nparts - 1) * plane + (size_t)m * N + col;
+                v[p] = make_float2(load_agent(src), load_agent(src + 1));
             }
+            sum = make_float2(0.f, 0.f);
+#pragma unroll
+            for (int p = 0; p < kColsParts; ++p)
+                if (p < nparts) {
+                    sum.x += v[p].x;
+                    sum.y += v[p].y;
+                }
         }
     }
     if (!worker) return;
@@ -286,11 +316,9 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         // out is the residual stream: h += y in fp16, h * next_norm_w for the consumer,
         // and the sum of squares of the tile's 32 new values (the row's 16 threads
         // are adjacent lanes of one wave)
-        const half2_t h = *op + y;
+        const half2_t h = ep_h + y;  // ep_h: this thread's two elements of the stream, read at the start
         *op = h;
-        if (fuse.xw_out)
-            *reinterpret_cast<half2_t*>(fuse.xw_out + (size_t)m * N + col) =
-                h * *reinterpret_cast<const half2_t*>(fuse.next_norm_w + col);
+        if (fuse.xw_out) *reinterpret_cast<half2_t*>(fuse.xw_out + (size_t)m * N + col) = h * ep_w;
         float ss = (float)h[0] * (float)h[0] + (float)h[1] * (float)h[1];
 #pragma unroll
         for (int off = 1; off < kColsTile / 2; off <<= 1) ss += __shfl_xor(ss, off);
@@ -300,7 +328,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     if (epilogue == kEpilogueRopeAppend) {
         // the two columns are one interleaved pair of a head of 128 dims (gptq_common.h)
         const int head = col / 128, d = col % 128;
-        const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
+        const int pos = ep_pos;  // clamped to the cache at the start
         if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
             half_t* dst = fuse.vt_cache +
                           (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;
@@ -308,7 +336,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
             dst[fuse.max_seq] = y[1];
             return;
         }
-        const float cs = fuse.rope_cos[(size_t)pos * 64 + d / 2], sn = fuse.rope_sin[(size_t)pos * 64 + d / 2];
+        const float cs = ep_cos, sn = ep_sin;
         const float re = (float)y[0], im = (float)y[1];
         const half2_t o = {(half_t)(re * cs - im * sn), (half_t)(im * cs + re * sn)};
         half_t* dst = head < fuse.q_heads
@@ -319,8 +347,6 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     }
     *op = y;
 }
-
-constexpr int kColsParts = 4;  // K ranges of a tile that is cut, when there are more tiles than CUs
 
 bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_COLS");
