@@ -611,12 +611,35 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             }
             return s;
         };
+        // two runs of partials (same slots), requested together: one wait instead of two
+        auto sum_splits2 = [&](const float* p, const float* q, float4_t& a, float4_t& b) {
+            constexpr int HALF = BATCH / 2;
+            a = float4_t{0.f, 0.f, 0.f, 0.f};
+            b = a;
+            for (int sp = 0; sp < nseg; sp += HALF) {
+                float4_t v[BATCH];
+#pragma unroll
+                for (int u = 0; u < HALF; ++u) {
+                    const bool live = sp + u < nseg;
+                    v[u] = live ? load_agent4(p + (size_t)(sp + u) * plane) : float4_t{0.f, 0.f, 0.f, 0.f};
+                    v[HALF + u] = live ? load_agent4(q + (size_t)(sp + u) * plane) : float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+                wait_agent_loads(v);
+#pragma unroll
+                for (int u = 0; u < HALF; ++u)
+                    if (sp + u < nseg) {
+                        a += v[u];
+                        b += v[HALF + u];
+                    }
+            }
+        };
         if (epilogue == kEpilogueSiluPairs) {
             // columns [0, 128) of the tile are gate, [128, 256) the matching up columns
             for (int item = tid; item < M * (kGemmCols / 8); item += 256) {
                 const int m = item / (kGemmCols / 8), c4 = item % (kGemmCols / 8) * 4;
                 const float* p = partial + (size_t)m * N + tile * kGemmCols + c4;
-                const float4_t g = sum_splits(p), u = sum_splits(p + kGemmCols / 2);
+                float4_t g, u;
+                sum_splits2(p, p + kGemmCols / 2, g, u);
                 half4_t h;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
@@ -628,19 +651,28 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             // four consecutive columns = two interleaved pairs of one head
             for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
                 const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
-                const float4_t sum = sum_splits(partial + (size_t)m * N + c);
-                const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                // the row's position and its cos/sin are requested before the partials,
+                // whose wait then covers them
                 const int head = c / 128, d = c % 128;
                 const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
-                if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
+                const bool rotated = head < fuse.q_heads + fuse.kv_heads;
+                float cr[2] = {0.f, 0.f}, sr[2] = {0.f, 0.f};
+                if (rotated) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        cr[j] = fuse.rope_cos[(size_t)pos * 64 + d / 2 + j];
+                        sr[j] = fuse.rope_sin[(size_t)pos * 64 + d / 2 + j];
+                    }
+                }
+                const float4_t sum = sum_splits(partial + (size_t)m * N + c);
+                const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                if (!rotated) {  // value head: copied, cache is dim-major
                     half_t* dst = fuse.vt_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) *
                                                       fuse.max_seq + pos;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
                     continue;
                 }
-                const float* cr = fuse.rope_cos + (size_t)pos * 64 + d / 2;
-                const float* sr = fuse.rope_sin + (size_t)pos * 64 + d / 2;
                 half4_t o;
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -662,14 +694,17 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 const int m = base / (kGemmCols / 4) + wave, c = tile * kGemmCols + lane * 4;
                 float ss = 0.f;
                 if (m < M) {
-                    const float4_t s = sum_splits(partial + (size_t)m * N + c);
+                    // the old value of the stream and the next norm's weight are requested
+                    // before the partials, whose wait then covers them
                     half_t* hp = out + (size_t)m * N + c;
+                    const half4_t h_old = *reinterpret_cast<const half4_t*>(hp);
+                    half4_t nw = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+                    if (fuse.xw_out) nw = *reinterpret_cast<const half4_t*>(fuse.next_norm_w + c);
+                    const float4_t s = sum_splits(partial + (size_t)m * N + c);
                     const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
-                    const half4_t h = *reinterpret_cast<const half4_t*>(hp) + y;  // fp16 add, one rounding
+                    const half4_t h = h_old + y;  // fp16 add, one rounding
                     *reinterpret_cast<half4_t*>(hp) = h;
-                    if (fuse.xw_out)
-                        *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) =
-                            h * *reinterpret_cast<const half4_t*>(fuse.next_norm_w + c);
+                    if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) = h * nw;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
                 }
