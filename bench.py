@@ -220,6 +220,21 @@ def bench_small_configs(lib, HIPTensor, memory, ws):
         block.append({"M": m, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
                       "tflops": round(2.0 * m * 3 * hidden * ffn / us / 1e6, 2)})
     res["mlp_block_cfg1"] = block
+    del gate_up, down, halves
+    # the unquantized lm_head of the decode loop: fp16 [vocab, hidden] (2.1 GB, streamed once per launch)
+    vocab, hid = 128256, 8192
+    w = HIPTensor.allocate((vocab, hid), "float16")
+    lib.call("mh_synth_normal", None, w.data_ptr, vocab * hid, 0.0, 0.02, 0, 0.0, 43, 0)
+    head = []
+    for m in (1, 4, 8, 32):
+        x = HIPTensor.allocate((m, hid), "float16")
+        lib.call("mh_synth_normal", None, x.data_ptr, m * hid, 0.0, 1.0, 0, 0.0, 44, 0)
+        y = HIPTensor.allocate((m, vocab), "float16")
+        us = _time_launches(memory, lambda i: lib.call("mh_f16_matmul_nk", None, x.data_ptr, w.data_ptr, y.data_ptr,
+                                                       m, vocab, hid), iters=10, warmup=2)
+        nbytes = 2 * (vocab * hid + m * hid + m * vocab)
+        head.append({"M": m, "us": round(us, 1), "gbps": round(nbytes / us / 1e3, 1)})
+    res["lm_head_f16"] = head
     return res
 
 

@@ -94,6 +94,104 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
     }
 }
 
+// One to four rows of a (decode): a dot-product kernel.  The MFMA kernel above reads b
+// in 64-byte pieces of 16 rows per wave load and leaves most of the MFMA tile empty; here
+// a wave streams whole rows of b, 1 KiB per load (lane l holds k = 512 i + 8 l .. + 8),
+// four rows at a time, against a copy of a in LDS (one 16-byte LDS read per row of a
+// serves the four rows of b), with two steps of loads in flight across the boundaries
+// between row groups.  Products of fp16 pairs are added in fp32 (v_dot2_f32_f16), the
+// 64 lanes' sums by shuffles.  K is a multiple of 1024; a wave owns a contiguous run of
+// row groups.
+constexpr int kGemvRows = 4;  // rows of b per wave and step
+
+template <int MR>
+__global__ __launch_bounds__(256) void f16_gemv_nk_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
+                                                          half_t* __restrict__ out, int M, int N, int K) {
+    extern __shared__ uint4_t gemv_xs[];  // [MR][K / 8]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int k8 = K / 8;
+    for (int i = tid; i < MR * k8; i += 256) {
+        const int m = min(i / k8, M - 1);
+        gemv_xs[i] = *reinterpret_cast<const uint4_t*>(a + (size_t)m * K + (size_t)(i % k8) * 8);
+    }
+    __syncthreads();
+
+    // row groups of this wave: the first `extra` waves of the grid take one more
+    const int groups = (N + kGemvRows - 1) / kGemvRows, waves = gridDim.x * 4, w = blockIdx.x * 4 + wave;
+    const int share = groups / waves, extra = groups % waves;
+    const int first = w * share + min(w, extra), count = share + (w < extra ? 1 : 0);
+    if (count == 0) return;
+    const int kc = K / 512;  // steps per row group (even)
+    const int total = count * kc;
+
+    // (group, step) of the next load, advanced in wave-uniform registers
+    int lg = first, ls = 0, issued = 0;
+    auto load = [&](uint4_t (&q)[kGemvRows]) {
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r) {
+            const int n = min(lg * kGemvRows + r, N - 1);
+            q[r] = __builtin_nontemporal_load(
+                reinterpret_cast<const uint4_t*>(b + (size_t)n * K + (size_t)ls * 512 + lane * 8));
+        }
+        if (++issued < total) {  // past the end the last step is read again and not used
+            if (++ls == kc) {
+                ls = 0;
+                ++lg;
+            }
+        }
+    };
+    float acc[kGemvRows][MR];
+    auto clear = [&]() {
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r)
+#pragma unroll
+            for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
+    };
+    auto consume = [&](const uint4_t (&q)[kGemvRows], int step) {
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const uint4_t xv = gemv_xs[m * k8 + step * 64 + lane];
+            const unsigned int xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int r = 0; r < kGemvRows; ++r) {
+                const unsigned int bw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc[r][m] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, xw[e]),
+                                                       __builtin_bit_cast(half2_t, bw[e]), acc[r][m], false);
+            }
+        }
+    };
+    auto finish = [&](int group) {
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r)
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                const float v = wave_sum(acc[r][m]);
+                const int n = group * kGemvRows + r;
+                if (lane == 0 && m < M && n < N) out[(size_t)m * N + n] = (half_t)v;
+            }
+        clear();
+    };
+
+    uint4_t q0[kGemvRows], q1[kGemvRows];
+    clear();
+    load(q0);
+    int group = first;
+    for (int step = 0, done = 0; done < total; done += 2) {
+        load(q1);
+        consume(q0, step);
+        load(q0);
+        consume(q1, step + 1);
+        step += 2;
+        if (step == kc) {
+            finish(group);
+            step = 0;
+            ++group;
+        }
+    }
+}
+
 // Any K (no divisibility or alignment assumptions): one thread per output.
 __global__ void f16_matmul_nk_generic_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
                                              half_t* __restrict__ out, int M, int N, int K) {
@@ -124,6 +222,25 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
         if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL(f16_matmul_nk_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
                            (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K);
+        MH_CHECK_LAUNCH();
+        return MH_OK;
+    }
+    // one to four rows against a weight with at least one row group per wave: dot products
+    static const char* no_gemv = getenv("MH_F16_NO_GEMV");
+    const int gemv_wgs = compute_units() * 2;
+    if (M <= 4 && K % 1024 == 0 && (size_t)M * K * sizeof(half_t) <= 65536 && N >= gemv_wgs * 4 * kGemvRows &&
+        !(no_gemv && *no_gemv && atoi(no_gemv))) {
+        const int mr = M == 1 ? 1 : M == 2 ? 2 : 4;
+        const size_t lds = (size_t)mr * K * sizeof(half_t);
+#define MH_GEMV(MR)                                                                                              \
+    hipLaunchKernelGGL((f16_gemv_nk_kernel<MR>), dim3(gemv_wgs), dim3(256), lds, st, (const half_t*)a,            \
+                       (const half_t*)b, (half_t*)out, M, N, K)
+        switch (mr) {
+            case 1: MH_GEMV(1); break;
+            case 2: MH_GEMV(2); break;
+            default: MH_GEMV(4); break;
+        }
+#undef MH_GEMV
         MH_CHECK_LAUNCH();
         return MH_OK;
     }

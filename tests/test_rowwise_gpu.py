@@ -190,7 +190,11 @@ def test_sigmoid_multiply_compose_to_silu(hip):
     np.testing.assert_array_equal(F.add(dg, du).numpy().view(np.uint16), O.add(g, u).view(np.uint16))
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 1000, 512), (8, 128256, 256), (40, 72, 4096), (3, 50, 37)])
+@pytest.mark.parametrize("m,n,k", [(1, 1000, 512), (8, 128256, 256), (40, 72, 4096), (3, 50, 37),
+                                   # one to four rows and a tall weight: the dot-product kernel (row groups of
+                                   # four, ragged last group, waves with one group more than others)
+                                   (1, 128256, 1024), (2, 8193, 2048), (3, 9001, 1024), (4, 8192, 8192),
+                                   (1, 8190, 4096)])
 def test_dense_matmul_nk(hip, m, n, k):
     import minit_amd.functional as F
     rng = np.random.default_rng(10)
