@@ -94,30 +94,32 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
     }
 }
 
-// One to four rows of a (decode): a dot-product kernel.  The MFMA kernel above reads b
+// One to eight rows of a (decode): a dot-product kernel.  The MFMA kernel above reads b
 // in 64-byte pieces of 16 rows per wave load and leaves most of the MFMA tile empty; here
 // a wave streams whole rows of b, 1 KiB per load (lane l holds k = 512 i + 8 l .. + 8),
 // four rows at a time, against a copy of a in LDS (one 16-byte LDS read per row of a
 // serves the four rows of b), with two steps of loads in flight across the boundaries
 // between row groups.  Products of fp16 pairs are added in fp32 (v_dot2_f32_f16), the
 // 64 lanes' sums by shuffles.  K is a multiple of 1024; a wave owns a contiguous run of
-// row groups.
+// row groups.  Up to four rows of a: two workgroups of four waves per CU; five to eight
+// rows (up to 128 KiB of LDS): one workgroup of eight waves.
 constexpr int kGemvRows = 4;  // rows of b per wave and step
 
 template <int MR>
-__global__ __launch_bounds__(256) void f16_gemv_nk_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
+__global__ __launch_bounds__(512) void f16_gemv_nk_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
                                                           half_t* __restrict__ out, int M, int N, int K) {
     extern __shared__ uint4_t gemv_xs[];  // [MR][K / 8]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wg_waves = blockDim.x >> 6;
     const int k8 = K / 8;
-    for (int i = tid; i < MR * k8; i += 256) {
+    for (int i = tid; i < MR * k8; i += blockDim.x) {
         const int m = min(i / k8, M - 1);
         gemv_xs[i] = *reinterpret_cast<const uint4_t*>(a + (size_t)m * K + (size_t)(i % k8) * 8);
     }
     __syncthreads();
 
     // row groups of this wave: the first `extra` waves of the grid take one more
-    const int groups = (N + kGemvRows - 1) / kGemvRows, waves = gridDim.x * 4, w = blockIdx.x * 4 + wave;
+    const int groups = (N + kGemvRows - 1) / kGemvRows, waves = gridDim.x * wg_waves, w = blockIdx.x * wg_waves + wave;
     const int share = groups / waves, extra = groups % waves;
     const int first = w * share + min(w, extra), count = share + (w < extra ? 1 : 0);
     if (count == 0) return;
@@ -225,20 +227,26 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
         MH_CHECK_LAUNCH();
         return MH_OK;
     }
-    // one to four rows against a weight with at least one row group per wave: dot products
+    // one to eight rows against a weight with at least one row group per wave: dot products
     static const char* no_gemv = getenv("MH_F16_NO_GEMV");
-    const int gemv_wgs = compute_units() * 2;
-    if (M <= 4 && K % 1024 == 0 && (size_t)M * K * sizeof(half_t) <= 65536 && N >= gemv_wgs * 4 * kGemvRows &&
+    const int mr = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : 8;
+    const size_t lds = (size_t)mr * K * sizeof(half_t);
+    if (M <= 8 && K % 1024 == 0 && lds <= (mr == 8 ? 131072u : 65536u) && N >= compute_units() * 8 * kGemvRows &&
         !(no_gemv && *no_gemv && atoi(no_gemv))) {
-        const int mr = M == 1 ? 1 : M == 2 ? 2 : 4;
-        const size_t lds = (size_t)mr * K * sizeof(half_t);
+        // eight waves per CU either way
+        const int wgs = mr == 8 ? compute_units() : compute_units() * 2, threads = mr == 8 ? 512 : 256;
 #define MH_GEMV(MR)                                                                                              \
-    hipLaunchKernelGGL((f16_gemv_nk_kernel<MR>), dim3(gemv_wgs), dim3(256), lds, st, (const half_t*)a,            \
+    hipLaunchKernelGGL((f16_gemv_nk_kernel<MR>), dim3(wgs), dim3(threads), lds, st, (const half_t*)a,             \
                        (const half_t*)b, (half_t*)out, M, N, K)
         switch (mr) {
             case 1: MH_GEMV(1); break;
             case 2: MH_GEMV(2); break;
-            default: MH_GEMV(4); break;
+            case 4: MH_GEMV(4); break;
+            default:
+                MH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&f16_gemv_nk_kernel<8>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 131072));
+                MH_GEMV(8);
+                break;
         }
 #undef MH_GEMV
         MH_CHECK_LAUNCH();

@@ -193,7 +193,7 @@ def test_sigmoid_multiply_compose_to_silu(hip):
 @pytest.mark.parametrize("m,n,k", [(1, 1000, 512), (8, 128256, 256), (40, 72, 4096), (3, 50, 37),
                                    # one to four rows and a tall weight: the dot-product kernel (row groups of
                                    # four, ragged last group, waves with one group more than others)
-                                   (1, 128256, 1024), (2, 8193, 2048), (3, 9001, 1024), (4, 8192, 8192),
+                                   (1, 128256, 1024), (2, 8193, 2048), (3, 9001, 1024), (4, 8192, 8192), (8, 8200, 8192), (5, 16390, 1024),
                                    (1, 8190, 4096)])
 def test_dense_matmul_nk(hip, m, n, k):
     import minit_amd.functional as F
