@@ -177,3 +177,31 @@ def test_eight_bit_gate_up_shape_one_hot_rows(hip, m):
     hip.call("mh_gptq_dequant", None, qweight.data_ptr, qzeros.data_ptr, scales.data_ptr, None, w.data_ptr, n, k,
              GROUP, bits)
     np.testing.assert_array_equal(out.numpy().view(np.uint16), w.numpy()[rows].view(np.uint16))
+
+
+@pytest.mark.parametrize("m", [1, 4, 8, 32])
+def test_lm_head_shape_dense_product(hip, m):
+    """The unquantized lm_head of the decode loop at its full shape (fp16 [128256, 8192]):
+    one-hot activations return columns of the weight bit for bit (every output index of
+    the dot-product kernel at 1-8 rows and of the MFMA kernel above), and a random
+    activation agrees with float64 on a sample of the outputs."""
+    from minit_amd.hip.tensor import HIPTensor
+    vocab, hidden = 128256, 8192
+    w = HIPTensor.allocate((vocab, hidden), "float16")
+    hip.call("mh_synth_normal", None, w.data_ptr, vocab * hidden, 0.0, 0.05, 0, 0.0, 77, 0)
+    wh = w.numpy()
+    rng = np.random.default_rng(100 + m)
+    ks = rng.choice(hidden, size=m, replace=False)
+    ks[0] = hidden - 1
+    x = np.zeros((m, hidden), dtype=np.float16)
+    x[np.arange(m), ks] = 1.0
+    out = HIPTensor.allocate((m, vocab), "float16")
+    dx = _dev(x)
+    hip.call("mh_f16_matmul_nk", None, dx.data_ptr, w.data_ptr, out.data_ptr, m, vocab, hidden)
+    np.testing.assert_array_equal(out.numpy().view(np.uint16), np.ascontiguousarray(wh[:, ks].T).view(np.uint16))
+    x = rng.normal(0, 1, size=(m, hidden)).astype(np.float16)
+    dx = _dev(x)
+    hip.call("mh_f16_matmul_nk", None, dx.data_ptr, w.data_ptr, out.data_ptr, m, vocab, hidden)
+    cols = np.concatenate([rng.choice(vocab, size=509, replace=False), [0, vocab - 1, vocab - 4]])
+    ref = x.astype(np.float64) @ wh[cols].astype(np.float64).T
+    assert_fp16_close(out.numpy()[:, cols], ref, what="lm_head dense")
