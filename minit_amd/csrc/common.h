@@ -34,6 +34,7 @@ inline hipStream_t as_stream(mh_stream_t s) { return reinterpret_cast<hipStream_
 
 // Number of compute units of the current device (cached per process).
 int compute_units();
+int f16_gemv_prepare();  // f16_matmul.hip: per-device set-up of the eight-row dot-product kernel
 
 typedef _Float16 half_t;
 // Buffer resource word 3 for raw (untyped, offset-addressed) buffer loads on gfx9:

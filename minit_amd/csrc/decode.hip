@@ -645,6 +645,10 @@ int mh_llama_create(void** handle, const mh_llama_config* cfg) {
     MH_REQUIRE(cfg->max_seq >= 8 && cfg->max_seq % 8 == 0, "mh_llama_create: max_seq must be a multiple of 8, got %d", cfg->max_seq);
     MH_REQUIRE(cfg->hidden % 8 == 0 && cfg->hidden <= 8192, "mh_llama_create: hidden must be <= 8192 and a multiple of 8");
     MH_REQUIRE(cfg->ffn % 128 == 0, "mh_llama_create: ffn must be a multiple of 128 (gate/up interleave)");
+    {
+        const int rc = f16_gemv_prepare();  // the lm_head kernel's LDS attribute, ahead of any recording
+        if (rc) return rc;
+    }
     Llama* m = new (std::nothrow) Llama();
     MH_REQUIRE(m != nullptr, "mh_llama_create: out of host memory");
     m->cfg = *cfg;

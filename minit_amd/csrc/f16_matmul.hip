@@ -207,6 +207,20 @@ __global__ void f16_matmul_nk_generic_kernel(const half_t* __restrict__ a, const
     }
 }
 
+// The eight-row dot-product kernel takes more dynamic LDS than a launch may ask for by
+// default: raised once per device.  Callers that record launches into a graph call this
+// beforehand (mh_llama_create does), so that no attribute call falls into a recording.
+int f16_gemv_prepare() {
+    static bool done[64] = {};
+    int dev = 0;
+    MH_CHECK_HIP(hipGetDevice(&dev));
+    if (dev >= 0 && dev < 64 && done[dev]) return MH_OK;
+    MH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&f16_gemv_nk_kernel<8>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 131072));
+    if (dev >= 0 && dev < 64) done[dev] = true;
+    return MH_OK;
+}
+
 }  // namespace mh
 
 using namespace mh;
@@ -242,11 +256,12 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
             case 1: MH_GEMV(1); break;
             case 2: MH_GEMV(2); break;
             case 4: MH_GEMV(4); break;
-            default:
-                MH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&f16_gemv_nk_kernel<8>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 131072));
+            default: {
+                const int rc = f16_gemv_prepare();
+                if (rc) return rc;
                 MH_GEMV(8);
                 break;
+            }
         }
 #undef MH_GEMV
         MH_CHECK_LAUNCH();
