@@ -171,6 +171,33 @@ def bench_rowwise(lib, HIPTensor, memory):
         add(f"softmax [512,{ctx}]", us, 2 * 512 * ctx * 2)
         us = _time_launches(memory, lambda i: lib.call("mh_sum", None, sc.data_ptr, rs.data_ptr, 512, ctx, 1, f16))
         add(f"row_sum [512,{ctx}]", us, 512 * ctx * 2 + 512 * 2)
+    del sc, so, rs
+
+    # The same kernels on operands beyond the 256 MB Infinity Cache (512 MB each): these
+    # lines are the HBM-bound ones.
+    rows, width = 32768, 8192
+    big = HIPTensor.allocate((rows, width), "float16")
+    big_out = HIPTensor.allocate((rows, width), "float16")
+    w8 = HIPTensor.allocate((width,), "float16")
+    col = HIPTensor.allocate((rows, 1), "float16")
+    lib.call("mh_synth_normal", None, big.data_ptr, rows * width, 0.0, 1.0, 0, 0.0, 36, 0)
+    lib.call("mh_synth_normal", None, w8.data_ptr, width, 1.0, 0.1, 0, 0.0, 37, 0)
+    nb = rows * width * 2
+    us = _time_launches(memory, lambda i: lib.call("mh_rms_norm", None, big.data_ptr, w8.data_ptr, big_out.data_ptr,
+                                                    rows, width, 1, 1e-6, f16), iters=20, warmup=3)
+    add(f"rms_norm [{rows},{width}]", us, 2 * nb + width * 2)
+    us = _time_launches(memory, lambda i: lib.call("mh_softmax", None, big.data_ptr, big_out.data_ptr, rows, width, 1,
+                                                    f16), iters=20, warmup=3)
+    add(f"softmax [{rows},{width}]", us, 2 * nb)
+    us = _time_launches(memory, lambda i: lib.call("mh_sum", None, big.data_ptr, col.data_ptr, rows, width, 1, f16),
+                        iters=20, warmup=3)
+    add(f"row_sum [{rows},{width}]", us, nb + rows * 2)
+    toks, heads = rows * width // (64 * 128), 64
+    pos = HIPTensor.from_numpy(np.random.default_rng(38).integers(0, 4096, size=(toks, 1)).astype(np.int32))
+    us = _time_launches(memory, lambda i: lib.call("mh_rope", None, big.data_ptr, dcos.data_ptr, dsin.data_ptr,
+                                                    pos.data_ptr, big_out.data_ptr, toks, 1, heads, 128, f16),
+                        iters=20, warmup=3)
+    add(f"rope [{toks},1,{heads},128]", us, 2 * nb + toks * 64 * 4 * 2)
     return out
 
 
@@ -281,6 +308,8 @@ def main():
                     help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
     ap.add_argument("--int8-library", action="store_true",
                     help="time the vendor library's int8 GEMM (torch._int_mm) on the W8A8 shapes, then exit")
+    ap.add_argument("--rowwise-only", action="store_true",
+                    help="time only the row-wise kernels (RMSNorm, RoPE, softmax, row sum) and print their lines")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the W8A8 GEMM lines (M=2048, K=4096, N in {4096, 11008}), then exit")
     args = ap.parse_args()
@@ -345,6 +374,10 @@ def main():
             res.append({"operands": label, "ms": round(ms, 2), "tops": round(tops, 1),
                         "frac_of_datasheet": round(tops / INT8_PEAK_TOPS, 4)})
         print(json.dumps({"kernel": "i8_mfma_probe_kernel", "waves_per_simd": 2, "results": res}))
+        return
+
+    if args.rowwise_only:
+        print(json.dumps({"rowwise_cfg3": bench_rowwise(lib, HIPTensor, memory)}))
         return
 
     if args.int8_only:
