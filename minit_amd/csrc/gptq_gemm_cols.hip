@@ -381,7 +381,8 @@ bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epil
     const long kb = (long)K * bits / 4;
     // measured at 8192x10240 (320 tiles on 256 CUs): 12.7 against 15.0 us at M = 1
     if (cols_use_cut(M, tiles, K, cus)) return kb <= 8192;
-    return tiles <= cus && (kb <= 8192 || 2 * tiles > cus) && (kb <= 16384 || M <= 2);
+    // 28672x8192 against the small-M kernel: 26.5 / 27.5 us at M = 3, 27.0 / 27.6 at 4, equal at 6, 30.2 / 29.2 at 8
+    return tiles <= cus && (kb <= 8192 || 2 * tiles > cus) && (kb <= 16384 || M <= 4);
 }
 
 // Bytes of workspace a launch of this kernel needs for the shape (0: none).

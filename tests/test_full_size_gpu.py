@@ -105,7 +105,7 @@ class _DeviceLinear:
 
 
 @pytest.mark.parametrize("name,k,n", LLAMA70B_LINEARS)
-@pytest.mark.parametrize("m", [1, 8, 32])
+@pytest.mark.parametrize("m", [1, 4, 8, 32])
 def test_llama70b_linear_one_hot_rows(hip, name, k, n, m):
     """x = e_k returns row k of the dequantized matrix, bit for bit, at full size."""
     lin = _DeviceLinear(hip, k, n, seed=31)
