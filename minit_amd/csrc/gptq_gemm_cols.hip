@@ -362,10 +362,13 @@ static bool cols_cut_plan(int tiles, int K, int cus) {
     return tiles > cus && (tiles - cus) * kColsParts <= cus && tiles - cus < kMaxTileCounters &&
            K % (32 * kColsStage * kColsCutWaves * kColsParts) == 0;
 }
-// The cut plan is taken for one or two rows (measured: no gain at 8 rows).
+// The cut plan is taken at every row count of the kernel (8192x10240 against the small-M
+// kernel: 13.4 / 15.8 us at 3 rows, 14.5 / 16.7 at 8; with eight waves per workgroup it
+// had shown no gain at 8 rows).
 static bool cols_use_cut(int M, int tiles, int K, int cus) {
     static const char* nocut = getenv("MH_GEMM_COLS_NO_CUT");
-    return M <= 2 && cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut));
+    (void)M;
+    return cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut));
 }
 
 // Where it measured faster than the small-M kernel: every CU gets at most one
@@ -422,16 +425,13 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, \
                        (half_t*)out, partial, counters, M, N, K, steps_total, spw, full_tiles, parts, part_spw,    \
                        epilogue, fuse)
-// the cut plan runs with one or two rows only
+// the cut plan runs with kColsCutWaves waves per workgroup
 #define MH_LAUNCH_COLS_B(BITS, SPG, MROWS)                               \
     do {                                                                 \
-        if constexpr (MROWS <= 2) {                                      \
-            if (cut) {                                                   \
-                MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsCutWaves);       \
-                break;                                                   \
-            }                                                            \
-        }                                                                \
-        MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsWaves);                  \
+        if (cut)                                                         \
+            MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsCutWaves);           \
+        else                                                             \
+            MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsWaves);              \
     } while (0)
 #define MH_LAUNCH_COLS_S(BITS, MROWS)                        \
     switch (group_size / 32) {                               \

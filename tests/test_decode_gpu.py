@@ -137,15 +137,16 @@ def test_attention_split_kv_consistency(hip):
     assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
 
 
-def test_decode_wide_qkv_on_cut_tiles(hip):
+@pytest.mark.parametrize("batch", [2, 4, 8])
+def test_decode_wide_qkv_on_cut_tiles(hip, batch):
     """The 70B projection widths (q|k|v 8192 -> 10240: 320 column tiles of 32 on 256
-    CUs, at most two rows): the fused q|k|v product then runs on the column-owner
+    CUs, up to eight rows): the fused q|k|v product then runs on the column-owner
     kernel with the tiles beyond one per CU cut along K, its norm prologue and
     RoPE/cache-append epilogue, and o on the same kernel with the residual epilogue.
     Two layers, so that the second one consumes the first one's sums of squares."""
     from minit_amd.decode import LlamaDecoder
     cfg = dict(CFG, n_layers=2, hidden=8192, n_q_heads=64, n_kv_heads=8, ffn=256, vocab=256)
-    batch, context, max_seq = 2, 10, 64
+    context, max_seq = 10, 64
     model = _host_model(cfg, seed=21)
     # sums over 8192 terms: keep the projections around unit size, or the fp16 scores of the
     # reference's attention (q . k before the 1/sqrt(d) scale) overflow
@@ -160,7 +161,7 @@ def test_decode_wide_qkv_on_cut_tiles(hip):
     for c in k_cache + v_cache:
         c[:, :, :context] = rng.normal(0, 1, (batch, cfg["n_kv_heads"], context, 128))
     tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
-    positions = np.asarray([context, context - 3], np.int32)
+    positions = np.asarray([context, context - 3, context - 1, 0, 7, context, 2, 5][:batch], np.int32)
     dec = LlamaDecoder(cfg, batch, max_seq)
     dec.load_host(model, k_cache, v_cache)
     _, got = dec.decode(tokens, positions, 1, want_logits=True)
