@@ -509,7 +509,7 @@ def main():
             if args.shapes_only:
                 raise RuntimeError("skipped (--shapes-only)")
             from minit_amd import decode
-            result["extra"]["decode_70b"] = decode.bench_tokens_per_second(batches=(1, 8, 32), tokens=16, log=log)
+            result["extra"]["decode_70b"] = decode.bench_tokens_per_second(batches=(1, 8, 32), tokens=128, log=log)
         except Exception as exc:
             result["extra"]["decode_70b_error"] = str(exc)
 
