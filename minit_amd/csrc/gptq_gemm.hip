@@ -884,7 +884,7 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     // the small-M kernel may be asked for an epilogue that goes through the partials even unsplit
     if (slots <= 1 && !use_small(M, group_size)) return 0;
     const size_t small = kTileCounterBytes + (size_t)slots * M * N * sizeof(float);
-    const size_t cols = M <= kFusedReduceMaxM ? gemm_cols_workspace_bytes(M, N, K) : 0;
+    const size_t cols = M <= kSmallMaxM ? gemm_cols_workspace_bytes(M, N, K) : 0;
     return small > cols ? small : cols;
 }
 

@@ -74,10 +74,15 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     constexpr int ROWS_PER_STEP = 32 / P;
     constexpr int LOADS = ROWS_PER_STEP / 4;
     constexpr int CS = R / SPG;                          // scale/zero slots
-    constexpr int XS = R / kColsStage;                   // activation stage slots
-    constexpr int XP = MROWS * 32 > 64 ? MROWS * 32 / 64 : 1;  // 16-byte chunks per lane and stage
-    constexpr int RS = 33;                               // padded row stride of the staging area
-    static_assert(R % kColsStage == 0 && R % SPG == 0, "slots must divide the ring");
+    constexpr int MT = MROWS > 16 ? 2 : 1;               // 16-row tiles of the activations
+    constexpr int STAGE = MROWS > 16 ? 4 : kColsStage;   // steps per activation stage (LDS: rows x stage per wave)
+    constexpr int CH = STAGE * 4;                        // 16-byte chunks per row and stage
+    constexpr int XS = R / STAGE;                        // activation stage slots
+    constexpr int XP = MROWS * CH > 64 ? MROWS * CH / 64 : 1;  // 16-byte chunks per lane and stage
+    constexpr int RS = CH + 1;                           // padded row stride of the staging area
+    constexpr int SSQ_ROWS = (MROWS * 32 + WAVES * 64 - 1) / (WAVES * 64);  // rows per 32 threads, norm prologue
+    static_assert(R % STAGE == 0 && R % SPG == 0 && kColsStage % STAGE == 0, "slots must divide the ring");
+    static_assert(MROWS * (kColsTile / 2) <= WAVES * 64, "one thread per row and column pair");
 
     __shared__ uint4 xs[WAVES][MROWS * RS];
     __shared__ float red[WAVES][MROWS][kColsTile];
@@ -106,7 +111,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     const int begin = (part * WAVES + wave) * steps_per_wave;
     const int end = min(begin + steps_per_wave, steps_total);
     const int last_step = steps_total - 1;
-    const int last_stage_step = (last_step / kColsStage) * kColsStage;
+    const int last_stage_step = (last_step / STAGE) * STAGE;
     const int ring_last = max(min(end, steps_total) - 1, 0);
 
     // ---- packed weights
@@ -144,8 +149,8 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
 #pragma unroll
     for (int u = 0; u < XP; ++u) {
         const int item = u * 64 + lane;
-        x_row[u] = min(item / 32, M - 1);
-        x_chunk[u] = item % 32;
+        x_row[u] = min(item / CH, M - 1);
+        x_chunk[u] = item % CH;
     }
     auto load_x = [&](int step, int slot) {
         const int s = min(step, last_stage_step);
@@ -165,19 +170,26 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
                 pair_activations<8>(in + 2, o + 2);
             }
             const bool live = step + x_chunk[u] / 4 < end;  // steps of another wave or past K add nothing
-            if (u * 64 + lane < MROWS * 32)
-                xs[wave][(u * 64 + lane) / 32 * RS + x_chunk[u]] =
+            if (u * 64 + lane < MROWS * CH)
+                xs[wave][(u * 64 + lane) / CH * RS + x_chunk[u]] =
                     live ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
         }
     };
 
     // the producer's sums of squares (norm prologue) are requested ahead of everything
     // else, so that waiting for them below leaves the ring in flight
-    const int ssq_row = tid >> 5, ssq_p0 = tid & 31;
-    const bool ssq_mine = fuse.ssq_in != nullptr && ssq_row < M;
-    const float* ssq_pieces = fuse.ssq_in + (size_t)(ssq_mine ? ssq_row : 0) * fuse.ssq_tiles;
-    SsqLane ssq_part = {};
-    if (ssq_mine) ssq_part = ssq_lane_load(ssq_pieces, fuse.ssq_tiles, ssq_p0);
+    const int ssq_p0 = tid & 31;
+    int ssq_row[SSQ_ROWS];
+    bool ssq_mine[SSQ_ROWS];
+    const float* ssq_pieces[SSQ_ROWS];
+    SsqLane ssq_part[SSQ_ROWS] = {};
+#pragma unroll
+    for (int j = 0; j < SSQ_ROWS; ++j) {
+        ssq_row[j] = (tid >> 5) + j * (WAVES * 2);
+        ssq_mine[j] = fuse.ssq_in != nullptr && ssq_row[j] < M;
+        ssq_pieces[j] = fuse.ssq_in + (size_t)(ssq_mine[j] ? ssq_row[j] : 0) * fuse.ssq_tiles;
+        if (ssq_mine[j]) ssq_part[j] = ssq_lane_load(ssq_pieces[j], fuse.ssq_tiles, ssq_p0);
+    }
 
     // Operands of the epilogue that do not depend on the product are requested here as
     // well (the row's position now, what hangs on it after the ring): at the end of
@@ -190,7 +202,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     // requests in the order of use
 #pragma unroll
     for (int d = 0; d < R; ++d) {
-        if (d % kColsStage == 0) load_x(begin + d, d / kColsStage);
+        if (d % STAGE == 0) load_x(begin + d, d / STAGE);
         if (d % SPG == 0) load_c(begin + d, d / SPG);
         load_q(begin + d, qb[d]);
     }
@@ -211,26 +223,34 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     if (fuse.ssq_in != nullptr) {
         // 1 / rms of the rows from the producer's sums of squares (see SmallFuse): 32
         // lanes per row, folded by shuffles in a fixed order; read after the K loop
-        float ss = 0.f;
-        if (ssq_mine) ss = ssq_lane_sum(ssq_part, ssq_pieces, fuse.ssq_tiles, ssq_p0);
 #pragma unroll
-        for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
-        if (ssq_p0 == 0 && ssq_row < MROWS) inv_rms_s[ssq_row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+        for (int j = 0; j < SSQ_ROWS; ++j) {
+            float ss = 0.f;
+            if (ssq_mine[j]) ss = ssq_lane_sum(ssq_part[j], ssq_pieces[j], fuse.ssq_tiles, ssq_p0);
+#pragma unroll
+            for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
+            if (ssq_p0 == 0 && ssq_row[j] < MROWS) inv_rms_s[ssq_row[j]] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+        }
     }
 
     DequantRegs regs;
     regs.init(BITS);
-    float4_t acc[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+    float4_t acc[MT][2];
+    int a_row[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        acc[mt][0] = acc[mt][1] = float4_t{0.f, 0.f, 0.f, 0.f};
+        a_row[mt] = min(mt * 16 + nl, M - 1);
+    }
     ColumnConst cc[2];
-    const int a_row = min(nl, M - 1);
 
     for (int base = 0; base < steps_per_wave; base += R) {
 #pragma unroll
         for (int d = 0; d < R; ++d) {
             const int step = begin + base + d;
-            if (d % kColsStage == 0) {
-                store_x(step, d / kColsStage);
-                load_x(step + R, d / kColsStage);
+            if (d % STAGE == 0) {
+                store_x(step, d / STAGE);
+                load_x(step + R, d / STAGE);
             }
             if (d % SPG == 0) {
                 const uint32_t sw = cs_scale[d / SPG], zw = cs_zero[d / SPG];
@@ -252,18 +272,24 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
             }
             load_q(step + R, q);
             __builtin_amdgcn_sched_barrier(0);  // keeps the reload at this place of the body
-            const half8_t a = __builtin_bit_cast(half8_t, xs[wave][a_row * RS + (d % kColsStage) * 4 + kq]);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[t], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) {
+                const half8_t a = __builtin_bit_cast(half8_t, xs[wave][a_row[mt] * RS + (d % STAGE) * 4 + kq]);
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[mt][t], 0, 0, 0);
+            }
         }
     }
 
     // ---- the eight partial sums of a column meet in LDS, in wave order
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int m = kq * 4 + r;
-        if (m < M) *reinterpret_cast<float2*>(&red[wave][m][nl * 2]) = make_float2(acc[0][r], acc[1][r]);
-    }
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = mt * 16 + kq * 4 + r;
+            if (m < M) *reinterpret_cast<float2*>(&red[wave][m][nl * 2]) = make_float2(acc[mt][0][r], acc[mt][1][r]);
+        }
     __syncthreads();
     const bool worker = tid < M * (kColsTile / 2);  // one thread per (row, column pair)
     const int m = tid / (kColsTile / 2), c = tid % (kColsTile / 2) * 2;
@@ -351,24 +377,26 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
 bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_COLS");
     if (off && *off && atoi(off)) return false;
-    if ((bits != 4 && bits != 8) || M < 1 || M > 8) return false;
+    if ((bits != 4 && bits != 8) || M < 1 || M > 32) return false;
     if (group_size != 32 && group_size != 64 && group_size != 128 && group_size != 256) return false;
     if (N % kColsTile != 0 || K % (32 * kColsStage) != 0) return false;
     return epilogue == kEpilogueNone || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend;
 }
 
 // Tiles beyond one per CU are cut into kColsParts K ranges, which must not outnumber the CUs.
-static bool cols_cut_plan(int tiles, int K, int cus) {
+static int cols_waves(int M, bool cut) { return cut && M <= 8 ? kColsCutWaves : kColsWaves; }
+static bool cols_cut_plan(int M, int tiles, int K, int cus) {
     return tiles > cus && (tiles - cus) * kColsParts <= cus && tiles - cus < kMaxTileCounters &&
-           K % (32 * kColsStage * kColsCutWaves * kColsParts) == 0;
+           K % (32 * kColsStage * cols_waves(M, true) * kColsParts) == 0;
 }
-// The cut plan is taken at every row count of the kernel (8192x10240 against the small-M
-// kernel: 13.4 / 15.8 us at 3 rows, 14.5 / 16.7 at 8; with eight waves per workgroup it
-// had shown no gain at 8 rows).
+// The cut plan is taken up to eight rows (8192x10240 against the small-M kernel: 13.4 /
+// 15.8 us at 3 rows, 14.5 / 16.7 at 8; with eight waves per workgroup it had shown no
+// gain at 8 rows).
 static bool cols_use_cut(int M, int tiles, int K, int cus) {
     static const char* nocut = getenv("MH_GEMM_COLS_NO_CUT");
-    (void)M;
-    return cols_cut_plan(tiles, K, cus) && !(nocut && *nocut && atoi(nocut));
+    // above 8 rows (eight waves per workgroup) the small-M kernel is faster: 8192x10240 at
+    // 12 / 16 / 32 rows 21.0 / 21.7 / 28.8 us against 18.7 / 19.4 / 25.5
+    return M <= 8 && cols_cut_plan(M, tiles, K, cus) && !(nocut && *nocut && atoi(nocut));
 }
 
 // Where it measured faster than the small-M kernel: every CU gets at most one
@@ -390,7 +418,7 @@ bool gemm_cols_preferred(int M, int N, int K, int group_size, int bits, int epil
 
 // Bytes of workspace a launch of this kernel needs for the shape (0: none).
 size_t gemm_cols_workspace_bytes(int M, int N, int K) {
-    return cols_cut_plan(N / kColsTile, K, compute_units()) ? kTileCounterBytes + (size_t)kColsParts * M * N * sizeof(float)
+    return cols_cut_plan(M, N / kColsTile, K, compute_units()) ? kTileCounterBytes + (size_t)kColsParts * M * N * sizeof(float)
                                                             : 0;
 }
 
@@ -402,7 +430,7 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
     const int steps_total = K / 32;
     const int tiles = N / kColsTile, cus = compute_units();
     const bool cut = cols_use_cut(M, tiles, K, cus);
-    const int waves = cut ? kColsCutWaves : kColsWaves;
+    const int waves = cols_waves(M, cut);
     int spw = (steps_total + waves - 1) / waves;
     spw = (spw + kColsStage - 1) / kColsStage * kColsStage;  // whole stages, hence whole groups
     int full_tiles = tiles, parts = 1, part_spw = spw;
@@ -425,13 +453,17 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, \
                        (half_t*)out, partial, counters, M, N, K, steps_total, spw, full_tiles, parts, part_spw,    \
                        epilogue, fuse)
-// the cut plan runs with kColsCutWaves waves per workgroup
+// the cut plan runs with kColsCutWaves waves per workgroup up to eight rows (above, a
+// workgroup of eight waves is what gives every row and column pair its thread)
 #define MH_LAUNCH_COLS_B(BITS, SPG, MROWS)                               \
     do {                                                                 \
-        if (cut)                                                         \
-            MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsCutWaves);           \
-        else                                                             \
-            MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsWaves);              \
+        if constexpr (MROWS <= 8) {                                      \
+            if (cut) {                                                   \
+                MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsCutWaves);       \
+                break;                                                   \
+            }                                                            \
+        }                                                                \
+        MH_LAUNCH_COLS_W(BITS, SPG, MROWS, kColsWaves);                  \
     } while (0)
 #define MH_LAUNCH_COLS_S(BITS, MROWS)                        \
     switch (group_size / 32) {                               \
@@ -454,8 +486,12 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
         MH_LAUNCH_COLS(2);
     else if (M <= 4)
         MH_LAUNCH_COLS(4);
-    else
+    else if (M <= 8)
         MH_LAUNCH_COLS(8);
+    else if (M <= 16)
+        MH_LAUNCH_COLS(16);
+    else
+        MH_LAUNCH_COLS(32);
 #undef MH_LAUNCH_COLS_W
 #undef MH_LAUNCH_COLS_B
 #undef MH_LAUNCH_COLS_S

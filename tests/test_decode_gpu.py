@@ -137,10 +137,10 @@ def test_attention_split_kv_consistency(hip):
     assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
 
 
-@pytest.mark.parametrize("batch", [2, 4, 8])
+@pytest.mark.parametrize("batch", [2, 4, 8, 13, 32])
 def test_decode_wide_qkv_on_cut_tiles(hip, batch):
     """The 70B projection widths (q|k|v 8192 -> 10240: 320 column tiles of 32 on 256
-    CUs, up to eight rows): the fused q|k|v product then runs on the column-owner
+    CUs, up to 32 rows): the fused q|k|v product then runs on the column-owner
     kernel with the tiles beyond one per CU cut along K, its norm prologue and
     RoPE/cache-append epilogue, and o on the same kernel with the residual epilogue.
     Two layers, so that the second one consumes the first one's sums of squares."""
@@ -161,7 +161,7 @@ def test_decode_wide_qkv_on_cut_tiles(hip, batch):
     for c in k_cache + v_cache:
         c[:, :, :context] = rng.normal(0, 1, (batch, cfg["n_kv_heads"], context, 128))
     tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
-    positions = np.asarray([context, context - 3, context - 1, 0, 7, context, 2, 5][:batch], np.int32)
+    positions = np.asarray(([context, context - 3, context - 1, 0, 7, context, 2, 5] * 4)[:batch], np.int32)
     dec = LlamaDecoder(cfg, batch, max_seq)
     dec.load_host(model, k_cache, v_cache)
     _, got = dec.decode(tokens, positions, 1, want_logits=True)
