@@ -532,10 +532,15 @@ def main():
             t = time.perf_counter()
             cpu_out = [cport.matmul(hx[lin.k], *h, None, BITS, GROUP) for lin, h in zip(layers[0], host)]
             times.append(time.perf_counter() - t)
+        n_out = n_one_step = n_coarse = 0
         for g, c in zip(gpu_out, cpu_out):
             d = np.abs(g.astype(np.float64) - c.astype(np.float64))
-            tol = np.maximum(1e-2, np.spacing(np.abs(c)).astype(np.float64))
+            spacing = np.spacing(np.abs(c)).astype(np.float64)
+            tol = np.maximum(1e-2, spacing)
             worst = max(worst, float((d / tol).max()))
+            n_out += d.size
+            n_one_step += int((d > 1e-2).sum())      # outputs that needed the one-fp16-step allowance
+            n_coarse += int((spacing > 1e-2).sum())  # outputs large enough (|y| >= 16) to be granted it
         cpu_s = min(times)
         result["cpu_baseline"] = {
             "value": round(step_bytes / cpu_s / 1e9, 2),
@@ -545,6 +550,9 @@ def main():
             "sample": f"one layer (4 GEMVs, {step_bytes / 1e6:.0f} MB) x 2 runs, best of 2, "
                       f"{cpu_s:.2f} s per run, OpenMP over output columns",
             "gpu_vs_cpu_worst_err_over_tol": round(worst, 3),
+            "gpu_vs_cpu_outputs": n_out,
+            "gpu_vs_cpu_outputs_fp16_coarser_than_1e-2": n_coarse,
+            "gpu_vs_cpu_outputs_one_fp16_step_off": n_one_step,
         }
         log(f"cpu baseline: {cpu_s:.2f} s per layer on {threads} threads; "
             f"GPU vs CPU worst error / tolerance = {worst:.3f}")

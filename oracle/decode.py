@@ -11,6 +11,10 @@ single new token), softmax, P.V, output projection, residual adds in fp16,
 
 Grouped-query attention: query head j uses KV head ``j // (QH / KVH)``
 (the reference repeats each KV head, llama3_70b.py:85-93).
+
+Pinned by tests/test_oracle_decode.py: a known-answer step worked out scalar by
+scalar (tests/golden/decode_step.json) and models whose projections are exact
+zeros, identities or channel selections, for which the step has a closed form.
 """
 import numpy as np
 
@@ -49,8 +53,13 @@ def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, positions
     return out
 
 
-def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache: list, v_cache: list):
-    """Returns fp16 logits ``[B, vocab]``; caches ``[B, KVH, T, D]`` are updated in place."""
+def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache: list, v_cache: list,
+                linear=None):
+    """Returns fp16 logits ``[B, vocab]``; caches ``[B, KVH, T, D]`` are updated in place.
+
+    ``linear(x, (qweight, qzeros, scales, group_size), bits)`` replaces the numpy quantized
+    product (full-width layers use the C restatement, which is held bit-exact to it)."""
+    _linear = linear or globals()["_linear"]
     cfg = model["config"]
     qh, kvh, d = cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     rep = qh // kvh
@@ -85,13 +94,13 @@ def decode_step(model: dict, tokens: np.ndarray, positions: np.ndarray, k_cache:
     return gptq.dense_matmul(xn, model["lm_head"].T.astype(np.float16))
 
 
-def greedy(model, tokens, positions, k_cache, v_cache, n_steps):
+def greedy(model, tokens, positions, k_cache, v_cache, n_steps, linear=None):
     """Returns ``(out_tokens [n_steps, B], logits of every step)``."""
     tokens = np.array(tokens, np.int64)
     positions = np.array(positions, np.int64)
     out, all_logits = [], []
     for _ in range(n_steps):
-        logits = decode_step(model, tokens, positions, k_cache, v_cache)
+        logits = decode_step(model, tokens, positions, k_cache, v_cache, linear)
         tokens = logits.astype(np.float32).argmax(axis=-1)
         positions = positions + 1
         out.append(tokens.copy())

@@ -1,0 +1,106 @@
+"""GPU parity of the decode loop at the Llama-3-70B layer widths (config 4):
+hidden 8192, 64 query / 8 KV heads of 128, ffn 28672, context 2048, batch 1, 8
+and 32 -- the shapes the tokens-per-second figure is timed on, two layers deep so
+that the second layer consumes what the fused epilogues of the first one wrote
+(residual stream, sums of squares, cache rows).  At these widths the step runs
+the norm-prologue + SiLU-epilogue gate|up product at 8192 x 57344, the
+residual-epilogue down product at 28672 x 8192, the cut-tile q|k|v product with
+its RoPE / cache-append epilogue and, above 8 rows, the second-stage kernels.
+
+Checker: oracle.decode.decode_step (examples/llama3_70b.py:157-162,215-228 op by
+op) with the C restatement of the quantized product (bit-exact to the numpy one,
+tests/test_oracle_cport.py) so that it runs in seconds.  The vocabulary is small:
+the lm_head product at its real size is covered in test_gptq_gpu.py.
+"""
+import numpy as np
+import pytest
+
+from oracle import cport
+from oracle import decode as OD
+from oracle import special as OS
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(n_layers=2, hidden=8192, n_q_heads=64, n_kv_heads=8, head_dim=128, ffn=28672, vocab=256,
+           group_size=128, bits=4, rope_theta=5e5, rms_eps=1e-5)
+CONTEXT, MAX_SEQ = 2048, 2048 + 64
+
+
+def _c_linear(x, w, bits=4):
+    qweight, qzeros, scales, group_size = w
+    return cport.matmul(x, qweight, qzeros, scales, None, bits, group_size)
+
+
+@pytest.fixture(scope="module")
+def wide_model():
+    from minit_amd import synthetic
+    cport.lib()
+    rng = np.random.default_rng(70)
+    d = CFG["head_dim"]
+    shapes = {"qkv": (CFG["hidden"], (CFG["n_q_heads"] + 2 * CFG["n_kv_heads"]) * d),
+              "o": (CFG["n_q_heads"] * d, CFG["hidden"]),
+              "gate_up": (CFG["hidden"], 2 * CFG["ffn"]),
+              "down": (CFG["ffn"], CFG["hidden"])}
+    layers = []
+    for l in range(CFG["n_layers"]):
+        layer = {}
+        for name, (k, n) in shapes.items():
+            qw, qz, sc = synthetic.gptq_weights("wide70b", f"{l}.{name}", k, n, CFG["group_size"], 4)
+            # sums over 8192 / 28672 terms: keep the projections around unit size, or the reference's fp16
+            # attention scores (q . k before the 1/sqrt(d) scale) overflow
+            layer[name] = (qw, qz, (sc.astype(np.float32) / 16).astype(np.float16), CFG["group_size"])
+        layer["input_norm"] = rng.normal(1, 0.1, CFG["hidden"]).astype(np.float16)
+        layer["post_norm"] = rng.normal(1, 0.1, CFG["hidden"]).astype(np.float16)
+        layers.append(layer)
+    cos, sin = OS.rope_tables(d, MAX_SEQ, CFG["rope_theta"])
+    return {"config": CFG, "layers": layers,
+            "embed": rng.normal(0, 1.0, (CFG["vocab"], CFG["hidden"])).astype(np.float16),
+            "lm_head": rng.normal(0, 0.02, (CFG["vocab"], CFG["hidden"])).astype(np.float16),
+            "final_norm": rng.normal(1, 0.1, CFG["hidden"]).astype(np.float16), "cos": cos, "sin": sin}
+
+
+@pytest.mark.parametrize("batch", [1, 8, 32])
+def test_two_layers_at_70b_widths(hip, wide_model, batch):
+    from minit_amd.decode import LlamaDecoder
+    model = wide_model
+    rng = np.random.default_rng(700 + batch)
+    shape = (batch, CFG["n_kv_heads"], MAX_SEQ, CFG["head_dim"])
+    k_cache = [rng.standard_normal(shape, np.float32).astype(np.float16) for _ in range(CFG["n_layers"])]
+    v_cache = [rng.standard_normal(shape, np.float32).astype(np.float16) for _ in range(CFG["n_layers"])]
+    tokens = rng.integers(0, CFG["vocab"], batch).astype(np.int32)
+    # context 2048, a few rows a little shorter: every row reads its own number of entries
+    positions = (CONTEXT - (np.arange(batch) % 5) * 3).astype(np.int32)
+    print(f"[70B widths] batch {batch}, positions {positions.min()}..{positions.max()}", flush=True)
+
+    dec = LlamaDecoder(CFG, batch, MAX_SEQ)
+    dec.load_host(model, k_cache, v_cache)
+    got_tokens, got = dec.decode(tokens, positions, 1, want_logits=True)
+
+    ref_k, ref_v = [c.copy() for c in k_cache], [c.copy() for c in v_cache]
+    ref = OD.decode_step(model, tokens, positions, ref_k, ref_v, linear=_c_linear)
+    g, r = got.astype(np.float64), ref.astype(np.float64)
+    assert np.isfinite(g).all()
+    rel = np.linalg.norm(g - r) / np.linalg.norm(r)
+    worst = np.abs(g - r).max()
+    print(f"[70B widths] batch {batch}: logits rel L2 {rel:.3g}, worst |err| {worst:.3g} of {np.abs(r).max():.3g}", flush=True)
+    assert rel <= 1e-2, f"relative L2 error of the logits {rel:.3g}"
+    assert worst <= 2e-2 * max(1.0, np.abs(r).max())
+    ref_tok = ref.astype(np.float32).argmax(-1)
+    for b in range(batch):
+        if got_tokens[0, b] != ref_tok[b]:
+            row = np.sort(r[b])
+            assert row[-1] - row[-2] < 2e-2, f"row {b}: token differs with a clear margin"
+
+    # appended keys and values, each row at its own position: layer 0 sees only the q|k|v product and RoPE,
+    # layer 1 everything the first layer computed (attention, o + residual, gate|up + SiLU, down + residual, norm)
+    for layer in range(CFG["n_layers"]):
+        kc, vc = dec.k_cache[layer].numpy(), dec.v_cache[layer].numpy()      # V is kept [B, KVH, D, T]
+        tol = 2e-2 if layer == 0 else 6e-2
+        for b in range(batch):
+            p = int(positions[b])
+            ek = np.abs(kc[b, :, p].astype(np.float64) - ref_k[layer][b, :, p].astype(np.float64)).max()
+            ev = np.abs(vc[b, :, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max()
+            assert ek <= tol and ev <= tol, f"layer {layer} row {b}: appended k/v off by {ek:.3g} / {ev:.3g}"
+        # what was already in the cache stays (row 0, below its position)
+        p0 = int(positions[0])
+        assert np.array_equal(kc[0, :, :p0].view(np.uint16), k_cache[layer][0, :, :p0].view(np.uint16))
