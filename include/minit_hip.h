@@ -125,6 +125,25 @@ int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight,
                    void* out, int M, int N, int K, int group_size, int bits,
                    void* workspace, size_t workspace_bytes);
 
+/* mh_gptq_matmul for callers that cannot allocate device memory or pass a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference (its fused product
+ * accumulates with atomics into a zeroed output and needs no scratch,
+ * examples/qwen1_5_int8.py:198,263).  Same arguments and results as
+ * mh_gptq_matmul without the workspace pair: the split-K counters and partial
+ * sums live in a buffer of MH_GPTQ_STATIC_SCRATCH_BYTES that the library holds
+ * in device memory on every GPU it runs on until the process ends.  The call
+ * allocates and frees nothing.  A shape whose mh_gptq_workspace_bytes exceeds
+ * that size is rejected with MH_ERR_WORKSPACE.  Every call on a GPU uses that
+ * GPU's one buffer (of the device that is current at the call): calls that
+ * overlap on one GPU -- different streams, or threads -- race on it and give
+ * wrong sums; calls ordered on one stream are safe. */
+#define MH_GPTQ_STATIC_SCRATCH_BYTES (24u << 20)
+size_t mh_gptq_static_scratch_bytes(void);
+int mh_gptq_matmul_static(mh_stream_t stream, const void* x, const int32_t* qweight,
+                          const int32_t* qzeros, const void* scales, const int32_t* g_idx,
+                          void* out, int M, int N, int K, int group_size, int bits);
+
 /* The gate|up projection of a gated MLP with SiLU*up fused into the reduction of
  * the product (examples/llama3_70b.py:126-130 runs the product, sigmoid,
  * multiply, multiply as four launches).  The N = 2 * ffn columns are laid out

@@ -2,6 +2,8 @@
 // the choice between the VALU GEMV, the MFMA GEMM and the generic fallback.
 #include "gptq_common.h"
 
+#include <pthread.h>
+
 namespace mh {
 bool gemv_supported(int M, int N, int K, int group_size, int bits);
 size_t gemv_workspace_bytes(int M, int N, int K, int group_size, int bits);
@@ -54,9 +56,77 @@ int gptq_matmul_fused(hipStream_t stream, const void* x, const int32_t* qweight,
 }
 }  // namespace mh
 
+// ---- the product for callers that cannot allocate -----------------------------------------
+// mh_gptq_matmul_static keeps the split-K workspace (arrival counters + fp32 partial sums) in
+// device memory that belongs to the library: a file-scope array, one copy per GPU, held until
+// the process ends.  In host code the array's name is only a handle for the runtime; the
+// address kernels and fills may use comes from hipGetSymbolAddress, once per device.
+namespace mh {
+constexpr size_t kStaticScratchBytes = (size_t)MH_GPTQ_STATIC_SCRATCH_BYTES;
+constexpr int kStaticMaxDevices = 64;
+}  // namespace mh
+static __device__ __align__(256) unsigned char scratch[mh::kStaticScratchBytes];
+
+namespace mh {
+static void* g_static_scratch[kStaticMaxDevices];   // device address of `scratch` per GPU, 0 = not looked up yet
+static pthread_mutex_t g_static_lock = PTHREAD_MUTEX_INITIALIZER;
+
+__global__ void static_scratch_clear_kernel(uint4* p, int n16) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// The current device's copy of `scratch` (looked up on first use on that device).
+static int static_scratch_pointer(void** out) {
+    int dev = 0;
+    MH_CHECK_HIP(hipGetDevice(&dev));
+    MH_REQUIRE(dev >= 0 && dev < kStaticMaxDevices, "mh_gptq_matmul_static: device index %d out of range", dev);
+    pthread_mutex_lock(&g_static_lock);
+    void* ptr = g_static_scratch[dev];
+    hipError_t err = hipSuccess;
+    if (ptr == nullptr) {
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err == hipSuccess) g_static_scratch[dev] = ptr;
+    }
+    pthread_mutex_unlock(&g_static_lock);
+    if (err != hipSuccess || ptr == nullptr)
+        return fail(MH_ERR_HIP, "mh_gptq_matmul_static: hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
+    *out = ptr;
+    return MH_OK;
+}
+}  // namespace mh
+
 using namespace mh;
 
 extern "C" {
+
+size_t mh_gptq_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int mh_gptq_matmul_static(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                          const void* scales, const int32_t* g_idx, void* out, int M, int N, int K,
+                          int group_size, int bits) {
+    int rc = check_gptq_args("mh_gptq_matmul_static", x, qweight, qzeros, scales, out, M, N, K, group_size, bits);
+    if (rc) return rc;
+    if (M == 0) return MH_OK;
+    const size_t need = g_idx == nullptr ? mh_gptq_workspace_bytes(M, N, K, group_size, bits) : 0;
+    if (need > kStaticScratchBytes)
+        return fail(MH_ERR_WORKSPACE,
+                    "mh_gptq_matmul_static: M=%d N=%d K=%d needs %zu bytes of split-K scratch, the built-in buffer "
+                    "holds %zu; use mh_gptq_matmul with a caller-owned workspace",
+                    M, N, K, need, kStaticScratchBytes);
+    void* ws = nullptr;
+    if (need != 0) {
+        rc = static_scratch_pointer(&ws);
+        if (rc) return rc;
+        // the arrival counters must start at zero; the buffer keeps whatever the previous call (or a call
+        // that was interrupted) left, so clear them with a kernel (no memset node, safe under graph capture)
+        const int n16 = (int)(kTileCounterBytes / 16);
+        static_scratch_clear_kernel<<<(n16 + 255) / 256, 256, 0, as_stream(stream)>>>(static_cast<uint4*>(ws), n16);
+        MH_CHECK_LAUNCH();
+    }
+    return mh_gptq_matmul(stream, x, qweight, qzeros, scales, g_idx, out, M, N, K, group_size, bits, ws,
+                          ws ? kStaticScratchBytes : 0);
+}
 
 size_t mh_gptq_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     if (M <= 0 || N <= 0 || K <= 0 || group_size <= 0 || (bits != 4 && bits != 8)) return 0;
