@@ -306,6 +306,12 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
+    ap.add_argument("--calibrate-issue", action="store_true",
+                    help="run only the register-resident vector + MFMA instruction mix at 1, 2 and 4 waves per "
+                         "SIMD (do vector and matrix instructions of one SIMD's waves overlap?), then exit")
+    ap.add_argument("--issue-case", default="",
+                    help="with --calibrate-issue: run one case only, 'valu,mfma,dependent,waves_per_simd' "
+                         "(for a counter run under rocprofv3)")
     ap.add_argument("--int8-library", action="store_true",
                     help="time the vendor library's int8 GEMM (torch._int_mm) on the W8A8 shapes, then exit")
     ap.add_argument("--rowwise-only", action="store_true",
@@ -374,6 +380,35 @@ def main():
             res.append({"operands": label, "ms": round(ms, 2), "tops": round(tops, 1),
                         "frac_of_datasheet": round(tops / INT8_PEAK_TOPS, 4)})
         print(json.dumps({"kernel": "i8_mfma_probe_kernel", "waves_per_simd": 2, "results": res}))
+        return
+
+    if args.calibrate_issue:
+        cus = info["compute_units"]
+        iters = 20000
+        cases = [(52, 0, 0), (0, 4, 0), (52, 4, 0), (52, 4, 1), (26, 4, 1), (104, 4, 1), (0, 8, 0)]
+        waves = (1, 2, 4)
+        if args.issue_case:
+            nv, nm, dep, w = (int(v) for v in args.issue_case.split(","))
+            cases, waves = [(nv, nm, dep)], (w,)
+        rows = []
+        for wps in waves:
+            blocks = cus * wps                      # 256 threads = 4 waves = one per SIMD and block
+            sink = HIPTensor.allocate((blocks * 256,), "float32")
+            for nv, nm, dep in cases:
+                lib.call("mh_issue_probe", None, sink.data_ptr, blocks, 200, nv, nm, dep)
+                memory.synchronize()
+                e0, e1 = memory.Event(), memory.Event()
+                e0.record()
+                lib.call("mh_issue_probe", None, sink.data_ptr, blocks, iters, nv, nm, dep)
+                e1.record()
+                e1.synchronize()
+                ns = e0.elapsed_ms(e1) * 1e6 / iters           # per iteration of every wave of a SIMD
+                rows.append({"waves_per_simd": wps, "valu": nv, "mfma": nm, "dependent": bool(dep),
+                             "ns_per_iteration_per_simd": round(ns / wps, 1),
+                             "ns_per_iteration_per_wave": round(ns, 1)})
+                log(f"waves/SIMD {wps}: {nv:3d} vector + {nm} MFMA (dependent={dep}): "
+                    f"{ns / wps:7.1f} ns per iteration per SIMD")
+        print(json.dumps({"kernel": "issue_probe_kernel", "iterations": iters, "results": rows}))
         return
 
     if args.rowwise_only:

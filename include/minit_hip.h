@@ -186,6 +186,14 @@ int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w,
  * out receives blocks * 512 int32.  Used by bench.py --calibrate-mfma to find the
  * int8 rate the matrix pipes sustain on this box for given operand values. */
 int mh_i8_mfma_probe(mh_stream_t stream, const int8_t* operands, int32_t* out, int blocks, int iters);
+/* Calibration, no counterpart in the reference: blocks x 256 threads each run iters
+ * times n_valu packed-fp16 vector instructions and n_mfma v_mfma_f32_16x16x32_f16 from
+ * registers (dependent != 0: the MFMA operands come from the vector results of the same
+ * iteration).  Instances: (52,0,0) (0,4,0) (52,4,0) (52,4,1) (26,4,1) (104,4,1) (0,8,0).
+ * out receives blocks * 256 floats.  Used by bench.py --calibrate-issue to measure
+ * whether vector and matrix instructions of the waves of one SIMD overlap. */
+int mh_issue_probe(mh_stream_t stream, float* out, int blocks, int iters, int n_valu, int n_mfma,
+                   int dependent);
 /* out[n, k] = in[k, n]: one-time layout conversion for weights stored [K, N]. */
 int mh_i8_transpose(mh_stream_t stream, const int8_t* in, int8_t* out, int rows, int cols);
 

@@ -535,6 +535,11 @@ __global__ __launch_bounds__(256) void i8_transpose_kernel(const int8_t* __restr
     }
 }
 
+// i8_gemm_dma.hip: the same tiling with operand tiles loaded straight into LDS
+bool i8_gemm_dma_supported(int M, int N, int K);
+int i8_gemm_dma_launch(hipStream_t stream, const int8_t* a, const int8_t* w, const float* a_scale,
+                       const float* w_scale, void* out_f16, int32_t* acc_i32, int M, int N, int K);
+
 }  // namespace mh
 
 using namespace mh;
@@ -555,6 +560,8 @@ int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w, const float
     const int tiles = tiles_m * tiles_n;
     const int group_m = tiles_m < 8 ? tiles_m : 8;
     const int xcd_chunk = (tiles % 8 == 0) ? tiles / 8 : 0;
+    if (i8_gemm_dma_supported(M, N, K))
+        return i8_gemm_dma_launch(as_stream(stream), a, w, a_scale, w_scale, out_f16, acc_i32, M, N, K);
     static const char* no128 = getenv("MH_I8_NO_K128");
     // the 128-k kernel addresses its operands with 32-bit buffer offsets
     if (K % 128 == 0 && (size_t)M * K < ((size_t)1 << 31) && (size_t)N * K < ((size_t)1 << 31) &&

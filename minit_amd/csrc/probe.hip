@@ -1,0 +1,71 @@
+// Instruction-issue calibration for the GPTQ MFMA kernels (no counterpart in the
+// reference): a register-resident loop that issues, per iteration and wave, NV packed
+// fp16 vector instructions (the kind the in-register dequantisation is made of) and NM
+// v_mfma_f32_16x16x32_f16, with no memory traffic.  Timed with one, two and four waves
+// per SIMD it answers whether vector and matrix instructions of the waves of one SIMD
+// overlap or queue behind each other, which sets the issue-bound ceiling of a kernel
+// that needs 13 vector instructions per packed word next to one MFMA per 64 words.
+#include "common.h"
+
+namespace mh {
+
+// DEP: the MFMA's B operand is built from the vector results of the same iteration (as
+// in the real kernel, where the dequantised words feed the MFMA); otherwise constant.
+template <int NV, int NM, bool DEP>
+__global__ void __launch_bounds__(256) issue_probe_kernel(float* __restrict__ out, int iters, half2_t a) {
+    half2_t x[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) x[i] = half2_t{(half_t)(float)(threadIdx.x & 7), (half_t)(float)i};
+    float4_t acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    half8_t av;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) av[i] = (half_t)(0.01f * i);
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) x[i % 12] = x[i % 12] * a;     // v_pk_mul_f16 on 12 independent chains
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            half8_t b = av;
+            if (DEP) {
+                const half2_t p0 = x[(i * 3) % 12], p1 = x[(i * 3 + 1) % 12], p2 = x[(i * 3 + 2) % 12];
+                b = half8_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p0[0], p0[1]};
+            }
+            acc[i % 4] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, b, acc[i % 4], 0, 0, 0);
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 12; ++i) s += (float)x[i][0] + (float)x[i][1];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s += acc[i][0] + acc[i][3];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+}  // namespace mh
+
+using namespace mh;
+
+extern "C" int mh_issue_probe(mh_stream_t stream, float* out, int blocks, int iters, int n_valu, int n_mfma,
+                              int dependent) {
+    MH_REQUIRE(out != nullptr && blocks > 0 && iters > 0, "mh_issue_probe: bad argument");
+    const half2_t a = half2_t{(half_t)1.001f, (half_t)0.999f};
+    hipStream_t s = as_stream(stream);
+#define MH_PROBE(NV, NM, DEP)                                                         \
+    if (n_valu == NV && n_mfma == NM && (dependent != 0) == DEP) {                     \
+        issue_probe_kernel<NV, NM, DEP><<<blocks, 256, 0, s>>>(out, iters, a);         \
+        MH_CHECK_LAUNCH();                                                             \
+        return MH_OK;                                                                  \
+    }
+    MH_PROBE(52, 0, false)
+    MH_PROBE(0, 4, false)
+    MH_PROBE(52, 4, false)
+    MH_PROBE(52, 4, true)
+    MH_PROBE(26, 4, true)
+    MH_PROBE(104, 4, true)
+    MH_PROBE(0, 8, false)
+#undef MH_PROBE
+    return fail(MH_ERR_INVALID, "mh_issue_probe: no instance for %d vector + %d matrix instructions (dependent=%d)",
+                n_valu, n_mfma, dependent);
+}
