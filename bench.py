@@ -30,14 +30,29 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# HBM bytes per launch (mean over the four launches of a step, which run the
-# library's two MFMA GPTQ kernels) on this workload, measured with two
+# HBM bytes per launch of the dominant kernel (the gate|up product) come from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, in KiB per
 # dispatch, scaled by what the same counters read for the 1 GiB copy kernel of
-# --calibrate-copy: x2.000 and x1.000); the summary with the commands is kept
-# under profiles/.  A counter cannot be read from inside this process, so the
-# figure is carried here and is only reported for the entry point it was taken on.
-MEASURED_TRAFFIC = {"mh_gptq_matmul": 116_336_217}
+# --calibrate-copy).  A process cannot read those counters itself, so the figure is
+# read from the committed summary of those runs, which carries a line
+#   bench-traffic: entry=<entry point> kernel=<name> bytes_per_launch=<n> commit=<hash>
+# and is reported with the commit it was measured at (null if the line is missing).
+TRAFFIC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                               "gptq_decode_gemvs_llama70b_m1.md")
+
+
+def measured_traffic(entry):
+    import re
+    try:
+        text = open(TRAFFIC_SUMMARY).read()
+    except OSError:
+        return None, None
+    for m in re.finditer(r"bench-traffic:\s*entry=(\S+)\s+kernel=(\S+)\s+bytes_per_launch=(\d+)\s+commit=(\S+)", text):
+        if m.group(1) == entry:
+            return int(m.group(3)), m.group(4)
+    return None, None
+
+
 HBM_PEAK_GBPS = 8000.0
 INT8_PEAK_TOPS = 5000.0
 
@@ -460,6 +475,25 @@ def main():
     log(f"{args.steps} steps: {dev_ms:.2f} ms on device ({wall * 1e3:.2f} ms wall), "
         f"{ms_per_step * 1e3:.1f} us/step, {gbps:.0f} GB/s")
 
+    # ---- the dominant kernel (gate|up: 55 % of the step's bytes), timed launch by launch with an
+    # event pair around it inside a second pass over the same steps, same launch sequence
+    dom = max(range(len(LINEARS)), key=lambda j: linear_bytes(1, LINEARS[j][1], LINEARS[j][2]))
+    dom_name, dom_k, dom_n = LINEARS[dom]
+    pairs = [(memory.Event(), memory.Event()) for _ in range(args.steps)]
+    for i in range(args.steps):
+        for j, lin in enumerate(layers[i % args.layers]):
+            if j == dom:
+                pairs[i][0].record()
+            run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
+            if j == dom:
+                pairs[i][1].record()
+    memory.synchronize()
+    dom_us = float(np.mean([a.elapsed_ms(b) for a, b in pairs])) * 1e3
+    dom_bytes = linear_bytes(1, dom_k, dom_n)
+    dom_gbps = dom_bytes / dom_us / 1e3
+    traffic, traffic_commit = measured_traffic(ENTRY)
+    log(f"dominant kernel ({dom_name} {dom_k}x{dom_n}): {dom_us:.2f} us per launch in the layer sequence, {dom_gbps:.0f} GB/s")
+
     result = {
         "metric": "w4a16_gemv_hbm_gbps",
         "value": round(gbps, 1),
@@ -482,15 +516,20 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gptq_gemv_kernel<4,1,8>" if ENTRY == "mh_gptq_gemv" else "gptq_gemm_cols_kernel<4,4,1,{4,8}> (qkv, o, down) + gptq_gemm_small_kernel<4,1,4> (gate_up)",
+            "kernel": ("gptq_gemv_kernel<4,1,8>" if ENTRY == "mh_gptq_gemv" else "gptq_gemm_small_kernel<4,1,4,false,true>")
+                      + f" ({dom_name} {dom_k}x{dom_n}, M=1)",
             "entry": ENTRY,
-            "achieved": round(gbps, 1),
+            "achieved": round(dom_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBPS, 4),
-            "avg_launch_us": round(dev_ms * 1e3 / launches, 3),
-            "bytes_per_launch": step_bytes // len(LINEARS),
-            "traffic": MEASURED_TRAFFIC.get(ENTRY),
+            "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
+            "avg_launch_us": round(dom_us, 3),
+            "bytes_per_launch": dom_bytes,
+            "traffic": traffic,
+            "traffic_measured_at_commit": traffic_commit,
+            # the whole step (four launches, two kernels, launch gaps included) on the same scale
+            "step": {"achieved": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "avg_launch_us": round(dev_ms * 1e3 / launches, 3), "bytes_per_launch": step_bytes // len(LINEARS)},
         },
     }
 
@@ -563,10 +602,21 @@ def main():
             run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
             gpu_out.append(outs[lin.n].numpy().copy())
         times, worst = [], 0.0
-        for rep in range(2):
+        reps = 5
+        for rep in range(reps):
             t = time.perf_counter()
             cpu_out = [cport.matmul(hx[lin.k], *h, None, BITS, GROUP) for lin, h in zip(layers[0], host)]
             times.append(time.perf_counter() - t)
+        # one thread: the smallest linear of the layer (o_proj), scaled by its own bytes
+        small = min(range(len(LINEARS)), key=lambda j: linear_bytes(1, LINEARS[j][1], LINEARS[j][2]))
+        cport.set_threads(1)
+        times1 = []
+        for rep in range(reps):
+            t = time.perf_counter()
+            cport.matmul(hx[layers[0][small].k], *host[small], None, BITS, GROUP)
+            times1.append(time.perf_counter() - t)
+        cport.set_threads(threads)
+        small_bytes = linear_bytes(1, LINEARS[small][1], LINEARS[small][2])
         n_out = n_one_step = n_coarse = 0
         for g, c in zip(gpu_out, cpu_out):
             d = np.abs(g.astype(np.float64) - c.astype(np.float64))
@@ -576,20 +626,34 @@ def main():
             n_out += d.size
             n_one_step += int((d > 1e-2).sum())      # outputs that needed the one-fp16-step allowance
             n_coarse += int((spacing > 1e-2).sum())  # outputs large enough (|y| >= 16) to be granted it
-        cpu_s = min(times)
+        cpu_s = float(np.median(times))
+        cpu1_s = float(np.median(times1))
+        cpu_model = "unknown"
+        try:
+            for line in open("/proc/cpuinfo"):
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+        except OSError:
+            pass
         result["cpu_baseline"] = {
             "value": round(step_bytes / cpu_s / 1e9, 2),
             "unit": "GB/s",
             "cores": threads,
             "kind": "port",
-            "sample": f"one layer (4 GEMVs, {step_bytes / 1e6:.0f} MB) x 2 runs, best of 2, "
+            "sample": f"one layer (4 GEMVs, {step_bytes / 1e6:.0f} MB), median of {reps} runs, "
                       f"{cpu_s:.2f} s per run, OpenMP over output columns",
+            "cpu_model": cpu_model,
+            "one_thread": {"value": round(small_bytes / cpu1_s / 1e9, 3), "unit": "GB/s", "cores": 1,
+                           "sample": f"{LINEARS[small][0]} alone ({small_bytes / 1e6:.0f} MB), median of {reps} runs, "
+                                     f"{cpu1_s:.2f} s per run"},
             "gpu_vs_cpu_worst_err_over_tol": round(worst, 3),
             "gpu_vs_cpu_outputs": n_out,
             "gpu_vs_cpu_outputs_fp16_coarser_than_1e-2": n_coarse,
             "gpu_vs_cpu_outputs_one_fp16_step_off": n_one_step,
         }
-        log(f"cpu baseline: {cpu_s:.2f} s per layer on {threads} threads; "
+        log(f"cpu baseline ({cpu_model}): {cpu_s:.2f} s per layer on {threads} threads, {cpu1_s:.2f} s for "
+            f"{LINEARS[small][0]} on one; "
             f"GPU vs CPU worst error / tolerance = {worst:.3f}")
 
     print(json.dumps(result), flush=True)

@@ -159,7 +159,8 @@ int mh_gptq_gemm(mh_stream_t stream, const void* x, const int32_t* qweight, cons
     if (M == 0) return MH_OK;
     MH_REQUIRE(g_idx == nullptr, "mh_gptq_gemm: act-order g_idx is served by mh_gptq_matmul");
     MH_REQUIRE(gemm_supported(M, N, K, group_size, bits),
-               "mh_gptq_gemm: needs N %% 8 == 0, K %% 32 == 0, group_size %% 32 == 0 (M=%d N=%d K=%d g=%d)",
+               "mh_gptq_gemm: needs N %% 8 == 0, K %% 32 == 0, group_size %% 32 == 0 and packed weights below 2 GiB "
+               "(M=%d N=%d K=%d g=%d)",
                M, N, K, group_size);
     return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
                             workspace, workspace_bytes, kEpilogueNone, SmallFuse{});

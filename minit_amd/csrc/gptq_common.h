@@ -164,6 +164,16 @@ struct SmallFuse {
     int q_heads = 0, kv_heads = 0, max_seq = 0;
 };
 
+// xw = fp16(h * w) of the split norm, kept finite: where the reference's x / rms * w is of
+// order w, h * w can leave the fp16 range for a very large residual channel (|h| above
+// 65504 / w); the product then saturates at the largest finite value instead of becoming
+// an infinity that would turn the whole row of the next product into NaN.
+template <typename V>
+__device__ __forceinline__ V norm_weighted(V h, V w) {
+    const V hi = (half_t)65504.f - V{}, lo = -hi;
+    return __builtin_elementwise_max(__builtin_elementwise_min(h * w, hi), lo);
+}
+
 __device__ __forceinline__ half_t silu_pair(half_t gate, half_t up) {
     const float g = (float)gate;
     return (half_t)(g / (1.f + expf(-g)) * (float)up);

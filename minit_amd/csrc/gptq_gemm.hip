@@ -704,7 +704,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                     const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
                     const half4_t h = h_old + y;  // fp16 add, one rounding
                     *reinterpret_cast<half4_t*>(hp) = h;
-                    if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) = h * nw;
+                    if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) = norm_weighted(h, nw);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
                 }
@@ -839,9 +839,12 @@ GemmPlan plan_gemm(int M, int N, int K, int group_size, bool allow_balanced) {
     return p;
 }
 
+// The MFMA kernels address the packed weights of a matrix with 32-bit buffer offsets.
+static bool packed_weights_addressable(int N, int K, int bits) { return (size_t)K * N * bits / 8 < ((size_t)1 << 31); }
+
 bool gemm_supported(int M, int N, int K, int group_size, int bits) {
     return M >= 1 && (bits == 4 || bits == 8) && N % 8 == 0 && K % 32 == 0 && group_size % 32 == 0 &&
-           K % group_size == 0;
+           K % group_size == 0 && packed_weights_addressable(N, K, bits);
 }
 
 // The epilogue out[m, j] = silu(y[m, gate(j)]) * y[m, up(j)] on column tiles laid out as
@@ -876,7 +879,8 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     if (row_blocked(M, group_size)) {
         // blocks of kSmallBlockM rows in one launch; partial sums [split][M][N]
         const GemmPlan p = plan_gemm_small(kSmallBlockM, N, K, false, (M + kSmallBlockM - 1) / kSmallBlockM);
-        return kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float);
+        // unsplit, the kernel stores its results directly and touches neither counters nor partials
+        return p.split_k > 1 ? kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float) : 0;
     }
     // either plan of the small-M kernel may be the one a launch takes
     const GemmPlan p = plan_gemm(M, N, K, group_size, false), pb = plan_gemm(M, N, K, group_size, true);
@@ -968,8 +972,9 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse) {
     // the MFMA kernels address the packed weights with 32-bit buffer offsets
-    if ((size_t)K * N * bits / 8 >= ((size_t)1 << 31))
-        return fail(MH_ERR_INVALID, "gptq gemm: packed weights of 2 GiB or more are not supported");
+    if (!packed_weights_addressable(N, K, bits))
+        return fail(MH_ERR_INVALID, "gptq gemm: packed weights of 2 GiB or more are not supported by the MFMA kernels "
+                    "(mh_gptq_matmul serves them with the per-element kernel)");
     // a narrow output goes to the kernel whose workgroups own their columns over all of K
     if (gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse,
@@ -983,10 +988,10 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
         if (epilogue != kEpilogueNone || fuse.ssq_in != nullptr)
             return fail(MH_ERR_INVALID, "gptq gemm: epilogues and norm fusion need M <= %d", kSmallMaxM);
         const size_t need = gemm_workspace_bytes(M, N, K, group_size, bits);
-        if (workspace == nullptr || workspace_bytes < need)
+        if (need != 0 && (workspace == nullptr || workspace_bytes < need))
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
                         workspace ? workspace_bytes : (size_t)0);
-        if ((uintptr_t)workspace % 256 != 0)
+        if (need != 0 && (uintptr_t)workspace % 256 != 0)
             return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace must be 256-byte aligned");
         // one launch: blockIdx.z walks the blocks of kSmallBlockM rows
         const GemmPlan p = plan_gemm_small(kSmallBlockM, N, K, false, (M + kSmallBlockM - 1) / kSmallBlockM);

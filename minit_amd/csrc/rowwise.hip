@@ -32,6 +32,16 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
     return raw;
 }
 
+// 16-byte accesses to data that is touched once: keep them from displacing what other
+// workgroups reuse.
+__device__ __forceinline__ uint4 stream_load(const uint4* p) {
+    const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void stream_store(uint4* p, const uint4& v) {
+    __builtin_nontemporal_store(uint4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<uint4_t*>(p));
+}
+
 // ---- RMSNorm ------------------------------------------------------------------------------
 // out = T( x / sqrt(sum(x^2)/b + eps) * w ), fp32 inside
 // (minit/cuda/kernel/cuda/rms_norm.py:69-89).
@@ -45,13 +55,22 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
     const uint4* wsrc = reinterpret_cast<const uint4*>(weight);
     uint4* dst = reinterpret_cast<uint4*>(out + row * b);
     const int nvec = (int)(b / kRowVec);
-    uint4 regs[kRowMaxChunks];
+    uint4 regs[kRowMaxChunks], wregs[kRowMaxChunks];
     float ss = 0.f;
+    // every load of the row and of the weight is requested before the first use; the row is read
+    // once (streaming hint), the weight by every row (it stays cached)
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
         const int v = c * kRowThreads + threadIdx.x;
         if (v < nvec) {
-            regs[c] = src[v];
+            regs[c] = stream_load(src + v);
+            wregs[c] = wsrc[v];
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < kRowMaxChunks; ++c) {
+        const int v = c * kRowThreads + threadIdx.x;
+        if (v < nvec) {
             float f[8];
             unpack8<T>(regs[c], f);
 #pragma unroll
@@ -60,17 +79,19 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
     }
     ss = block_sum(ss, smem);
     const float rms = sqrtf(ss / (float)b + eps);
+    // 16-bit storage: one division per row; x * (1 / rms) differs from x / rms by an fp32 ulp at most,
+    // far below the storage type's step.  fp32 storage keeps the reference's x / rms * w.
+    const float inv = 1.0f / rms;
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
         const int v = c * kRowThreads + threadIdx.x;
         if (v < nvec) {
             float f[8], w[8];
             unpack8<T>(regs[c], f);
-            const uint4 wr = wsrc[v];
-            unpack8<T>(wr, w);
+            unpack8<T>(wregs[c], w);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) f[i] = f[i] / rms * w[i];
-            dst[v] = pack8<T>(f);
+            for (int i = 0; i < 8; ++i) f[i] = sizeof(T) == 2 ? f[i] * inv * w[i] : f[i] / rms * w[i];
+            stream_store(dst + v, pack8<T>(f));
         }
     }
 }
@@ -119,7 +140,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
     for (int c = 0; c < kRowMaxChunks; ++c) {
         const int v = c * kRowThreads + threadIdx.x;
         if (v < nvec) {
-            const uint4 raw = src[v];
+            const uint4 raw = stream_load(src + v);
             unpack8<T>(raw, vals[c]);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -141,19 +162,23 @@ __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
         if (v < nvec) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                vals[c][i] = expf(vals[c][i] - mx);
+                // 16-bit storage: exp(d) as 2^(d * log2 e) on the hardware's base-2 exponential (about an
+                // fp32 ulp from expf, three orders below the storage step); fp32 storage keeps expf
+                vals[c][i] = sizeof(T) == 2 ? __builtin_amdgcn_exp2f((vals[c][i] - mx) * 1.44269504088896340736f)
+                                            : expf(vals[c][i] - mx);
                 sum += vals[c][i];
             }
         }
     }
     sum = block_sum(sum, smem);
+    const float inv = 1.0f / sum;  // one division per row for 16-bit storage
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
         const int v = c * kRowThreads + threadIdx.x;
         if (v < nvec) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vals[c][i] = vals[c][i] / sum;
-            dst[v] = pack8<T>(vals[c]);
+            for (int i = 0; i < 8; ++i) vals[c][i] = sizeof(T) == 2 ? vals[c][i] * inv : vals[c][i] / sum;
+            stream_store(dst + v, pack8<T>(vals[c]));
         }
     }
 }
@@ -275,7 +300,7 @@ __global__ void rope_vec_kernel(const T* __restrict__ in, const float* __restric
         const size_t pos = positions ? (size_t)positions[bsq] : bsq % seq;
         const float4 c = *reinterpret_cast<const float4*>(freqs_cos + pos * half + qd * 4);
         const float4 s = *reinterpret_cast<const float4*>(freqs_sin + pos * half + qd * 4);
-        const uint4 raw = reinterpret_cast<const uint4*>(in)[idx];
+        const uint4 raw = stream_load(reinterpret_cast<const uint4*>(in) + idx);  // x is touched once, the tables by every head
         float f[8], o[8];
         unpack8<T>(raw, f);
         const float cs[4] = {c.x, c.y, c.z, c.w}, sn[4] = {s.x, s.y, s.z, s.w};
@@ -284,7 +309,7 @@ __global__ void rope_vec_kernel(const T* __restrict__ in, const float* __restric
             o[2 * p] = f[2 * p] * cs[p] - f[2 * p + 1] * sn[p];
             o[2 * p + 1] = f[2 * p + 1] * cs[p] + f[2 * p] * sn[p];
         }
-        reinterpret_cast<uint4*>(out)[idx] = pack8<T>(o);
+        stream_store(reinterpret_cast<uint4*>(out) + idx, pack8<T>(o));
     }
 }
 

@@ -79,6 +79,15 @@ int oracle_threads(void) {
 #endif
 }
 
+/* number of OpenMP threads of the following calls (the timed CPU baseline runs with all threads and with one) */
+void oracle_set_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
 uint16_t oracle_double_to_half(double v) { return double_to_half(v); }
 float oracle_half_to_float(uint16_t h) { return half_to_float(h); }
 

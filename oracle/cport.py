@@ -40,6 +40,10 @@ def threads() -> int:
     return lib().oracle_threads()
 
 
+def set_threads(n: int) -> None:
+    lib().oracle_set_threads(ctypes.c_int(n))
+
+
 def dequant(qweight, qzeros, scales, g_idx=None, bits=4, group_size=128):
     per = 32 // bits
     k, n = qweight.shape[0] * per, qweight.shape[1]

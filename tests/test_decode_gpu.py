@@ -306,3 +306,46 @@ def test_greedy_decode_eight_bit_weights(hip, batch):
     ref_tokens, ref_logits = OD.greedy(model, tokens, positions, [c.copy() for c in k_cache],
                                        [c.copy() for c in v_cache], n_steps)
     _check_greedy(dec, tokens, positions, got_tokens, got_logits, ref_tokens, ref_logits)
+
+
+@pytest.mark.parametrize("batch", [2, 9])
+def test_large_residual_channels(hip, batch):
+    """Residual channels of magnitude 2e4 under norm weights up to 3: the fused residual + norm
+    path rounds h * w (up to 6e4, still inside fp16) before the row factor where the reference
+    rounds x / rms * w; the step must match the oracle all the same.  With h * w beyond 65504 the
+    product saturates instead of becoming infinite: the logits stay finite."""
+    from minit_amd.decode import LlamaDecoder
+    cfg = dict(CFG, hidden=1024, ffn=256)          # 1024: the fused norm also rides on the second stage (9 rows)
+    model = _host_model(cfg, seed=90 + batch)
+    rng = np.random.default_rng(900 + batch)
+    big = rng.choice(cfg["hidden"], 6, replace=False)
+    model["embed"] = model["embed"].copy()
+    model["embed"][:, big] = (2e4 * rng.choice([-1.0, 1.0], (cfg["vocab"], 6))).astype(np.float16)
+    for layer in model["layers"]:
+        for name in ("input_norm", "post_norm"):
+            w = layer[name].copy()
+            w[big] = rng.uniform(2.0, 3.0, 6).astype(np.float16)
+            layer[name] = w
+    context, max_seq = 9, 64
+    shape = (batch, cfg["n_kv_heads"], max_seq, 128)
+    k_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    v_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    for c in k_cache + v_cache:
+        c[:, :, :context] = rng.normal(0, 1, (batch, cfg["n_kv_heads"], context, 128))
+    tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
+    positions = np.full(batch, context, np.int32)
+    dec = LlamaDecoder(cfg, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+    _, got = dec.decode(tokens, positions, 1, want_logits=True)
+    ref = OD.decode_step(model, tokens, positions, [c.copy() for c in k_cache], [c.copy() for c in v_cache])
+    g, r = got.astype(np.float64), ref.astype(np.float64)
+    assert np.isfinite(g).all()
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+    assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
+
+    # beyond the fp16 range: 3e4 * 3 = 9e4
+    model["embed"][:, big] = (3e4 * np.sign(model["embed"][:, big].astype(np.float32))).astype(np.float16)
+    dec2 = LlamaDecoder(cfg, batch, max_seq)
+    dec2.load_host(model, k_cache, v_cache)
+    _, got2 = dec2.decode(tokens, positions, 1, want_logits=True)
+    assert np.isfinite(got2.astype(np.float64)).all(), "a saturated h * w must not turn the step into NaN"

@@ -42,6 +42,23 @@ def test_status_codes_raise_with_message():
     assert lib.call("mh_gptq_workspace_bytes", 1, 4096, 4100, 128, 4) == 0   # contract violated
 
 
+def test_oversized_matrices_are_kept_off_the_mfma_kernels():
+    """The MFMA kernels address a matrix's packed weights with 32-bit offsets: 2 GiB and more go to
+    the per-element kernel through mh_gptq_matmul, and mh_gptq_gemm says so instead of launching
+    (argument checks only: nothing is dereferenced or launched here)."""
+    from minit_amd import lib
+    k = n = 65536                          # 4-bit: k * n / 2 = 2 GiB exactly
+    fake = 4096                            # a non-null pointer value; the size check comes before any use
+    with pytest.raises(lib.HipError, match="2 GiB"):
+        lib.call("mh_gptq_gemm", None, fake, fake, fake, fake, None, fake, 16, n, k, 128, 4, None, 0)
+    # the same matrix just below the limit is accepted by the planner
+    assert lib.call("mh_gptq_workspace_bytes", 16, n - 8, k, 128, 4) > 0
+    # a plain product of more than 32 rows that is not split along K needs no workspace
+    assert lib.call("mh_gptq_workspace_bytes", 2048, 57344, 8192, 128, 4) == 0
+    # ... and the split one still does
+    assert lib.call("mh_gptq_workspace_bytes", 64, 4096, 14336, 128, 4) > 0
+
+
 def test_dispatch_rules():
     from minit_amd.core.dispatch import DISPATCH_CACHE, DISPATCH_TABLE, dispatch, register_dispatch
     from minit_amd.core.operator import Operator
