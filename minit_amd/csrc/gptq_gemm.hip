@@ -732,6 +732,13 @@ int gptq_gemm_cols_launch(hipStream_t stream, const void* x, const int32_t* qwei
                           const void* scales, void* out, int M, int N, int K, int group_size, int bits, int epilogue,
                           const SmallFuse& fuse, void* workspace, size_t workspace_bytes);
 
+// gptq_gemm_wide.hip: more than 64 rows, dequantised weight tiles staged in LDS
+bool gemm_wide_preferred(int M, int N, int K, int group_size, int bits, int epilogue);
+size_t gemm_wide_workspace_bytes(int M, int N, int K);
+int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                          const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
+                          size_t workspace_bytes);
+
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
     int col_tiles;
@@ -875,7 +882,7 @@ int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
 static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_small(kSmallMaxM, group_size); }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
-    (void)bits;
+    if (gemm_wide_preferred(M, N, K, group_size, bits, kEpilogueNone)) return gemm_wide_workspace_bytes(M, N, K);
     if (row_blocked(M, group_size)) {
         // blocks of kSmallBlockM rows in one launch; partial sums [split][M][N]
         const GemmPlan p = plan_gemm_small(kSmallBlockM, N, K, false, (M + kSmallBlockM - 1) / kSmallBlockM);
@@ -975,6 +982,10 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     if (!packed_weights_addressable(N, K, bits))
         return fail(MH_ERR_INVALID, "gptq gemm: packed weights of 2 GiB or more are not supported by the MFMA kernels "
                     "(mh_gptq_matmul serves them with the per-element kernel)");
+    // many rows: the kernel that dequantises a weight tile once for 128 rows
+    if (fuse.ssq_in == nullptr && gemm_wide_preferred(M, N, K, group_size, bits, epilogue))
+        return gptq_gemm_wide_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,
+                                     workspace_bytes);
     // a narrow output goes to the kernel whose workgroups own their columns over all of K
     if (gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse,

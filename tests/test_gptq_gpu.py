@@ -172,6 +172,30 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     assert_fp16_close(got, ref, what=f"gemm {m}x{k}x{n} b{bits}")
 
 
+@pytest.mark.parametrize("m,k,n,group_size", [
+    (384, 1024, 776, 128),     # ragged last column tile, unsplit
+    (500, 2048, 256, 64),      # ragged last row tile, two groups per 128 k
+    (512, 8192, 128, 128),     # one column tile, K split over workgroups (partial sums + second stage)
+    (1000, 1024, 1032, 256),   # groups longer than a stage
+])
+def test_gemm_many_rows(hip, m, k, n, group_size):
+    """Several hundred rows: the kernel that stages dequantised fp16 weight tiles in LDS."""
+    from minit_amd import synthetic
+    qweight, qzeros, scales = _weights(k, n, group_size, 4, seed=9)
+    x = synthetic.activations("test9", f"x{m}", (m, k))
+    got = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, group_size, 4)
+    ref = O.matmul_f64(x, qweight, qzeros, scales, None, 4, group_size)
+    assert_fp16_close(got, ref, what=f"many rows {m}x{k}x{n} g{group_size}")
+    # one-hot rows pick rows of the dequantized matrix bit for bit (k order inside the LDS tiles)
+    rows = np.random.default_rng(m).integers(0, k, m)
+    rows[:4] = [0, 63, 64, k - 1]
+    onehot = np.zeros((m, k), dtype=np.float16)
+    onehot[np.arange(m), rows] = 1.0
+    got = _run_linear(hip, "mh_gptq_matmul", onehot, qweight, qzeros, scales, group_size, 4)
+    w = O.dequantize_packed(qweight, qzeros, scales, None, 4, group_size)
+    np.testing.assert_array_equal(got.view(np.uint16), w[rows].view(np.uint16))
+
+
 def test_repeated_calls_are_deterministic(hip):
     """Split-K partials are summed in a fixed order: bitwise repeatable, and the
     arrival counters are left zeroed for the next call."""
