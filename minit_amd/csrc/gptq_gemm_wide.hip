@@ -28,7 +28,7 @@
 
 namespace mh {
 
-constexpr int kWideBM = 128, kWideBN = 128, kWideBK = 64, kWideThreads = 256;
+constexpr int kWideBM = 128, kWideBN = 128, kWideBK = 64;
 constexpr int kWideTileBytes = kWideBM * kWideBK * 2;  // 16 KiB: one operand tile of a stage
 
 void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
@@ -58,29 +58,46 @@ __device__ __forceinline__ void wide_load_b32_stream(uint32_t& dst, int voffset,
 __device__ __forceinline__ void wide_load_b32(uint32_t& dst, int voffset, const int4_t& rsrc, int soffset) {
     asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
 }
-template <int NEWEST>
-__device__ __forceinline__ void wide_wait(uint4_t& a0, uint4_t& a1, uint4_t& a2, uint4_t& a3, uint32_t& q0, uint32_t& q1,
-                                          uint32_t& q2, uint32_t& q3, uint32_t& c0, uint32_t& c1) {
-    asm volatile("s_waitcnt vmcnt(%10)"
-                 : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(q0), "+v"(q1), "+v"(q2), "+v"(q3), "+v"(c0), "+v"(c1)
-                 : "n"(NEWEST)
-                 : "memory");
+// Everything but the newest NEWEST loads has arrived; the registers that the next uses read pass
+// through the wait, so that no use can be scheduled above it.
+template <int NEWEST, int PT>
+__device__ __forceinline__ void wide_wait(uint4_t (&a)[PT], uint32_t (&q)[PT], uint32_t& c0, uint32_t& c1) {
+    if constexpr (PT == 4) {
+        asm volatile("s_waitcnt vmcnt(%10)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]),
+                       "+v"(c0), "+v"(c1)
+                     : "n"(NEWEST)
+                     : "memory");
+    } else {
+        static_assert(PT == 2, "four or two pieces per thread");
+        asm volatile("s_waitcnt vmcnt(%6)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(q[0]), "+v"(q[1]), "+v"(c0), "+v"(c1)
+                     : "n"(NEWEST)
+                     : "memory");
+    }
 }
 __device__ __forceinline__ void wide_load_u16(uint32_t& dst, int voffset, const int4_t& rsrc, int soffset) {
     asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
 }
 
-__global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
+// WN: waves along the columns of the tile.  WN = 2: four waves 2 x 2, 64 x 64 each (fewest fragment
+// reads per MFMA; two workgroups per CU); WN = 4: eight waves 2 x 4, 64 x 32 each, for products of
+// one or two row tiles, where the tiles are too few to give every SIMD two waves otherwise.
+template <int WN>
+__global__ __launch_bounds__(128 * WN, 2) void gptq_gemm_wide_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
     int group_size, int stages_per_block, int split_k) {
+    constexpr int T = 128 * WN;          // threads
+    constexpr int PT = 1024 / T;         // per thread and stage: 16-byte chunks of activations = packed words
+    constexpr int CT = 8 / WN;           // 16-column MFMA tiles per wave
     __shared__ __attribute__((aligned(16))) int8_t smem[2 * 2 * kWideTileBytes];  // [buffer][A | W]
     auto As = [&](int buf) { return smem + buf * 2 * kWideTileBytes; };
     auto Ws = [&](int buf) { return smem + buf * 2 * kWideTileBytes + kWideTileBytes; };
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wy = wave >> 1, wx = wave & 1;
+    const int wy = wave / WN, wx = wave % WN;
     const int nl = lane & 15, kq = lane >> 4;
     const int m0 = blockIdx.x * kWideBM, n0 = blockIdx.y * kWideBN;
     const int stages_total = K / kWideBK;
@@ -88,44 +105,40 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
     const int n_stages = min(stages_per_block, stages_total - s_begin);
 
     // ---- what a thread fetches per stage
-    // activations: chunk id j * 256 + tid of the 128 x 8 chunks of the tile
-    int a_off[4], a_lds[4];
+    // activations: chunk id j * T + tid of the 128 x 8 chunks of the tile
+    int a_off[PT], a_lds[PT];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int id = j * 256 + tid, row = id >> 3, c = id & 7;
+    for (int j = 0; j < PT; ++j) {
+        const int id = j * T + tid, row = id >> 3, c = id & 7;
         a_off[j] = (min(m0 + row, M - 1) * K + c * 8) * 2;   // rows past M feed accumulator rows that are never stored
         a_lds[j] = wide_swz(row, c);
     }
-    // weights: column tid % 128, packed rows (tid / 128) * 4 .. + 3 of the stage's eight: four 4-byte
-    // loads (a wave load is 256 contiguous bytes of one packed row), and four LDS writes in which
-    // sixteen consecutive lanes hold sixteen consecutive columns at one chunk index -- the pattern
-    // of the fragment reads, free of bank conflicts (a 16-byte load of four columns per thread
-    // makes every LDS write a four-way conflict, and LDS writes are what this kernel waits for)
-    const int w_prow = (tid >> 7) * 4, w_col = tid & 127;
+    // weights: column tid % 128, PT consecutive packed rows of the stage's eight: 4-byte loads (a wave
+    // load is 256 contiguous bytes of one packed row), and LDS writes in which sixteen consecutive
+    // lanes hold sixteen consecutive columns at one chunk index -- the pattern of the fragment
+    // reads, free of bank conflicts (a 16-byte load of four columns per thread makes every LDS
+    // write a four-way conflict)
+    const int w_prow = (tid >> 7) * PT, w_col = tid & 127;
     const bool w_live = n0 + w_col < N;
     const int w_cg = w_live ? n0 + w_col : 0;                  // a dead thread re-reads column 0 (never stored)
     const int4_t x_rsrc = wide_rsrc(x, (uint32_t)((size_t)M * K * 2));
     const int4_t q_rsrc = wide_rsrc(qweight, (uint32_t)((size_t)(K / 8) * N * 4));
     const int4_t s_rsrc = wide_rsrc(scales, (uint32_t)((size_t)(K / group_size) * N * 2));
     const int4_t z_rsrc = wide_rsrc(qzeros, (uint32_t)((size_t)(K / group_size) * (N / 8) * 4));
-    int q_off[4];
+    int q_off[PT];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) q_off[j] = ((w_prow + j) * N + w_cg) * 4;
+    for (int j = 0; j < PT; ++j) q_off[j] = ((w_prow + j) * N + w_cg) * 4;
 
-    // eight loads per stage, in this order
-    uint4_t ra[2][4];
-    uint32_t rq[2][4];
+    // 2 PT loads per stage, in this order
+    uint4_t ra[2][PT];
+    uint32_t rq[2][PT];
     auto fetch = [&](int slot, int stage) {
         const int s = min(stage, stages_total - 1);            // past the end: a repeat of the last stage, never used
 #pragma unroll
-        for (int j = 0; j < 4; ++j) wide_load_b128(ra[slot][j], a_off[j], x_rsrc, s * kWideBK * 2);
+        for (int j = 0; j < PT; ++j) wide_load_b128(ra[slot][j], a_off[j], x_rsrc, s * kWideBK * 2);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) wide_load_b32_stream(rq[slot][j], q_off[j], q_rsrc, s * (kWideBK / 8) * N * 4);
+        for (int j = 0; j < PT; ++j) wide_load_b32_stream(rq[slot][j], q_off[j], q_rsrc, s * (kWideBK / 8) * N * 4);
     };
-    // everything but the newest NEWEST loads has arrived; the registers of `slot` pass through
-#define WIDE_WAIT(NEWEST, slot) \
-    wide_wait<NEWEST>(ra[slot][0], ra[slot][1], ra[slot][2], ra[slot][3], rq[slot][0], rq[slot][1], rq[slot][2], \
-                      rq[slot][3], raw_s, raw_z)
 
     // per-group constants of the thread's column
     DequantRegs regs;
@@ -143,7 +156,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
         cc = make_column_const(__builtin_bit_cast(half_t, (uint16_t)raw_s), (raw_z >> ((w_cg & 7) * 4)) & 0xFu);
     };
 
-    // registers -> LDS, one quarter of a thread's share: a chunk of activations as it is, one packed
+    // registers -> LDS, one piece of a thread's share: a chunk of activations as it is, one packed
     // word dequantised into k order
     auto produce_piece = [&](int slot, int buf, int j) {
         *reinterpret_cast<uint4_t*>(As(buf) + a_lds[j]) = ra[slot][j];
@@ -153,16 +166,12 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
         const uint4_t packed = {as_u32(o0), as_u32(o1), as_u32(o2), as_u32(o3)};
         *reinterpret_cast<uint4_t*>(Ws(buf) + wide_swz(w_col, w_prow + j)) = packed;
     };
-    auto produce = [&](int slot, int buf) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) produce_piece(slot, buf, j);
-    };
 
-    float4_t acc[4][4];
+    float4_t acc[4][CT];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < CT; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // ---- pipeline: stage s is fetched during stage s - 2, written to LDS during stage s - 1
     const int spg = group_size / kWideBK;                       // stages per group (group_size is a multiple of 64)
@@ -172,10 +181,11 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
     fetch(0, s_begin);
     fetch_consts(s_begin / spg);
     fetch(1, s_begin + 1);
-    WIDE_WAIT(8, 0);                                            // all but stage s_begin + 1
+    wide_wait<2 * PT, PT>(ra[0], rq[0], raw_s, raw_z);          // all but stage s_begin + 1
     make_consts();
     fetch_consts((s_begin + 1) / spg);
-    produce(0, 0);
+#pragma unroll
+    for (int j = 0; j < PT; ++j) produce_piece(0, 0, j);
     fetch(0, s_begin + 2);
     __syncthreads();
 
@@ -186,30 +196,32 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
         const int stage = s_begin + i;
         // The order below is pinned with scheduling barriers: left alone, the compiler moves the
         // whole of the next stage's LDS writes in front of this stage's MFMAs.  First half: four
-        // groups of four MFMAs, each followed by a quarter of the next stage's production (into the
-        // other buffer, which every wave left at the last barrier); the second half's fragments are
-        // requested under the second group.  Second half: MFMAs only, the loads of stage + 3 first.
-        half8_t fa[2][4], fb[2][4];
+        // groups of MFMAs, the first PT of them followed by a piece of the next stage's production
+        // (into the other buffer, which every wave left at the last barrier); the second half's
+        // fragments are requested under the second group.  Second half: MFMAs only, the loads of
+        // stage + 3 first.
+        half8_t fa[2][4], fb[2][CT];
         auto read_frags = [&](int half) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < 4; ++t)
                 fa[half][t] = *reinterpret_cast<const half8_t*>(As(PAR) + wide_swz(wy * 64 + t * 16 + nl, half * 4 + kq));
-                fb[half][t] = *reinterpret_cast<const half8_t*>(Ws(PAR) + wide_swz(wx * 64 + t * 16 + nl, half * 4 + kq));
-            }
+#pragma unroll
+            for (int t = 0; t < CT; ++t)
+                fb[half][t] = *reinterpret_cast<const half8_t*>(Ws(PAR) + wide_swz((wx * CT + t) * 16 + nl, half * 4 + kq));
         };
         read_frags(0);
         // in flight at this point, oldest first: stage + 1 (other slot), the constants of its group,
-        // stage + 2 (eight loads, may stay in flight)
-        WIDE_WAIT(8, PAR ^ 1);
+        // stage + 2 (2 PT loads, may stay in flight)
+        wide_wait<2 * PT, PT>(ra[PAR ^ 1], rq[PAR ^ 1], raw_s, raw_z);
         make_consts();                                          // of stage + 1
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
+            for (int c = 0; c < CT; ++c)
                 acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[0][r], fb[0][c], acc[r][c], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            produce_piece(PAR ^ 1, PAR ^ 1, r);
+            if (r < PT) produce_piece(PAR ^ 1, PAR ^ 1, r);
             if (r == 1) read_frags(1);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -219,7 +231,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
+            for (int c = 0; c < CT; ++c)
                 acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[1][r], fb[1][c], acc[r][c], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
@@ -233,7 +245,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
     // to the compiler from here on, so let them land before anything else is put there
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- results: acc[r][c][e] is row wy*64 + r*16 + kq*4 + e, column wx*64 + c*16 + nl of the tile
+    // ---- results: acc[r][c][e] is row wy*64 + r*16 + kq*4 + e, column (wx*CT + c)*16 + nl of the tile
 #pragma unroll
     for (int r = 0; r < 4; ++r)
 #pragma unroll
@@ -241,8 +253,8 @@ __global__ __launch_bounds__(kWideThreads, 2) void gptq_gemm_wide_kernel(
             const int m = m0 + wy * 64 + r * 16 + kq * 4 + e;
             if (m >= M) continue;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int n = n0 + wx * 64 + c * 16 + nl;
+            for (int c = 0; c < CT; ++c) {
+                const int n = n0 + (wx * CT + c) * 16 + nl;
                 if (n >= N) continue;
                 if (split_k == 1)
                     out[(size_t)m * N + n] = (half_t)acc[r][c][e];
@@ -279,12 +291,12 @@ static WidePlan plan_wide(int M, int N, int K) {
 bool gemm_wide_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_WIDE");
     if (off && *off && atoi(off)) return false;
-    // measured against the 64-row blocks of the small-M kernel at 4096 x 14336: 128 rows 44.7 against
-    // 37.7 us (too few workgroups for the chip, and split-K partial sums), 256 rows 72.4 / 70.0,
-    // 512 rows 91.9 / 102.1, 2048 rows 316 / 355; MH_GEMM_WIDE_MIN_M moves the switch
+    // measured against the 64-row blocks of the small-M kernel at 4096 x 14336 (us, this kernel /
+    // that one): 128 rows 39.4 / 37.7 (224 workgroups: one per CU, and split-K partial sums), 256 rows
+    // 65.4 / 70.0, 512 rows 91.9 / 102.1, 2048 rows 316 / 355; MH_GEMM_WIDE_MIN_M moves the switch
     static const int min_m = [] {
         const char* v = getenv("MH_GEMM_WIDE_MIN_M");
-        return v && *v ? atoi(v) : 384;
+        return v && *v ? atoi(v) : 192;
     }();
     return bits == 4 && epilogue == kEpilogueNone && M >= min_m && K % kWideBK == 0 && group_size % kWideBK == 0 &&
            K % group_size == 0 && N % 8 == 0 && (size_t)M * K * 2 < ((size_t)1 << 31) &&
@@ -305,9 +317,15 @@ int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qwei
         return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
     float* partial = need ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes) : nullptr;
-    hipLaunchKernelGGL(gptq_gemm_wide_kernel, dim3(p.tiles_m, p.tiles_n, p.split_k), dim3(kWideThreads), 0, stream,
-                       (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
-                       (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k);
+    // one or two row tiles: eight waves per workgroup, so that the few tiles still give every SIMD two waves
+    if (p.tiles_m <= 2)
+        hipLaunchKernelGGL(gptq_gemm_wide_kernel<4>, dim3(p.tiles_m, p.tiles_n, p.split_k), dim3(512), 0, stream,
+                           (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
+                           (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k);
+    else
+        hipLaunchKernelGGL(gptq_gemm_wide_kernel<2>, dim3(p.tiles_m, p.tiles_n, p.split_k), dim3(256), 0, stream,
+                           (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
+                           (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k);
     MH_CHECK_LAUNCH();
     if (p.split_k > 1) {
         launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, SmallFuse{});
