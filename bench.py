@@ -234,35 +234,28 @@ def bench_small_configs(lib, HIPTensor, memory, ws):
     gate_up = [DeviceLinear(lib, HIPTensor, hidden, 2 * ffn, 600 + i) for i in range(sets // 4)]
     down = [DeviceLinear(lib, HIPTensor, ffn, hidden, 700 + i) for i in range(sets // 4)]
     block = []
-    halves = None
     for m in (1, 8, 32, 128):
         x = HIPTensor.allocate((m, hidden), "float16")
         lib.call("mh_synth_normal", None, x.data_ptr, m * hidden, 0.0, 1.0, 0, 0.0, 42, 0)
         h = HIPTensor.allocate((m, ffn), "float16")
         y = HIPTensor.allocate((m, hidden), "float16")
 
-        if m <= 32:   # one launch for gate|up with SiLU*up in its reduction
-            def step(i):
-                gu, dn = gate_up[i % len(gate_up)], down[i % len(down)]
-                lib.call("mh_gptq_matmul_silu_pairs", None, x.data_ptr, gu.qweight.data_ptr, gu.qzeros.data_ptr,
-                         gu.scales.data_ptr, h.data_ptr, m, 2 * ffn, hidden, GROUP, BITS, ws._pointer, ws._size)
-                run_gemv(lib, h, dn, y, ws, m=m)
-        else:         # above 32 rows: gate, up, SiLU*up, down as four launches
-            if halves is None:
-                halves = [DeviceLinear(lib, HIPTensor, hidden, ffn, 800 + i) for i in range(8)]
-            g, u = HIPTensor.allocate((m, ffn), "float16"), HIPTensor.allocate((m, ffn), "float16")
+        # gate|up through mh_gptq_matmul_silu_pairs: up to 32 rows one launch with SiLU*up in its
+        # reduction, above that the fused product and one pass over it; then down
+        ws_pairs = memory.workspace(max(lib.call("mh_gptq_silu_pairs_workspace_bytes", m, 2 * ffn, hidden, GROUP, BITS),
+                                        ws._size))
 
-            def step(i, g=g, u=u):
-                run_gemv(lib, x, halves[(2 * i) % 8], g, ws, m=m)
-                run_gemv(lib, x, halves[(2 * i + 1) % 8], u, ws, m=m)
-                lib.call("mh_silu_mul", None, g.data_ptr, u.data_ptr, h.data_ptr, m * ffn, 0, 0)
-                run_gemv(lib, h, down[i % len(down)], y, ws, m=m)
+        def step(i, ws_pairs=ws_pairs):
+            gu, dn = gate_up[i % len(gate_up)], down[i % len(down)]
+            lib.call("mh_gptq_matmul_silu_pairs", None, x.data_ptr, gu.qweight.data_ptr, gu.qzeros.data_ptr,
+                     gu.scales.data_ptr, h.data_ptr, m, 2 * ffn, hidden, GROUP, BITS, ws_pairs._pointer, ws_pairs._size)
+            run_gemv(lib, h, dn, y, ws_pairs, m=m)
         us = _time_launches(memory, step, iters=40, warmup=4)
         nbytes = linear_bytes(m, hidden, 2 * ffn) - m * ffn * 2 + linear_bytes(m, ffn, hidden)
         block.append({"M": m, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
                       "tflops": round(2.0 * m * 3 * hidden * ffn / us / 1e6, 2)})
     res["mlp_block_cfg1"] = block
-    del gate_up, down, halves
+    del gate_up, down
     # the unquantized lm_head of the decode loop: fp16 [vocab, hidden] (2.1 GB, streamed once per launch)
     vocab, hid = 128256, 8192
     w = HIPTensor.allocate((vocab, hid), "float16")

@@ -152,9 +152,12 @@ int mh_gptq_matmul_static(mh_stream_t stream, const void* x, const int32_t* qwei
  * is up column t*128 + c; qzeros and scales permuted alike -- a load-time
  * permutation of whole 8-column words).  out is [M, N / 2]:
  *   out[m, t*128 + c] = fp16( silu(y[m, t*256 + c]) * y[m, t*256 + 128 + c] ),
- * y the fp16-rounded product, silu and the multiply in fp32.  M <= 32,
- * N % 256 == 0, group_size in {32, 64, 128, 256}; workspace as above and always
- * required. */
+ * y the fp16-rounded product, silu and the multiply in fp32.  N % 256 == 0.  Up to
+ * 32 rows with group_size in {32, 64, 128, 256} it is one launch (the epilogue
+ * runs in the product's reduction); otherwise the product goes to the workspace
+ * and one more pass applies the epilogue.  The workspace is always required:
+ * mh_gptq_silu_pairs_workspace_bytes(M, N, K, ...) bytes, zero-filled once. */
+size_t mh_gptq_silu_pairs_workspace_bytes(int M, int N, int K, int group_size, int bits);
 int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* qweight,
                               const int32_t* qzeros, const void* scales, void* out,
                               int M, int N, int K, int group_size, int bits,

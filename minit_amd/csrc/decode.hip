@@ -153,6 +153,17 @@ __global__ void silu_mul_fused_kernel(const half_t* __restrict__ gu, half_t* __r
     }
 }
 
+int silu_pairs_launch(hipStream_t stream, const void* gate_up, void* out, int rows, int ffn) {
+    const size_t n8 = (size_t)rows * ffn / 8;
+    size_t grid = (n8 + 255) / 256;
+    const size_t cap = (size_t)compute_units() * 16;
+    if (grid > cap) grid = cap;
+    hipLaunchKernelGGL(silu_mul_fused_kernel, dim3((unsigned)grid), dim3(256), 0, stream, (const half_t*)gate_up,
+                       (half_t*)out, rows, ffn);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
 // token[b] = argmax_v logits[b, v] (first maximum); appended to the output
 // stream and fed back as the next input; positions[b] += 1.  out_tokens points
 // at this step's row of the output, or, when pos_base is given, at the whole

@@ -20,6 +20,7 @@ int gptq_generic_launch(hipStream_t stream, const void* x, const int32_t* qweigh
                         const void* scales, const int32_t* g_idx, void* out, int M, int N, int K,
                         int group_size, int bits);
 int gemv_gemm_crossover();
+int silu_pairs_launch(hipStream_t stream, const void* gate_up, void* out, int rows, int ffn);  // decode.hip
 }  // namespace mh
 
 namespace mh {
@@ -184,14 +185,41 @@ int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight, co
                                group_size, bits);
 }
 
+// Where the plain product sits in the workspace of the two-pass SiLU-pairs path: behind what the
+// product itself needs, and never on the arrival counters at the head of a workspace (they must
+// stay zero for every later call that shares the buffer, also when this product needs none).
+static size_t silu_pairs_product_offset(size_t product_bytes) {
+    const size_t floor = product_bytes > kTileCounterBytes ? product_bytes : kTileCounterBytes;
+    return (floor + 255) / 256 * 256;
+}
+
+size_t mh_gptq_silu_pairs_workspace_bytes(int M, int N, int K, int group_size, int bits) {
+    const size_t product = mh_gptq_workspace_bytes(M, N, K, group_size, bits);
+    if (gemm_silu_pairs_supported(M, N, K, group_size, bits)) return product;
+    return silu_pairs_product_offset(product) + (size_t)M * N * sizeof(half_t);
+}
+
 int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                               void* workspace, size_t workspace_bytes) {
     int rc = check_gptq_args("mh_gptq_matmul_silu_pairs", x, qweight, qzeros, scales, out, M, N, K, group_size, bits);
     if (rc) return rc;
     if (M == 0) return MH_OK;
-    return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
-                            workspace, workspace_bytes, kEpilogueSiluPairs, SmallFuse{});
+    MH_REQUIRE(N % 256 == 0, "mh_gptq_matmul_silu_pairs: N=%d must be a multiple of 256 (128 gate + 128 up columns per block)", N);
+    if (gemm_silu_pairs_supported(M, N, K, group_size, bits))
+        return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
+                                workspace, workspace_bytes, kEpilogueSiluPairs, SmallFuse{});
+    // more rows (or a group size) than the fused reduction serves: the product into the workspace,
+    // then one pass that applies silu(gate) * up to the fp16-rounded sums
+    const size_t product = silu_pairs_product_offset(mh_gptq_workspace_bytes(M, N, K, group_size, bits));
+    const size_t need = product + (size_t)M * N * sizeof(half_t);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(MH_ERR_WORKSPACE, "mh_gptq_matmul_silu_pairs: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    half_t* gu = reinterpret_cast<half_t*>(static_cast<char*>(workspace) + product);
+    rc = mh_gptq_matmul(stream, x, qweight, qzeros, scales, nullptr, gu, M, N, K, group_size, bits, workspace, product);
+    if (rc) return rc;
+    return silu_pairs_launch(as_stream(stream), gu, out, M, N / 2);
 }
 
 }  // extern "C"

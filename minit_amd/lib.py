@@ -50,6 +50,7 @@ PROTOTYPES = {
     "mh_gptq_matmul": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_gptq_static_scratch_bytes": (c_size_t, []),
     "mh_gptq_matmul_static": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mh_gptq_silu_pairs_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "mh_gptq_matmul_silu_pairs": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_f16_matmul_nk": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
     "mh_i8_gemm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int]),
@@ -88,7 +89,7 @@ PROTOTYPES = {
 }
 
 # functions whose return value is not a status code
-_NOT_STATUS = {"mh_abi_version", "mh_last_error", "mh_gptq_workspace_bytes", "mh_gptq_static_scratch_bytes", "mh_llama_scratch_bytes",
+_NOT_STATUS = {"mh_abi_version", "mh_last_error", "mh_gptq_workspace_bytes", "mh_gptq_static_scratch_bytes", "mh_gptq_silu_pairs_workspace_bytes", "mh_llama_scratch_bytes",
                "mh_attn_decode_workspace_bytes"}
 
 DTYPE_CODES = {"float16": 0, "bfloat16": 1, "float32": 2}

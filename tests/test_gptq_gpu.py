@@ -268,7 +268,8 @@ def test_operator_api_drop_in(hip):
                                   O.dequantize_packed(qweight, qzeros, scales, None, 4, g).view(np.uint16))
 
 
-@pytest.mark.parametrize("m,k,ffn", [(1, 512, 256), (3, 1024, 384), (8, 256, 128), (16, 512, 256), (32, 768, 512)])
+@pytest.mark.parametrize("m,k,ffn", [(1, 512, 256), (3, 1024, 384), (8, 256, 128), (16, 512, 256), (32, 768, 512),
+                                     (40, 512, 256), (130, 1024, 384)])   # above 32 rows: product, then one pass
 def test_silu_pairs_epilogue(hip, m, k, ffn):
     """gate|up product with SiLU*up applied in the reduction: equals the plain
     product followed by silu(gate) * up on the interleaved column blocks."""
@@ -281,7 +282,7 @@ def test_silu_pairs_epilogue(hip, m, k, ffn):
     x = synthetic.activations("test21", f"x{m}", (m, k))
     dx, dq, dz, ds = _dev(hip, x), _dev(hip, qweight), _dev(hip, qzeros), _dev(hip, scales)
     out = HIPTensor.allocate((m, ffn), "float16")
-    ws = memory.workspace(max(hip.call("mh_gptq_workspace_bytes", m, 2 * ffn, k, g, 4), 256))
+    ws = memory.workspace(max(hip.call("mh_gptq_silu_pairs_workspace_bytes", m, 2 * ffn, k, g, 4), 256))
     hip.call("mh_gptq_matmul_silu_pairs", None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, out.data_ptr,
              m, 2 * ffn, k, g, 4, ws._pointer, ws._size)
     y = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, 4)      # the same device product
