@@ -1,4 +1,4 @@
-from .linalg import matrix_multiply
+from .linalg import batch_matrix_multiply, matrix_multiply
 from .reduce import max, mean, sum
 from .arith import add, multiply
 from .special import rms_norm, rope, sigmoid, softmax

@@ -7,7 +7,7 @@ against the HIP library.
 from ..core.dispatch import register_dispatch
 from ..core.tensor import Tensor
 from ..lib import DTYPE_CODES, call
-from ..operator import Add, MatrixMultiply, Max, Mean, Multiply, RMSNorm, RoPE, Sigmoid, Softmax, Sum
+from ..operator import Add, BatchMatrixMultiply, MatrixMultiply, Max, Mean, Multiply, RMSNorm, RoPE, Sigmoid, Softmax, Sum
 from ..quantize.operator import Dequantize
 from ..quantize.tensor import QuantizedTensor, _NoGroup
 from . import memory
@@ -79,6 +79,22 @@ def dispatch_matmul(op: MatrixMultiply, a: HIPTensor, b: HIPTensor):
     assert a.dtype == b.dtype == "float16"
     c = HIPTensor.allocate((m, n), a.dtype)
     call("mh_f16_matmul_nk", None, a.data_ptr, b.data_ptr, c.data_ptr, m, n, k0)
+    return (c,)
+
+
+@register_dispatch()
+def dispatch_batch_matmul(op: BatchMatrixMultiply, a: HIPTensor, b: HIPTensor):
+    # minit/cuda/dispatch.py:82-101: c[i] = a[i] @ b[i]^T for i < batch, b stored [batch, N, K];
+    # the reference hands the whole batch to one strided library call, here one launch per matrix
+    b0, m, k0 = a._shape
+    b1, n, k1 = b._shape
+    assert b0 == b1
+    assert k0 == k1
+    assert a.dtype == b.dtype == "float16"
+    c = HIPTensor.allocate((b0, m, n), a.dtype)
+    for i in range(b0):
+        call("mh_f16_matmul_nk", None, a.data_ptr + i * m * k0 * 2, b.data_ptr + i * n * k0 * 2,
+             c.data_ptr + i * m * n * 2, m, n, k0)
     return (c,)
 
 

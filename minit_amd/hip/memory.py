@@ -7,6 +7,7 @@ blocks go to a small size-keyed free list so a steady-state loop does not call
 ``hipMalloc`` / ``hipFree`` (which synchronises the device) per tensor.
 """
 import ctypes
+import threading
 from typing import Dict, List
 
 from .. import lib
@@ -130,15 +131,32 @@ def create_stream() -> int:
 
 
 _WORKSPACE = None
+_OWNER_THREAD = None
+
+
+def _single_thread(what: str) -> None:
+    """The operator API is the reference's: one host thread, every launch on the null stream
+    (minit/cuda/dispatch.py passes ``None`` for the stream throughout).  The free list above
+    recycles a block as soon as its tensor dies and the workspace below is shared by every
+    split-K launch; both are only safe while launches are ordered on one stream by one thread,
+    so a second thread is refused instead of silently racing on partial sums."""
+    global _OWNER_THREAD
+    me = threading.get_ident()
+    if _OWNER_THREAD is None:
+        _OWNER_THREAD = me
+    elif _OWNER_THREAD != me:
+        raise lib.HipError(f"{what}: the operator API is single-threaded (null stream); callers with their own "
+                           "threads or streams pass their own workspace to the C ABI")
 
 
 def workspace(nbytes: int) -> HIPMemory:
-    """Zero-initialised scratch shared by the split-K kernels of one stream.
+    """Zero-initialised scratch shared by the split-K kernels of the null stream.
 
     The kernels leave the part that must be zero (their arrival counters) zeroed,
     so the buffer is cleared only when it is (re)allocated.
     """
     global _WORKSPACE
+    _single_thread("memory.workspace")
     if _WORKSPACE is None or _WORKSPACE._size < nbytes:
         size = max(_round(nbytes), 64 << 20)
         synchronize()

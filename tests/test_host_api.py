@@ -184,3 +184,24 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
                           text=True, timeout=120)
     assert proc.returncode != 0 and "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_shared_workspace_refuses_a_second_thread(monkeypatch):
+    """memory.workspace() is one buffer for every split-K launch of the null stream: a second host
+    thread would race on its arrival counters and partial sums, so it is refused."""
+    import threading
+    from minit_amd import lib
+    from minit_amd.hip import memory
+    monkeypatch.setattr(memory, "_OWNER_THREAD", threading.get_ident())
+    memory._single_thread("here")                      # the owner passes
+    seen = []
+
+    def other():
+        try:
+            memory._single_thread("there")
+        except lib.HipError as exc:
+            seen.append(str(exc))
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen and "single-threaded" in seen[0]

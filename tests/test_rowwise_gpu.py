@@ -202,3 +202,16 @@ def test_dense_matmul_nk(hip, m, n, k):
     b = rng.normal(0, 0.05, size=(n, k)).astype(np.float16)
     got = F.matrix_multiply(_t(a), _t(b)).numpy()
     assert_fp16_close(got, a.astype(np.float64) @ b.astype(np.float64).T, what="dense nk")
+
+
+def test_batch_matrix_multiply(hip):
+    """BatchMatrixMultiply (minit/cuda/dispatch.py:82-101): c[i] = a[i] @ b[i]^T, leading axes folded
+    (minit/functional/linalg.py:23-33) -- the two products either side of the models' softmax."""
+    import minit_amd.functional as F
+    rng = np.random.default_rng(12)
+    a = rng.normal(0, 1, size=(2, 3, 5, 128)).astype(np.float16)       # [b, heads, s, d]
+    b = rng.normal(0, 0.2, size=(2, 3, 40, 128)).astype(np.float16)    # [b, heads, t, d]
+    got = F.batch_matrix_multiply(_t(a), _t(b)).numpy()
+    assert got.shape == (2, 3, 5, 40)
+    ref = np.einsum("bhsd,bhtd->bhst", a.astype(np.float64), b.astype(np.float64))
+    assert_fp16_close(got.reshape(-1, 40), ref.reshape(-1, 40), what="batched nk")
