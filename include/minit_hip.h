@@ -125,6 +125,17 @@ int mh_gptq_matmul(mh_stream_t stream, const void* x, const int32_t* qweight,
                    void* out, int M, int N, int K, int group_size, int bits,
                    void* workspace, size_t workspace_bytes);
 
+/* The product with the bias of QLinearWithBias.forward (examples/qwen1_5_int8.py:311-317:
+ * `output = quantized_matrix_multiply(...)`, then `output += bias`, two launches and two fp16
+ * roundings there): out[m, n] = fp16( fp16(y[m, n]) + bias[n] ), bias fp16 [N] or NULL (then
+ * exactly mh_gptq_matmul).  The add rides on the product kernel's own stores -- one launch, or
+ * two where K is split and a second stage adds the partial sums -- except for act-order
+ * weights (g_idx) and group sizes other than 32 / 64 / 128 / 256, where it is a launch of its
+ * own (mh_add_bias).  Workspace as for mh_gptq_matmul. */
+int mh_gptq_linear(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                   const void* scales, const int32_t* g_idx, const void* bias, void* out,
+                   int M, int N, int K, int group_size, int bits, void* workspace, size_t workspace_bytes);
+
 /* mh_gptq_matmul for callers that cannot allocate device memory or pass a
  * workspace: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  No counterpart in the reference (its fused product

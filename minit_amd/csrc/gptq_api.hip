@@ -20,6 +20,7 @@ int gptq_generic_launch(hipStream_t stream, const void* x, const int32_t* qweigh
                         const void* scales, const int32_t* g_idx, void* out, int M, int N, int K,
                         int group_size, int bits);
 int gemv_gemm_crossover();
+bool gemm_bias_supported(int M, int N, int K, int group_size, int bits);
 int silu_pairs_launch(hipStream_t stream, const void* gate_up, void* out, int rows, int ffn);  // decode.hip
 }  // namespace mh
 
@@ -197,6 +198,28 @@ size_t mh_gptq_silu_pairs_workspace_bytes(int M, int N, int K, int group_size, i
     const size_t product = mh_gptq_workspace_bytes(M, N, K, group_size, bits);
     if (gemm_silu_pairs_supported(M, N, K, group_size, bits)) return product;
     return silu_pairs_product_offset(product) + (size_t)M * N * sizeof(half_t);
+}
+
+int mh_gptq_linear(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                   const void* scales, const int32_t* g_idx, const void* bias, void* out, int M, int N, int K,
+                   int group_size, int bits, void* workspace, size_t workspace_bytes) {
+    if (bias == nullptr)
+        return mh_gptq_matmul(stream, x, qweight, qzeros, scales, g_idx, out, M, N, K, group_size, bits, workspace,
+                              workspace_bytes);
+    int rc = check_gptq_args("mh_gptq_linear", x, qweight, qzeros, scales, out, M, N, K, group_size, bits);
+    if (rc) return rc;
+    if (M == 0) return MH_OK;
+    const bool gemv = M <= gemv_gemm_crossover() && gemv_supported(M, N, K, group_size, bits);
+    if (g_idx == nullptr && !gemv && gemm_bias_supported(M, N, K, group_size, bits)) {
+        SmallFuse fuse;  // the bias rides on the product's own stores: one launch (two with a split-K second stage)
+        fuse.bias = static_cast<const half_t*>(bias);
+        return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
+                                workspace, workspace_bytes, kEpilogueNone, fuse);
+    }
+    rc = mh_gptq_matmul(stream, x, qweight, qzeros, scales, g_idx, out, M, N, K, group_size, bits, workspace,
+                        workspace_bytes);
+    if (rc) return rc;
+    return mh_add_bias(stream, out, bias, (size_t)M, (size_t)N, MH_F16);
 }
 
 int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,

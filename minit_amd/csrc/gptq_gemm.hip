@@ -564,7 +564,8 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 for (int t = 0; t < 4; ++t) v[t] = first_of_two ? acc_first[STREAM ? mt : 0][t][r] : acc[mt][t][r];
                 if constexpr (NORM) v *= inv_rms_s[m];
                 if (direct) {
-                    const half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    if (fuse.bias) h = h + *reinterpret_cast<const half4_t*>(fuse.bias + col);
                     *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
                 } else {
                     float* dst = partial + (size_t)slot * plane + (size_t)m * N + col;
@@ -717,7 +718,8 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
             if (c >= N) continue;
             const float4_t s = sum_splits(partial + (size_t)m * N + c);
-            const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+            half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+            if (fuse.bias) h = h + *reinterpret_cast<const half4_t*>(fuse.bias + c);
             *reinterpret_cast<half4_t*>(out + (size_t)m * N + c) = h;
         }
     };
@@ -737,7 +739,7 @@ bool gemm_wide_preferred(int M, int N, int K, int group_size, int bits, int epil
 size_t gemm_wide_workspace_bytes(int M, int N, int K);
 int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                           const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
-                          size_t workspace_bytes);
+                          size_t workspace_bytes, const half_t* bias);
 
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
@@ -873,6 +875,15 @@ bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, i
     return N % (epilogue == kEpilogueResidual ? 1024 : kGemmCols) == 0;
 }
 
+// The bias of a plain product (SmallFuse::bias) is added where the results are stored by every
+// kernel except the staged one (group sizes other than 32 / 64 / 128 / 256).
+bool gemm_bias_supported(int M, int N, int K, int group_size, int bits) {
+    return gemm_supported(M, N, K, group_size, bits) &&
+           (gemm_wide_preferred(M, N, K, group_size, bits, kEpilogueNone) ||
+            gemm_cols_preferred(M, N, K, group_size, bits, kEpilogueNone) ||
+            use_small(M < kSmallMaxM ? M : kSmallMaxM, group_size));
+}
+
 // Per-row pieces a kEpilogueResidual producer leaves in ssq_out for this shape.
 int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
     if (gemm_cols_preferred(M, N, K, group_size, bits, kEpilogueResidual)) return N / 32;
@@ -911,6 +922,7 @@ static void launch_gemm(hipStream_t stream, const GemmPlan& p, const void* x, co
                        p.steps_total, p.steps_per_block, p.split_k);
     if (p.split_k > 1) launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, SmallFuse{});
 }
+
 
 template <int BITS, int MT>
 static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void* x, const int32_t* qweight,
@@ -985,7 +997,7 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     // many rows: the kernel that dequantises a weight tile once for 128 rows
     if (fuse.ssq_in == nullptr && gemm_wide_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_wide_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,
-                                     workspace_bytes);
+                                     workspace_bytes, fuse.bias);
     // a narrow output goes to the kernel whose workgroups own their columns over all of K
     if (gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_cols_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, bits, epilogue, fuse,

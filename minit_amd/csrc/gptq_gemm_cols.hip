@@ -371,7 +371,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         *reinterpret_cast<half2_t*>(dst) = o;
         return;
     }
-    *op = y;
+    *op = fuse.bias ? y + *reinterpret_cast<const half2_t*>(fuse.bias + col) : y;
 }
 
 bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {

@@ -87,7 +87,7 @@ template <int WN>
 __global__ __launch_bounds__(128 * WN, 2) void gptq_gemm_wide_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
-    int group_size, int stages_per_block, int split_k) {
+    int group_size, int stages_per_block, int split_k, const half_t* __restrict__ bias) {
     constexpr int T = 128 * WN;          // threads
     constexpr int PT = 1024 / T;         // per thread and stage: 16-byte chunks of activations = packed words
     constexpr int CT = 8 / WN;           // 16-column MFMA tiles per wave
@@ -257,7 +257,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gptq_gemm_wide_kernel(
                 const int n = n0 + (wx * CT + c) * 16 + nl;
                 if (n >= N) continue;
                 if (split_k == 1)
-                    out[(size_t)m * N + n] = (half_t)acc[r][c][e];
+                    out[(size_t)m * N + n] = bias ? (half_t)acc[r][c][e] + bias[n] : (half_t)acc[r][c][e];
                 else
                     partial[((size_t)blockIdx.z * M + m) * N + n] = acc[r][c][e];
             }
@@ -310,7 +310,7 @@ size_t gemm_wide_workspace_bytes(int M, int N, int K) {
 
 int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                           const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
-                          size_t workspace_bytes) {
+                          size_t workspace_bytes, const half_t* bias) {
     const WidePlan p = plan_wide(M, N, K);
     const size_t need = gemm_wide_workspace_bytes(M, N, K);
     if (need != 0 && (workspace == nullptr || workspace_bytes < need))
@@ -321,14 +321,16 @@ int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qwei
     if (p.tiles_m <= 2)
         hipLaunchKernelGGL(gptq_gemm_wide_kernel<4>, dim3(p.tiles_m, p.tiles_n, p.split_k), dim3(512), 0, stream,
                            (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
-                           (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k);
+                           (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k, bias);
     else
         hipLaunchKernelGGL(gptq_gemm_wide_kernel<2>, dim3(p.tiles_m, p.tiles_n, p.split_k), dim3(256), 0, stream,
                            (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
-                           (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k);
+                           (half_t*)out, partial, M, N, K, group_size, p.stages_per_block, p.split_k, bias);
     MH_CHECK_LAUNCH();
     if (p.split_k > 1) {
-        launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, SmallFuse{});
+        SmallFuse fuse;
+        fuse.bias = bias;
+        launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, fuse);
         MH_CHECK_LAUNCH();
     }
     return MH_OK;

@@ -157,7 +157,8 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
 // out[i] = fp16(sum over splits, in split order).  The kernel boundary makes
 // the partials visible without any device-scope fence or atomic.
 __global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __restrict__ partial,
-                                                              half_t* __restrict__ out, size_t mn, int split_k) {
+                                                              half_t* __restrict__ out, size_t mn, int split_k,
+                                                              const half_t* __restrict__ bias, int N) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
     float4_t s = {0.f, 0.f, 0.f, 0.f};
@@ -170,7 +171,8 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __res
         for (int u = 0; u < 8; ++u) s += v[u];
     }
     for (; sp < split_k; ++sp) s += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
-    const half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+    half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+    if (bias) h = h + *reinterpret_cast<const half4_t*>(bias + i % N);  // N % 8 == 0: four columns of one row
     *reinterpret_cast<half4_t*>(out + i) = h;
 }
 
@@ -274,7 +276,7 @@ void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out,
     const size_t mn = (size_t)M * N;
     const size_t threads = (mn + 3) / 4;
     hipLaunchKernelGGL(splitk_finalize_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
-                       partial, (half_t*)out, mn, split_k);
+                       partial, (half_t*)out, mn, split_k, fuse.bias, N);
 }
 
 // ---- host side -----------------------------------------------------------------------

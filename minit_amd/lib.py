@@ -48,6 +48,7 @@ PROTOTYPES = {
     "mh_gptq_gemv": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_gptq_gemm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_gptq_matmul": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
+    "mh_gptq_linear": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_gptq_static_scratch_bytes": (c_size_t, []),
     "mh_gptq_matmul_static": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int]),
     "mh_gptq_silu_pairs_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),

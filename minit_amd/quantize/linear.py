@@ -3,14 +3,14 @@ packed checkpoint tensors: ``forward(x) = x @ dequant(W) [+ bias]``.
 
 The reference's modules unpack the sub-words into uint8 tensors for their
 ``weight`` property and call a fused kernel in ``forward``; here both go through
-the operator API (``matrix_multiply`` on a :class:`QuantizedTensor`, which the
-HIP rule serves from the packed words), and the bias is the library's in-place
-broadcast add.
+the packed words: ``weight`` is a :class:`QuantizedTensor` (the operator API's
+``matrix_multiply`` serves it as well), and ``forward`` is one ``mh_gptq_linear``
+call, the bias riding on the product kernel's stores.
 """
 from typing import Optional
 
-from ..functional.linalg import matrix_multiply
 from ..lib import DTYPE_CODES, call
+from ..hip import memory
 from ..hip.tensor import HIPTensor
 from .gptq import quantized_tensor_from_host, sort_rows_by_group
 from .tensor import QuantizedTensor
@@ -50,22 +50,28 @@ class QLinear:
         return cls(quantized_tensor_from_host(w.qweight, w.qzeros, w.scales, w.g_idx), bias)
 
     def forward(self, x):
+        """``x [..., K] -> [..., N]``: one ``mh_gptq_linear`` call (product and bias in one launch,
+        examples/qwen1_5_int8.py:311-317 runs them as two), after the gather of the activations'
+        columns when the weight's rows were sorted by group at load time."""
+        w = self.weight
+        k, n = w.in_features, w.out_features
+        assert x._shape[-1] == k, f"x has K={x._shape[-1]}, weight has K={k}"
+        assert x.dtype == "float16" and w._scale.dtype == x.dtype
+        rows = 1
+        for d in x._shape[:-1]:
+            rows *= d
         if self.input_order is not None:
-            k = self.weight.in_features
-            rows = 1
-            for d in x._shape[:-1]:
-                rows *= d
             gathered = HIPTensor.allocate(x._shape, x.dtype)
             call("mh_gather_columns", None, x.data_ptr, self.input_order.data_ptr, gathered.data_ptr, rows, k,
                  DTYPE_CODES[x.dtype])
             x = gathered
-        out = matrix_multiply(x, self.weight)
-        if self.bias is not None:
-            n = self.weight.out_features
-            rows = 1
-            for d in out._shape[:-1]:
-                rows *= d
-            call("mh_add_bias", None, out.data_ptr, self.bias.data_ptr, rows, n, DTYPE_CODES[out.dtype])
+        out = HIPTensor.allocate((*x._shape[:-1], n), x.dtype)
+        if rows == 0:
+            return out
+        ws = memory.workspace(max(call("mh_gptq_workspace_bytes", rows, n, k, w.group_size, w.bits), 256))
+        call("mh_gptq_linear", None, x.data_ptr, w._data.data_ptr, w._zero.data_ptr, w._scale.data_ptr,
+             None if w._group is None else w._group.data_ptr, None if self.bias is None else self.bias.data_ptr,
+             out.data_ptr, rows, n, k, w.group_size, w.bits, ws._pointer, ws._size)
         return out
 
     __call__ = forward

@@ -236,6 +236,76 @@ def test_act_order_through_matmul(hip):
     assert_fp16_close(got, ref, what="act-order")
 
 
+def _run_with_bias(hip, x, qweight, qzeros, scales, bias, group_size, bits, g_idx=None):
+    """(mh_gptq_linear's output, mh_gptq_matmul's, the latter after mh_add_bias)."""
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.lib import DTYPE_CODES
+    m, k = x.shape
+    n = qweight.shape[1]
+    dx, dq, dz, ds, db = (_dev(hip, a) for a in (x, qweight, qzeros, scales, bias))
+    dg = None if g_idx is None else _dev(hip, g_idx.astype(np.int32))
+    ws = memory.workspace(max(hip.call("mh_gptq_workspace_bytes", m, n, k, group_size, bits), 256))
+    outs = []
+    for entry in ("mh_gptq_linear", "mh_gptq_matmul"):
+        out = HIPTensor.from_numpy(np.full((m, n), np.nan, np.float16))
+        args = [None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, None if dg is None else dg.data_ptr]
+        if entry == "mh_gptq_linear":
+            args.append(db.data_ptr)
+        hip.call(entry, *args, out.data_ptr, m, n, k, group_size, bits, ws._pointer, ws._size)
+        outs.append(out.numpy())
+        if entry == "mh_gptq_matmul":
+            hip.call("mh_add_bias", None, out.data_ptr, db.data_ptr, m, n, DTYPE_CODES["float16"])
+            outs.append(out.numpy())
+    return outs
+
+
+# one case per place where a product kernel stores results: the column-owner kernel, the small-M
+# kernel's direct store, its in-kernel split-K reduction, the split-K second stage, row-blocked
+# launches, the wide kernel with four and with eight waves (direct and split), the 8-bit kernels;
+# then the launches that add the bias in a pass of their own (odd group size, act-order, VALU rows)
+@pytest.mark.parametrize("m,k,n,g,bits,act_order", [
+    (1, 1024, 256, 128, 4, False), (1, 4096, 8192, 128, 4, False), (1, 8192, 1024, 128, 4, False),
+    (4, 512, 28672, 128, 4, False), (8, 4096, 4096, 128, 4, False), (16, 4096, 1024, 128, 4, False),
+    (32, 2048, 2048, 64, 4, False), (100, 1024, 1536, 128, 4, False), (130, 4096, 512, 128, 4, False),
+    (200, 2048, 1024, 128, 4, False), (400, 1024, 2048, 64, 4, False), (256, 8192, 256, 128, 4, False),
+    (1, 2048, 2048, 128, 8, False), (24, 1024, 768, 64, 8, False), (300, 512, 512, 128, 8, False),
+    (3, 768, 264, 96, 4, False), (5, 1024, 512, 512, 4, False), (6, 1024, 256, 128, 4, True),
+])
+def test_linear_with_bias_is_the_product_then_one_fp16_add(hip, m, k, n, g, bits, act_order):
+    """mh_gptq_linear == mh_gptq_matmul followed by mh_add_bias == fp16(product + bias) computed
+    on the host from the device's fp16 product, all bit for bit (the bias is added to the
+    fp16-rounded product in fp16 wherever the kernels store it); the product itself against the
+    oracle."""
+    from minit_amd import synthetic
+    qweight, qzeros, scales = _weights(k, n, g, bits, seed=60 + m)
+    rng = np.random.default_rng(m * 7 + k)
+    bias = rng.normal(0, 0.5, size=(n,)).astype(np.float16)
+    g_idx = rng.permutation(k).astype(np.int32) // g if act_order else None
+    x = synthetic.activations("test60", f"x{m}x{k}", (m, k))
+    fused, product, two_pass = _run_with_bias(hip, x, qweight, qzeros, scales, bias, g, bits, g_idx)
+    np.testing.assert_array_equal(fused.view(np.uint16), two_pass.view(np.uint16))
+    np.testing.assert_array_equal(fused.view(np.uint16), (product + bias[None, :]).astype(np.float16).view(np.uint16))
+    assert_fp16_close(product, O.matmul_f64(x, qweight, qzeros, scales, g_idx, bits, g),
+                      what=f"product of linear {m}x{k}x{n}")
+
+
+def test_linear_without_bias_is_the_product(hip):
+    from minit_amd import synthetic
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    m, k, n, g = 7, 1024, 512, 128
+    qweight, qzeros, scales = _weights(k, n, g, 4, seed=77)
+    x = synthetic.activations("test77", "x", (m, k))
+    want = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, 4)
+    dx, dq, dz, ds = (_dev(hip, a) for a in (x, qweight, qzeros, scales))
+    out = HIPTensor.allocate((m, n), "float16")
+    ws = memory.workspace(max(hip.call("mh_gptq_workspace_bytes", m, n, k, g, 4), 256))
+    hip.call("mh_gptq_linear", None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, None, None,
+             out.data_ptr, m, n, k, g, 4, ws._pointer, ws._size)
+    np.testing.assert_array_equal(out.numpy().view(np.uint16), want.view(np.uint16))
+
+
 def test_bad_arguments_are_reported(hip):
     from minit_amd.lib import HipError
     with pytest.raises(HipError, match="bits"):
