@@ -291,16 +291,20 @@ static WidePlan plan_wide(int M, int N, int K) {
 bool gemm_wide_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_WIDE");
     if (off && *off && atoi(off)) return false;
-    // measured against the 64-row blocks of the small-M kernel at 4096 x 14336 (us, this kernel /
-    // that one): 128 rows 39.4 / 37.7 (224 workgroups: one per CU, and split-K partial sums), 256 rows
-    // 65.4 / 70.0, 512 rows 91.9 / 102.1, 2048 rows 316 / 355; MH_GEMM_WIDE_MIN_M moves the switch
+    // measured against the 64-row blocks of the small-M kernel (us, this kernel / that one): 4096 x 14336 at
+    // 192 rows 54.9 / 60.4, 256 rows 57.1 / 63.6, 512 rows 90.3 / 97.0, 2048 rows 315 / 336; 8192 x 28672 at 256
+    // rows 159 / 173; 128 rows 39.4 / 37.7 (224 workgroups: one per CU, and split-K partial sums).  With few
+    // tiles (14336 x 4096: 64 at 256 rows, 128 at 512) the long K walk of a tile needs a split whose fp32
+    // partial sums cost more than the shared dequantisation saves (63.9 / 57.8 and, unsplit, 186 / 89), so
+    // the tiles must cover three quarters of the CUs; MH_GEMM_WIDE_MIN_M moves the row switch
     static const int min_m = [] {
         const char* v = getenv("MH_GEMM_WIDE_MIN_M");
         return v && *v ? atoi(v) : 192;
     }();
-    return bits == 4 && epilogue == kEpilogueNone && M >= min_m && K % kWideBK == 0 && group_size % kWideBK == 0 &&
-           K % group_size == 0 && N % 8 == 0 && (size_t)M * K * 2 < ((size_t)1 << 31) &&
-           (size_t)K * N / 2 < ((size_t)1 << 31);
+    const long tiles = (long)((M + kWideBM - 1) / kWideBM) * ((N + kWideBN - 1) / kWideBN);
+    return bits == 4 && epilogue == kEpilogueNone && M >= min_m && 4 * tiles >= 3L * compute_units() &&
+           K % kWideBK == 0 && group_size % kWideBK == 0 && K % group_size == 0 && N % 8 == 0 &&
+           (size_t)M * K * 2 < ((size_t)1 << 31) && (size_t)K * N / 2 < ((size_t)1 << 31);
 }
 
 size_t gemm_wide_workspace_bytes(int M, int N, int K) {

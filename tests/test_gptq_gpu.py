@@ -172,11 +172,13 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     assert_fp16_close(got, ref, what=f"gemm {m}x{k}x{n} b{bits}")
 
 
+# the kernel takes launches of at least 192 tiles of 128 x 128 (three quarters of the CUs)
 @pytest.mark.parametrize("m,k,n,group_size", [
-    (384, 1024, 776, 128),     # ragged last column tile, unsplit
-    (500, 2048, 256, 64),      # ragged last row tile, two groups per 128 k
-    (512, 8192, 128, 128),     # one column tile, K split over workgroups (partial sums + second stage)
-    (1000, 1024, 1032, 256),   # groups longer than a stage
+    (384, 256, 8200, 128),     # 3 x 65 tiles, ragged last column tile, unsplit, four waves per workgroup
+    (500, 512, 6144, 64),      # 4 x 48 tiles, ragged last row tile, two groups per 128 k
+    (192, 6144, 12288, 128),   # 2 x 96 tiles, eight waves per workgroup, K split in two (partial sums + second stage)
+    (1000, 512, 3080, 256),    # 8 x 25 tiles, groups longer than a stage
+    (512, 8192, 128, 128),     # too few tiles: stays with the 64-row blocks of the small-M kernel
 ])
 def test_gemm_many_rows(hip, m, k, n, group_size):
     """Several hundred rows: the kernel that stages dequantised fp16 weight tiles in LDS."""
@@ -268,7 +270,7 @@ def _run_with_bias(hip, x, qweight, qzeros, scales, bias, group_size, bits, g_id
     (1, 1024, 256, 128, 4, False), (1, 4096, 8192, 128, 4, False), (1, 8192, 1024, 128, 4, False),
     (4, 512, 28672, 128, 4, False), (8, 4096, 4096, 128, 4, False), (16, 4096, 1024, 128, 4, False),
     (32, 2048, 2048, 64, 4, False), (100, 1024, 1536, 128, 4, False), (130, 4096, 512, 128, 4, False),
-    (200, 2048, 1024, 128, 4, False), (400, 1024, 2048, 64, 4, False), (256, 8192, 256, 128, 4, False),
+    (200, 512, 12288, 128, 4, False), (400, 256, 6144, 64, 4, False), (192, 6144, 12288, 128, 4, False),
     (1, 2048, 2048, 128, 8, False), (24, 1024, 768, 64, 8, False), (300, 512, 512, 128, 8, False),
     (3, 768, 264, 96, 4, False), (5, 1024, 512, 512, 4, False), (6, 1024, 256, 128, 4, True),
 ])
