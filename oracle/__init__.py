@@ -25,6 +25,14 @@ so none of this is pinned by the reference's own fixtures):
                        to one, RoPE at position 0 is the identity and composes
                        additively, RMSNorm of a constant row is sign * weight,
                        the sum of ones is the row length).
+* ``decode.*``         a known-answer decode step computed scalar by scalar
+                       with python floats (two layers, grouped heads, rows at
+                       different positions) held bit for bit, and constructed
+                       models whose logits the mathematics fixes (zeroed o and
+                       down projections, one visible cache entry, a zero norm
+                       weight, batch-row permutations); seeded slips in the
+                       operator order fail them.
 
-The checks live in ``tests/test_oracle_*.py``.
+The checks live in ``tests/test_oracle_*.py``; no function here is left
+unpinned.
 """
