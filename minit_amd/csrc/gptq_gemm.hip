@@ -741,6 +741,13 @@ int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qwei
                           const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
                           size_t workspace_bytes, const half_t* bias);
 
+// gptq_gemm_tall.hip: blocks of 128 rows, weights dequantised in registers, K sliced over the waves
+bool gemm_tall_preferred(int M, int N, int K, int group_size, int bits, int epilogue);
+size_t gemm_tall_workspace_bytes(int M, int N, int K);
+int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                          const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
+                          size_t workspace_bytes, const half_t* bias);
+
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
     int col_tiles;
@@ -879,7 +886,8 @@ bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, i
 // kernel except the staged one (group sizes other than 32 / 64 / 128 / 256).
 bool gemm_bias_supported(int M, int N, int K, int group_size, int bits) {
     return gemm_supported(M, N, K, group_size, bits) &&
-           (gemm_wide_preferred(M, N, K, group_size, bits, kEpilogueNone) ||
+           (gemm_tall_preferred(M, N, K, group_size, bits, kEpilogueNone) ||
+            gemm_wide_preferred(M, N, K, group_size, bits, kEpilogueNone) ||
             gemm_cols_preferred(M, N, K, group_size, bits, kEpilogueNone) ||
             use_small(M < kSmallMaxM ? M : kSmallMaxM, group_size));
 }
@@ -893,6 +901,7 @@ int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
 static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_small(kSmallMaxM, group_size); }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
+    if (gemm_tall_preferred(M, N, K, group_size, bits, kEpilogueNone)) return gemm_tall_workspace_bytes(M, N, K);
     if (gemm_wide_preferred(M, N, K, group_size, bits, kEpilogueNone)) return gemm_wide_workspace_bytes(M, N, K);
     if (row_blocked(M, group_size)) {
         // blocks of kSmallBlockM rows in one launch; partial sums [split][M][N]
@@ -994,6 +1003,10 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     if (!packed_weights_addressable(N, K, bits))
         return fail(MH_ERR_INVALID, "gptq gemm: packed weights of 2 GiB or more are not supported by the MFMA kernels "
                     "(mh_gptq_matmul serves them with the per-element kernel)");
+    // more than 64 rows: blocks of 128 rows, a packed word dequantised once per block
+    if (fuse.ssq_in == nullptr && gemm_tall_preferred(M, N, K, group_size, bits, epilogue))
+        return gptq_gemm_tall_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,
+                                     workspace_bytes, fuse.bias);
     // many rows: the kernel that dequantises a weight tile once for 128 rows
     if (fuse.ssq_in == nullptr && gemm_wide_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_wide_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,

@@ -1,0 +1,396 @@
+// GPTQ w4a16 product for blocks of 128 rows: weights dequantised in registers, straight into
+// the B operand of v_mfma_f32_16x16x32_f16, activations fetched by LDS-destination loads.
+//
+// Replaces the same reference pair as the other product kernels
+// (minit/quantize/dispatch.py:8-11 = Dequantize, then MatrixMultiply) between the small-M
+// kernel (a packed word dequantised once per 64 rows, one wave per SIMD at these sizes) and
+// several hundred rows.
+//
+// A workgroup of eight waves owns 128 rows x 128 columns over a K range, walked in rounds of
+// 128 k.  Wave (cg, ks) owns all 128 rows x 64 columns (cg = 0, 1) and the ks-th 32 k of every
+// round (ks = 0..3): 8 x 4 MFMA tiles, 128 accumulator registers, so a packed word is
+// dequantised once for 128 rows and the 32 MFMAs of a 32-k step (512 cycles) outweigh its ~80
+// vector instructions.  Lane (j, o) of a
+// wave holds columns 4j..4j+3 of the wave's 64 -- MFMA tile c takes column 4j + c -- and the
+// o-th eight k of the step: its four packed words are one 16-byte load, its four scales one
+// 8-byte load, its four zero points sit in one word.
+//
+// Per round every wave advances one step:
+//   * all global loads are issued from inline assembly and waited for by hand; one
+//     s_waitcnt vmcnt(14) per round covers everything the round consumes: the packed words and
+//     constants of step r + 1 (requested four rounds ahead into a ring of four) and the
+//     activation stage of round r (requested three rounds ahead into one of four 32 KiB LDS
+//     buffers by buffer_load_dwordx4 ... lds: 128 rows x 256 bytes as two halves of 128-byte
+//     rows; one load fills 1 KiB = eight rows of a half, whole 128-byte lines of the
+//     activation matrix -- with 64-byte pieces every line crossed the L2-to-CU path twice and
+//     the round took 1.35 us instead of the MFMAs' 0.62 -- and since the LDS side of such a
+//     load is lane-linear, the XOR swizzle that keeps the A-operand reads (16 rows x one
+//     16-byte chunk per quarter wave) free of bank conflicts is applied to the global address);
+//   * one barrier;
+//   * the 32 MFMAs of step r, with the round's seven loads and the dequantisation of step r + 1 (13 instructions per word
+//     = the bit-exact W of Dequantize, 4 to put the pairs back into k order) placed between
+//     them in four pieces.
+// At the end the four waves' shares of K are added through LDS (fixed order), the tile is turned into
+// row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias) or, with
+// K split over blockIdx.y, fp32 partial sums for splitk_finalize_kernel.
+#include "gptq_common.h"
+
+#include <type_traits>
+
+namespace mh {
+
+constexpr int kTallBM = 128, kTallBN = 128;
+constexpr int kTallRoundK = 128;                 // four waves x one 32-k step
+constexpr int kTallThreads = 512;
+constexpr int kTallStageBytes = 2 * 128 * 128;   // [half of the round's k][row][64 k], chunks swizzled
+constexpr int kTallStages = 4;
+
+void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
+                            int epilogue, const SmallFuse& fuse);
+
+__device__ __forceinline__ int tall_swz(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+__device__ __forceinline__ int4_t tall_rsrc(const void* base, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    int4_t r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xffffu));
+    r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+    r[3] = kBufferRsrcFlags;
+    return r;
+}
+// Loads the compiler does not count (see the waits below); out-of-range records read as zero.
+__device__ __forceinline__ void tall_load_b128_stream(uint4_t& dst, int voffset, const int4_t& rsrc, int soffset) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen sc1 nt" : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+__device__ __forceinline__ void tall_load_b64(uint2_t& dst, int voffset, const int4_t& rsrc, int soffset) {
+    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+__device__ __forceinline__ void tall_load_b32(uint32_t& dst, int voffset, const int4_t& rsrc, int soffset) {
+    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(dst) : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+// 16 bytes per lane, global -> LDS at m0 + lane * 16.
+__device__ __forceinline__ void tall_load_to_lds(uint32_t lds_addr, int voffset, const int4_t& rsrc, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+// Everything but the newest NEWEST loads has arrived; the registers read next pass through the
+// wait, so that no use can be scheduled above it.
+template <int NEWEST>
+__device__ __forceinline__ void tall_wait(uint4_t& q, uint2_t& s, uint32_t& z) {
+    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(q), "+v"(s), "+v"(z) : "n"(NEWEST) : "memory");
+}
+
+__global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
+    const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
+    int group_size, int rounds_per_block, int split_k, const half_t* __restrict__ bias) {
+    __shared__ __attribute__((aligned(1024))) int8_t smem[kTallStages * kTallStageBytes];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cg = wave & 1, ks = wave >> 1;
+    const int j = lane & 15, o = lane >> 4;
+    const int n0 = blockIdx.x * kTallBN, m0 = blockIdx.z * kTallBM;
+    const int rounds_total = K / kTallRoundK;
+    const int r_begin = blockIdx.y * rounds_per_block;
+    const int n_rounds = min(rounds_per_block, rounds_total - r_begin);
+    // this wave's 32 k of the workgroup's first round
+    const int k_wave = r_begin * kTallRoundK + ks * 32;
+    const int col = n0 + cg * 64 + 4 * j;  // first of the lane's four columns
+
+    const int4_t x_rsrc = tall_rsrc(x, (uint32_t)((size_t)M * K * 2));
+    const int4_t w_rsrc = tall_rsrc(qweight, (uint32_t)((size_t)(K / 8) * N * 4));
+    const int4_t s_rsrc = tall_rsrc(scales, (uint32_t)((size_t)(K / group_size) * N * 2));
+    const int4_t z_rsrc = tall_rsrc(qzeros, (uint32_t)((size_t)(K / group_size) * (N / 8) * 4));
+    const int4_t none = tall_rsrc(x, 0u);  // zero records: no traffic, zeros returned
+
+    // ---- what a lane fetches per round
+    // activations: of the stage's 32 pieces of 1 KiB (half h, rows 8p .. 8p+7) this wave loads h = wave / 4,
+    // p = (wave % 4) * 4 + i; lane l lands at row 8p + l / 8, chunk position l % 8, which holds the
+    // chunk (l % 8) ^ swizzle(row); rows past M are past the end of the buffer and read as zero
+    int x_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = ((wave & 3) * 4 + i) * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+        x_off[i] = ((m0 + row) * K + r_begin * kTallRoundK + (wave >> 2) * 64 + chunk * 8) * 2;
+    }
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)smem);
+    const uint32_t lds_wave = lds0 + (uint32_t)((wave >> 2) * 16 + (wave & 3) * 4) * 1024u;
+    const int w_off = ((k_wave / 8 + o) * N + col) * 4;
+    const int s_off = col * 2, z_off = (col >> 3) * 4;
+    const int z_shift = (j & 1) * 16;  // the lane's four zero points: nibbles 4 (j & 1) .. + 3 of the word
+
+    uint4_t rq[4];   // packed words of steps r .. r + 3
+    uint2_t rs[4];   // their scales
+    uint32_t rz[4];  // their zero-point words
+    // group of the step whose loads are issued next / whose constants are built next
+    int load_group = __builtin_amdgcn_readfirstlane(k_wave / group_size);
+    int load_in_group = __builtin_amdgcn_readfirstlane(k_wave % group_size);
+    int use_in_group = load_in_group;
+    // The seven loads that go with step `step`, in their fixed order: piece 0 the packed words, 1 the scales,
+    // 2 the zero points (all into ring slot S), 3..6 the four 1 KiB pieces of the activation stage of round
+    // step - 1 (into buffer (step - 1) % 4).  The main loop spreads the pieces over the round's MFMAs: issued
+    // back to back by all eight waves right after the barrier they fill the vector memory queue, and the
+    // waves stall in issue with the matrix pipes idle.
+    auto issue_piece = [&](auto slot, auto piece, int step) {
+        constexpr int S = decltype(slot)::value, I = decltype(piece)::value;
+        const bool live = step < n_rounds;
+        if constexpr (I == 0) tall_load_b128_stream(rq[S], w_off, live ? w_rsrc : none, step * 64 * N);
+        if constexpr (I == 1)
+            tall_load_b64(rs[S], s_off, live ? s_rsrc : none, __builtin_amdgcn_readfirstlane(load_group * N * 2));
+        if constexpr (I == 2) {
+            tall_load_b32(rz[S], z_off, live ? z_rsrc : none, __builtin_amdgcn_readfirstlane(load_group * (N / 8) * 4));
+            load_in_group += kTallRoundK;
+            while (load_in_group >= group_size) {
+                load_in_group -= group_size;
+                ++load_group;
+            }
+        }
+        if constexpr (I >= 3) {
+            const int stage = step - 1;
+            const uint32_t base = lds_wave + (uint32_t)((S + 3) & 3) * kTallStageBytes;
+            tall_load_to_lds(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], stage < n_rounds ? x_rsrc : none, stage * 256);
+        }
+    };
+    auto issue = [&](auto slot, int step, bool with_stage) {
+        issue_piece(slot, std::integral_constant<int, 0>{}, step);
+        issue_piece(slot, std::integral_constant<int, 1>{}, step);
+        issue_piece(slot, std::integral_constant<int, 2>{}, step);
+        if (with_stage) {
+            issue_piece(slot, std::integral_constant<int, 3>{}, step);
+            issue_piece(slot, std::integral_constant<int, 4>{}, step);
+            issue_piece(slot, std::integral_constant<int, 5>{}, step);
+            issue_piece(slot, std::integral_constant<int, 6>{}, step);
+        }
+    };
+
+    DequantRegs regs;
+    regs.init(4);
+    ColumnConst cc[4];
+    auto make_consts = [&](const uint2_t& s, uint32_t z) {
+        const half4_t sv = __builtin_bit_cast(half4_t, s);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) cc[c] = make_column_const(sv[c], (z >> (z_shift + 4 * c)) & 0xFu);
+    };
+    // one packed word -> the B operand of MFMA tile c: k0 .. k7 of column 4j + c
+    auto dequant_piece = [&](half8_t& b, uint32_t word, int c) {
+        half2_t w[4];
+        dequant_word<4>(word, cc[c], regs, w);
+        b = half8_t{w[0][0], w[1][0], w[2][0], w[3][0], w[0][1], w[1][1], w[2][1], w[3][1]};
+    };
+
+    // A operand of row tile rt: row rt*16 + j, chunk (ks & 1)*4 + o of the wave's half; the swizzle of
+    // row rt*16 + j does not depend on rt
+    const int a_off = tall_swz(j, (ks & 1) * 4 + o);
+    float4_t acc[8][4];
+#pragma unroll
+    for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[rt][c] = float4_t{0.f, 0.f, 0.f, 0.f};
+    half8_t b[2][4];
+
+    // ---- prologue: the loads of the virtual rounds -4 .. -1, then the operands of step 0
+    issue(std::integral_constant<int, 0>{}, 0, false);
+    issue(std::integral_constant<int, 1>{}, 1, true);
+    issue(std::integral_constant<int, 2>{}, 2, true);
+    issue(std::integral_constant<int, 3>{}, 3, true);
+    tall_wait<0>(rq[0], rs[0], rz[0]);
+    make_consts(rs[0], rz[0]);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) dequant_piece(b[0][c], rq[0][c], c);
+
+    // ---- one round: S = r % 4 (ring slot, stage buffer), P = r % 2 (B operand set)
+    auto round = [&](auto slot, int r) {
+        constexpr int S = decltype(slot)::value, P = S & 1, S1 = (S + 1) & 3;
+        // done after this wait: everything up to the stage of round r, which includes the words and
+        // constants of step r + 1; still in flight: the 2 x 7 loads of the last two rounds
+        tall_wait<14>(rq[S1], rs[S1], rz[S1]);
+        __syncthreads();
+        // from here on slot S is free (step r was dequantised last round) and so is the stage buffer of
+        // round r - 1: the loads of step r + 4 and stage r + 3 go out between the MFMAs below
+        use_in_group += kTallRoundK;
+        if (use_in_group >= group_size) {  // step r + 1 lies in another group than step r
+            do use_in_group -= group_size; while (use_in_group >= group_size);
+            make_consts(rs[S1], rz[S1]);
+        }
+        const int8_t* stage = smem + S * kTallStageBytes + (ks >> 1) * 16384 + a_off;
+        half8_t a[8];
+#pragma unroll
+        for (int rt = 0; rt < 8; ++rt) a[rt] = *reinterpret_cast<const half8_t*>(stage + rt * 2048);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int rt = 0; rt < 8; ++rt) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                acc[rt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[rt], b[P][c], acc[rt][c], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (rt == 0) issue_piece(slot, std::integral_constant<int, 0>{}, r + 4);
+            if (rt == 1) issue_piece(slot, std::integral_constant<int, 1>{}, r + 4);
+            if (rt == 2) issue_piece(slot, std::integral_constant<int, 2>{}, r + 4);
+            if (rt == 3) issue_piece(slot, std::integral_constant<int, 3>{}, r + 4);
+            if (rt == 4) issue_piece(slot, std::integral_constant<int, 4>{}, r + 4);
+            if (rt == 5) issue_piece(slot, std::integral_constant<int, 5>{}, r + 4);
+            if (rt == 6) issue_piece(slot, std::integral_constant<int, 6>{}, r + 4);
+            if (rt & 1) dequant_piece(b[P ^ 1][rt >> 1], rq[S1][rt >> 1], rt >> 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int r = 0; r < n_rounds; r += 4) {
+        round(std::integral_constant<int, 0>{}, r);
+        if (r + 1 < n_rounds) round(std::integral_constant<int, 1>{}, r + 1);
+        if (r + 2 < n_rounds) round(std::integral_constant<int, 2>{}, r + 2);
+        if (r + 3 < n_rounds) round(std::integral_constant<int, 3>{}, r + 3);
+    }
+
+    // the loads requested past the end are still in flight: their registers are dead to the compiler
+    // and their stages would land in LDS that the reduction is about to use
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    // ---- the four quarters of K, added in a fixed order: (0 + 1) + (2 + 3)
+    // a wave's accumulators as 32 blocks of 1 KiB, lane-linear on both sides
+    auto put = [&](int region) {
+        float4_t* dst = reinterpret_cast<float4_t*>(smem + region * 32768) + lane;
+#pragma unroll
+        for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) dst[(rt * 4 + c) * 64] = acc[rt][c];
+    };
+    auto add = [&](int region) {
+        const float4_t* src = reinterpret_cast<const float4_t*>(smem + region * 32768) + lane;
+#pragma unroll
+        for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[rt][c] += src[(rt * 4 + c) * 64];
+    };
+    if (ks & 1) put((ks >> 1) * 2 + cg);
+    __syncthreads();
+    if (!(ks & 1)) add((ks >> 1) * 2 + cg);
+    __syncthreads();
+    if (ks == 2) put(cg);
+    __syncthreads();
+    if (ks == 0) add(cg);
+    __syncthreads();
+
+    // ---- results: acc[rt][c][e] of a ks = 0 wave is row rt*16 + o*4 + e, column cg*64 + 4j + c of the tile
+    if (split_k == 1) {
+        constexpr int kRow = 256 + 16;  // bytes per tile row in LDS
+        if (ks == 0) {
+#pragma unroll
+            for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const half4_t h = {(half_t)acc[rt][0][e], (half_t)acc[rt][1][e], (half_t)acc[rt][2][e], (half_t)acc[rt][3][e]};
+                    *reinterpret_cast<half4_t*>(smem + (rt * 16 + o * 4 + e) * kRow + (cg * 64 + 4 * j) * 2) = h;
+                }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int id = i * kTallThreads + tid, row = id >> 4, ch = id & 15;
+            const int m = m0 + row, n = n0 + ch * 8;
+            if (m >= M || n >= N) continue;
+            half8_t h = *reinterpret_cast<const half8_t*>(smem + row * kRow + ch * 16);
+            if (bias) h = h + *reinterpret_cast<const half8_t*>(bias + n);
+            *reinterpret_cast<half8_t*>(out + (size_t)m * N + n) = h;
+        }
+    } else {
+        constexpr int kRow = 512 + 16;
+        if (ks == 0) {
+#pragma unroll
+            for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float4_t v = {acc[rt][0][e], acc[rt][1][e], acc[rt][2][e], acc[rt][3][e]};
+                    *reinterpret_cast<float4_t*>(smem + (rt * 16 + o * 4 + e) * kRow + (cg * 64 + 4 * j) * 4) = v;
+                }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int id = i * kTallThreads + tid, row = id >> 5, ch = id & 31;
+            const int m = m0 + row, n = n0 + ch * 4;
+            if (m >= M || n >= N) continue;
+            *reinterpret_cast<float4_t*>(partial + ((size_t)blockIdx.y * M + m) * N + n) =
+                *reinterpret_cast<const float4_t*>(smem + row * kRow + ch * 16);
+        }
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------
+
+struct TallPlan {
+    int tiles_n, row_blocks, split_k, rounds_per_block;
+};
+
+static TallPlan plan_tall(int M, int N, int K) {
+    TallPlan p;
+    p.tiles_n = (N + kTallBN - 1) / kTallBN;
+    p.row_blocks = (M + kTallBM - 1) / kTallBM;
+    const int rounds = K / kTallRoundK;
+    // one workgroup per CU (eight waves, 128 KiB of LDS); a workgroup keeps at least four rounds, and
+    // the fp32 partial sums (8 M N bytes per split, written and read) stay below the packed weights' bytes
+    long split = (long)compute_units() / ((long)p.tiles_n * p.row_blocks);
+    if (split > rounds / 4) split = rounds / 4;
+    const long traffic_cap = (long)K / (16L * (M < kTallBM ? M : kTallBM));
+    if (split > traffic_cap) split = traffic_cap;
+    if (split < 1) split = 1;
+    p.rounds_per_block = (int)((rounds + split - 1) / split);
+    p.split_k = (rounds + p.rounds_per_block - 1) / p.rounds_per_block;
+    return p;
+}
+
+static int tall_min_m() {
+    static const int v = [] {
+        const char* e = getenv("MH_GEMM_TALL_MIN_M");
+        return e && *e ? atoi(e) : 65;
+    }();
+    return v;
+}
+
+// Measured on one box against what served these shapes before (the small-M kernel's 64-row blocks up to
+// 191 rows, the LDS-staged kernel above; us, this kernel / before): 4096 x 28672 at 65 / 128 / 256 / 2048
+// rows 38.7 / 58.6, 41.2 / 62.3, 75.2 / 80.5, 561 / 567; 4096 x 14336: 29.1 / 33.0, 36.5 / 35.9, 40.1 /
+// 55.3, 278 / 310; 14336 x 4096: 28.3 / 33.8, 32.2 / 33.1, 43.1 / 60.0, 242 / 283; 8192 x 8192 at 512 rows
+// 72.0 / 113.5.  Never slower by more than 2 %, so every 4-bit product of more than 64 rows whose K is a
+// multiple of 128 comes here.  The kernel runs at the power limit of the part (15-20 % faster on all-zero
+// activations); ablations of the main loop at 128 x 8192 x 28672: MFMAs alone 0.58 us per round, loads
+// alone 0.64, together 1.1-1.2.
+bool gemm_tall_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
+    static const char* off = getenv("MH_GEMM_NO_TALL");
+    if (off && *off && atoi(off)) return false;
+    return bits == 4 && epilogue == kEpilogueNone && M >= tall_min_m() && K % kTallRoundK == 0 && K >= 4 * kTallRoundK &&
+           group_size % 32 == 0 && K % group_size == 0 && N % 8 == 0 && (size_t)M * K * 2 < ((size_t)1 << 31) &&
+           (size_t)K * N / 2 < ((size_t)1 << 31);
+}
+
+size_t gemm_tall_workspace_bytes(int M, int N, int K) {
+    const TallPlan p = plan_tall(M, N, K);
+    return p.split_k > 1 ? kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float) : 0;
+}
+
+int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
+                          const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
+                          size_t workspace_bytes, const half_t* bias) {
+    const TallPlan p = plan_tall(M, N, K);
+    const size_t need = gemm_tall_workspace_bytes(M, N, K);
+    if (need != 0 && (workspace == nullptr || workspace_bytes < need))
+        return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    float* partial = need ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes) : nullptr;
+    hipLaunchKernelGGL(gptq_gemm_tall_kernel, dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, stream,
+                       (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
+                       (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block, p.split_k, bias);
+    MH_CHECK_LAUNCH();
+    if (p.split_k > 1) {
+        SmallFuse fuse;
+        fuse.bias = bias;
+        launch_splitk_finalize(stream, partial, out, M, N, p.split_k, kEpilogueNone, fuse);
+        MH_CHECK_LAUNCH();
+    }
+    return MH_OK;
+}
+
+}  // namespace mh

@@ -172,16 +172,24 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     assert_fp16_close(got, ref, what=f"gemm {m}x{k}x{n} b{bits}")
 
 
-# the kernel takes launches of at least 192 tiles of 128 x 128 (three quarters of the CUs)
+# More than 64 rows.  K a multiple of 128: blocks of 128 rows with the weights dequantised in registers
+# (K walked in rounds of 128, a quarter per wave, the four shares added through LDS).  Other K that are
+# multiples of 64, from 192 rows and 192 tiles of 128 x 128: dequantised tiles staged in LDS.
 @pytest.mark.parametrize("m,k,n,group_size", [
-    (384, 256, 8200, 128),     # 3 x 65 tiles, ragged last column tile, unsplit, four waves per workgroup
-    (500, 512, 6144, 64),      # 4 x 48 tiles, ragged last row tile, two groups per 128 k
-    (192, 6144, 12288, 128),   # 2 x 96 tiles, eight waves per workgroup, K split in two (partial sums + second stage)
-    (1000, 512, 3080, 256),    # 8 x 25 tiles, groups longer than a stage
-    (512, 8192, 128, 128),     # too few tiles: stays with the 64-row blocks of the small-M kernel
+    (65, 512, 264, 128),       # one ragged row block, ragged last column tile, four rounds
+    (128, 4096, 1024, 128),    # 8 tiles: K split over workgroups (partial sums + second stage)
+    (200, 1024, 776, 64),      # two row blocks, two groups per round
+    (384, 2048, 520, 256),     # groups longer than a round
+    (130, 1536, 128, 32),      # four groups per round, one column tile
+    (1000, 640, 1032, 128),    # five rounds: the ring of four wraps once
+    (384, 320, 8200, 64),      # K % 128 == 64 -- 3 x 65 tiles, ragged last column tile, unsplit, four waves per workgroup
+    (500, 576, 6144, 64),      # K % 128 == 64 -- 4 x 48 tiles, ragged last row tile
+    (192, 6208, 12288, 64),    # K % 128 == 64 -- 2 x 96 tiles, eight waves per workgroup, K split in two
+    (1000, 576, 3080, 192),    # K % 128 == 64 -- 8 x 25 tiles, groups longer than a stage
+    (512, 8256, 128, 64),      # K % 128 == 64, too few tiles: the 64-row blocks of the small-M kernel
 ])
 def test_gemm_many_rows(hip, m, k, n, group_size):
-    """Several hundred rows: the kernel that stages dequantised fp16 weight tiles in LDS."""
+    """Rows beyond one block of 64: both kernels that dequantise a packed word once for 128 rows."""
     from minit_amd import synthetic
     qweight, qzeros, scales = _weights(k, n, group_size, 4, seed=9)
     x = synthetic.activations("test9", f"x{m}", (m, k))
@@ -264,13 +272,15 @@ def _run_with_bias(hip, x, qweight, qzeros, scales, bias, group_size, bits, g_id
 
 # one case per place where a product kernel stores results: the column-owner kernel, the small-M
 # kernel's direct store, its in-kernel split-K reduction, the split-K second stage, row-blocked
-# launches, the wide kernel with four and with eight waves (direct and split), the 8-bit kernels;
+# launches, the LDS-staged kernel with four and with eight waves (direct and split), the 128-row blocks
+# (split and direct), the 8-bit kernels;
 # then the launches that add the bias in a pass of their own (odd group size, act-order, VALU rows)
 @pytest.mark.parametrize("m,k,n,g,bits,act_order", [
     (1, 1024, 256, 128, 4, False), (1, 4096, 8192, 128, 4, False), (1, 8192, 1024, 128, 4, False),
     (4, 512, 28672, 128, 4, False), (8, 4096, 4096, 128, 4, False), (16, 4096, 1024, 128, 4, False),
-    (32, 2048, 2048, 64, 4, False), (100, 1024, 1536, 128, 4, False), (130, 4096, 512, 128, 4, False),
-    (200, 512, 12288, 128, 4, False), (400, 256, 6144, 64, 4, False), (192, 6144, 12288, 128, 4, False),
+    (32, 2048, 2048, 64, 4, False), (100, 1088, 1536, 64, 4, False), (130, 4160, 512, 64, 4, False),
+    (200, 576, 12288, 64, 4, False), (400, 320, 6144, 64, 4, False), (192, 6208, 12288, 64, 4, False),
+    (128, 4096, 1024, 128, 4, False), (300, 1024, 1032, 128, 4, False),
     (1, 2048, 2048, 128, 8, False), (24, 1024, 768, 64, 8, False), (300, 512, 512, 128, 8, False),
     (3, 768, 264, 96, 4, False), (5, 1024, 512, 512, 4, False), (6, 1024, 256, 128, 4, True),
 ])

@@ -53,7 +53,7 @@ def test_static_scratch_rejects_what_does_not_fit(hip):
     limit = hip.call("mh_gptq_static_scratch_bytes")
     assert limit == 24 << 20
     # a product whose split-K partial sums exceed the built-in buffer (the plan depends on the CU count)
-    shapes = [(128, 28672, 8192), (256, 28672, 8192), (32, 8192, 57344), (96, 14336, 16384)]
+    shapes = [(64, 8192, 57344), (48, 16384, 57344), (128, 28672, 8192), (32, 8192, 57344), (64, 16384, 28672)]
     needs = [hip.call("mh_gptq_workspace_bytes", m, n, k, GROUP, BITS) for m, k, n in shapes]
     assert max(needs) > limit, f"no shape exceeds the built-in buffer: {needs}"
     (m, k, n), need = max(zip(shapes, needs), key=lambda t: t[1])
