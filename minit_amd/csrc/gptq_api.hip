@@ -13,6 +13,7 @@ int gptq_gemv_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
 bool gemm_supported(int M, int N, int K, int group_size, int bits);
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits);
 bool gemm_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
+bool gemm_tall_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
 int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                      const void* scales, void* out, int M, int N, int K, int group_size, int bits,
                      void* workspace, size_t workspace_bytes, int epilogue, const SmallFuse& fuse);
@@ -196,7 +197,8 @@ static size_t silu_pairs_product_offset(size_t product_bytes) {
 
 size_t mh_gptq_silu_pairs_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     const size_t product = mh_gptq_workspace_bytes(M, N, K, group_size, bits);
-    if (gemm_silu_pairs_supported(M, N, K, group_size, bits)) return product;
+    if (gemm_silu_pairs_supported(M, N, K, group_size, bits) || gemm_tall_silu_pairs_supported(M, N, K, group_size, bits))
+        return product;
     return silu_pairs_product_offset(product) + (size_t)M * N * sizeof(half_t);
 }
 
@@ -229,10 +231,11 @@ int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* 
     if (rc) return rc;
     if (M == 0) return MH_OK;
     MH_REQUIRE(N % 256 == 0, "mh_gptq_matmul_silu_pairs: N=%d must be a multiple of 256 (128 gate + 128 up columns per block)", N);
-    if (gemm_silu_pairs_supported(M, N, K, group_size, bits))
+    // up to 64 rows in the small-M kernel's reduction, above in the store of the 128-row blocks when K is unsplit
+    if (gemm_silu_pairs_supported(M, N, K, group_size, bits) || gemm_tall_silu_pairs_supported(M, N, K, group_size, bits))
         return gptq_gemm_launch(as_stream(stream), x, qweight, qzeros, scales, out, M, N, K, group_size, bits,
                                 workspace, workspace_bytes, kEpilogueSiluPairs, SmallFuse{});
-    // more rows (or a group size) than the fused reduction serves: the product into the workspace,
+    // more rows (or a group size) than either serves: the product into the workspace,
     // then one pass that applies silu(gate) * up to the fp16-rounded sums
     const size_t product = silu_pairs_product_offset(mh_gptq_workspace_bytes(M, N, K, group_size, bits));
     const size_t need = product + (size_t)M * N * sizeof(half_t);

@@ -744,9 +744,10 @@ int gptq_gemm_wide_launch(hipStream_t stream, const void* x, const int32_t* qwei
 // gptq_gemm_tall.hip: blocks of 128 rows, weights dequantised in registers, K sliced over the waves
 bool gemm_tall_preferred(int M, int N, int K, int group_size, int bits, int epilogue);
 size_t gemm_tall_workspace_bytes(int M, int N, int K);
+bool gemm_tall_silu_pairs_supported(int M, int N, int K, int group_size, int bits);
 int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                           const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
-                          size_t workspace_bytes, const half_t* bias);
+                          size_t workspace_bytes, const half_t* bias, int epilogue);
 
 struct GemmPlan {
     int mt;  // 16-row tiles per block: 1, 2, 4 or 8
@@ -1006,7 +1007,10 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
     // more than 64 rows: blocks of 128 rows, a packed word dequantised once per block
     if (fuse.ssq_in == nullptr && gemm_tall_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_tall_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,
-                                     workspace_bytes, fuse.bias);
+                                     workspace_bytes, fuse.bias, kEpilogueNone);
+    if (fuse.ssq_in == nullptr && epilogue == kEpilogueSiluPairs && gemm_tall_silu_pairs_supported(M, N, K, group_size, bits))
+        return gptq_gemm_tall_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,
+                                     workspace_bytes, nullptr, kEpilogueSiluPairs);
     // many rows: the kernel that dequantises a weight tile once for 128 rows
     if (fuse.ssq_in == nullptr && gemm_wide_preferred(M, N, K, group_size, bits, epilogue))
         return gptq_gemm_wide_launch(stream, x, qweight, qzeros, scales, out, M, N, K, group_size, workspace,

@@ -31,8 +31,9 @@
 //     = the bit-exact W of Dequantize, 4 to put the pairs back into k order) placed between
 //     them in four pieces.
 // At the end the four waves' shares of K are added through LDS (fixed order), the tile is turned into
-// row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias) or, with
-// K split over blockIdx.y, fp32 partial sums for splitk_finalize_kernel.
+// row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias), with
+// kEpilogueSiluPairs silu(gate) * up of a tile made of 64 gate and the 64 matching up columns, or,
+// with K split over blockIdx.y, fp32 partial sums for splitk_finalize_kernel.
 #include "gptq_common.h"
 
 #include <type_traits>
@@ -84,7 +85,7 @@ __device__ __forceinline__ void tall_wait(uint4_t& q, uint2_t& s, uint32_t& z) {
 __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
-    int group_size, int rounds_per_block, int split_k, const half_t* __restrict__ bias) {
+    int group_size, int rounds_per_block, int split_k, const half_t* __restrict__ bias, int epilogue) {
     __shared__ __attribute__((aligned(1024))) int8_t smem[kTallStages * kTallStageBytes];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -97,7 +98,11 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const int n_rounds = min(rounds_per_block, rounds_total - r_begin);
     // this wave's 32 k of the workgroup's first round
     const int k_wave = r_begin * kTallRoundK + ks * 32;
-    const int col = n0 + cg * 64 + 4 * j;  // first of the lane's four columns
+    // first of the lane's four columns.  kEpilogueSiluPairs (columns in blocks of 128 gate + 128 up): the
+    // tile is 64 gate columns (cg = 0) and the 64 matching up columns (cg = 1) of block blockIdx.x / 2
+    const bool silu = epilogue == kEpilogueSiluPairs;
+    const int pair_col = (blockIdx.x >> 1) * 256 + cg * 128 + (blockIdx.x & 1) * 64;
+    const int col = (silu ? pair_col : n0 + cg * 64) + 4 * j;
 
     const int4_t x_rsrc = tall_rsrc(x, (uint32_t)((size_t)M * K * 2));
     const int4_t w_rsrc = tall_rsrc(qweight, (uint32_t)((size_t)(K / 8) * N * 4));
@@ -287,6 +292,22 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
                 }
         }
         __syncthreads();
+        if (silu) {
+            // out[m, b*128 + h*64 + c] = silu(gate) * up of the fp16-rounded sums, b = blockIdx.x / 2, h = blockIdx.x % 2
+            half_t* dst = out + (blockIdx.x >> 1) * 128 + (blockIdx.x & 1) * 64;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int id = i * kTallThreads + tid, row = id >> 3, ch = id & 7;
+                if (m0 + row >= M) continue;
+                const half8_t g = *reinterpret_cast<const half8_t*>(smem + row * kRow + ch * 16);
+                const half8_t u = *reinterpret_cast<const half8_t*>(smem + row * kRow + 128 + ch * 16);
+                half8_t h;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) h[e] = silu_pair(g[e], u[e]);
+                *reinterpret_cast<half8_t*>(dst + (size_t)(m0 + row) * (N / 2) + ch * 8) = h;
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int id = i * kTallThreads + tid, row = id >> 4, ch = id & 15;
@@ -371,10 +392,17 @@ size_t gemm_tall_workspace_bytes(int M, int N, int K) {
     return p.split_k > 1 ? kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float) : 0;
 }
 
+// kEpilogueSiluPairs in the kernel's own store: an unsplit plan, whole blocks of 128 + 128 columns.
+bool gemm_tall_silu_pairs_supported(int M, int N, int K, int group_size, int bits) {
+    return gemm_tall_preferred(M, N, K, group_size, bits, kEpilogueNone) && N % 256 == 0 && plan_tall(M, N, K).split_k == 1;
+}
+
 int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qweight, const int32_t* qzeros,
                           const void* scales, void* out, int M, int N, int K, int group_size, void* workspace,
-                          size_t workspace_bytes, const half_t* bias) {
+                          size_t workspace_bytes, const half_t* bias, int epilogue) {
     const TallPlan p = plan_tall(M, N, K);
+    if (epilogue != kEpilogueNone && (epilogue != kEpilogueSiluPairs || p.split_k != 1 || N % 256 != 0 || bias))
+        return fail(MH_ERR_INVALID, "gptq gemm (128-row blocks): epilogue %d is not served for M=%d N=%d K=%d", epilogue, M, N, K);
     const size_t need = gemm_tall_workspace_bytes(M, N, K);
     if (need != 0 && (workspace == nullptr || workspace_bytes < need))
         return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
@@ -382,7 +410,7 @@ int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qwei
     float* partial = need ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes) : nullptr;
     hipLaunchKernelGGL(gptq_gemm_tall_kernel, dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, stream,
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
-                       (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block, p.split_k, bias);
+                       (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block, p.split_k, bias, epilogue);
     MH_CHECK_LAUNCH();
     if (p.split_k > 1) {
         SmallFuse fuse;

@@ -351,7 +351,9 @@ def test_operator_api_drop_in(hip):
 
 
 @pytest.mark.parametrize("m,k,ffn", [(1, 512, 256), (3, 1024, 384), (8, 256, 128), (16, 512, 256), (32, 768, 512),
-                                     (40, 512, 256), (130, 1024, 384)])   # above 32 rows: product, then one pass
+                                     (40, 512, 256),     # 33 to 64 rows: product, then one pass
+                                     (130, 1024, 384), (200, 512, 640),   # 128-row blocks, SiLU*up in their store
+                                     (128, 4096, 512)])  # ... K split over workgroups: product, then one pass
 def test_silu_pairs_epilogue(hip, m, k, ffn):
     """gate|up product with SiLU*up applied in the reduction: equals the plain
     product followed by silu(gate) * up on the interleaved column blocks."""
