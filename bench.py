@@ -324,6 +324,9 @@ def main():
                     help="time the vendor library's int8 GEMM (torch._int_mm) on the W8A8 shapes, then exit")
     ap.add_argument("--rowwise-only", action="store_true",
                     help="time only the row-wise kernels (RMSNorm, RoPE, softmax, row sum) and print their lines")
+    ap.add_argument("--small-configs-only", action="store_true",
+                    help="run only config 0 (GEMV 4096x4096), config 1 (Mistral-shape MLP block at 1 to 128 rows) and "
+                         "the lm_head lines, then exit")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the W8A8 GEMM lines (M=2048, K=4096, N in {4096, 11008}), then exit")
     args = ap.parse_args()
@@ -421,6 +424,10 @@ def main():
 
     if args.rowwise_only:
         print(json.dumps({"rowwise_cfg3": bench_rowwise(lib, HIPTensor, memory)}))
+        return
+
+    if args.small_configs_only:
+        print(json.dumps(bench_small_configs(lib, HIPTensor, memory, memory.workspace(64 << 20))))
         return
 
     if args.int8_only:
