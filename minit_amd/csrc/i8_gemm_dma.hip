@@ -101,13 +101,14 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)smem) + (uint32_t)wave * 1024u;
     const int KT = K / BK;
     // part 0: the A rows and one W load, part 1: the other three W loads
-    auto load_stage_part = [&](int part, int stage) {
+    auto load_stage_piece = [&](int j, int stage) {
         const bool live = stage < KT;
-        const int k0 = stage * BK;
         const uint32_t base = lds0 + (uint32_t)(stage % kDmaStages) * kDmaStageBytes;
+        load_to_lds(base + (uint32_t)j * 8192u, voff[j], live ? (j < 2 ? a_rsrc : w_rsrc) : none, stage * BK);
+    };
+    auto load_stage_part = [&](int part, int stage) {
 #pragma unroll
-        for (int j = part * 3; j < part * 3 + 3; ++j)
-            load_to_lds(base + (uint32_t)j * 8192u, voff[j], live ? (j < 2 ? a_rsrc : w_rsrc) : none, k0);
+        for (int j = part * 3; j < part * 3 + 3; ++j) load_stage_piece(j, stage);
     };
 
     auto swz128 = [](int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); };
@@ -147,12 +148,22 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     for (int kt = 0; kt < KT; ++kt) {
         const int nbuf = buf == kDmaStages - 1 ? 0 : buf + 1;
         // quarter 0 (second half of the loads of stage kt + 2)
+        // (one load between two MFMAs: issued back to back by all eight waves the loads fill the vector
+        // memory queue and the waves stall in issue with the matrix pipes idle)
         mfma_one(0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (kt > 0) load_stage_part(1, kt + 2);
+        if (kt > 0) load_stage_piece(3, kt + 2);
         read_frag(1, buf, 1);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_rest(0);
+        mfma_one(0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt > 0) load_stage_piece(4, kt + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(0, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt > 0) load_stage_piece(5, kt + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(0, 3);
         __builtin_amdgcn_sched_barrier(0);
         // quarter 1
         mfma_one(1, 0);
@@ -175,10 +186,18 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
         // quarter 3 (first half of the loads of stage kt + 3 into the buffer just released)
         mfma_one(1, 0);
         __builtin_amdgcn_sched_barrier(0);
-        load_stage_part(0, kt + 3);
+        load_stage_piece(0, kt + 3);
         read_frag(0, nbuf, 0);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_rest(1);
+        mfma_one(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_stage_piece(1, kt + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(1, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        load_stage_piece(2, kt + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(1, 3);
         __builtin_amdgcn_sched_barrier(0);
         buf = nbuf;
     }
