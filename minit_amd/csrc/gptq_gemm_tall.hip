@@ -40,11 +40,19 @@
 
 namespace mh {
 
-constexpr int kTallBM = 128, kTallBN = 128;
+constexpr int kTallBN = 128;
 constexpr int kTallRoundK = 128;                 // four waves x one 32-k step
 constexpr int kTallThreads = 512;
-constexpr int kTallStageBytes = 2 * 128 * 128;   // [half of the round's k][row][64 k], chunks swizzled
 constexpr int kTallStages = 4;
+
+// A compile-time loop: f(integral_constant<int, S>) for S = BEGIN .. END - 1.
+template <int BEGIN, int END, class F>
+__device__ __forceinline__ void tall_static_for(F&& f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        tall_static_for<BEGIN + 1, END>(f);
+    }
+}
 
 void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out, int M, int N, int split_k,
                             int epilogue, const SmallFuse& fuse);
@@ -82,17 +90,27 @@ __device__ __forceinline__ void tall_wait(uint4_t& q, uint2_t& s, uint32_t& z) {
     asm volatile("s_waitcnt vmcnt(%3)" : "+v"(q), "+v"(s), "+v"(z) : "n"(NEWEST) : "memory");
 }
 
+// MT: 16-row MFMA tiles per block of rows (8: blocks of 128 rows; 4: one block of up to 64 rows; 2: up to 32
+// rows, reached only when MH_GEMM_TALL_MIN_M is lowered), the same walk with fewer MFMAs per dequantised word.
+template <int MT>
 __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
     int group_size, int rounds_per_block, int split_k, const half_t* __restrict__ bias, int epilogue) {
-    __shared__ __attribute__((aligned(1024))) int8_t smem[kTallStages * kTallStageBytes];
+    constexpr int BM = 16 * MT;
+    constexpr int kHalfBytes = BM * 128;           // [row][64 k], chunks swizzled
+    constexpr int kStageBytes = 2 * kHalfBytes;    // the two halves of a round's 128 k
+    constexpr int PW = MT / 2;                     // 1 KiB pieces of a stage per wave
+    constexpr int LR = 3 + PW;                     // loads per wave and round
+    constexpr int kRegion = MT * 4096;             // a wave's accumulators in LDS
+    static_assert(MT == 2 || MT == 4 || MT == 8, "two, four or eight row tiles");
+    __shared__ __attribute__((aligned(1024))) int8_t smem[kTallStages * kStageBytes];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cg = wave & 1, ks = wave >> 1;
     const int j = lane & 15, o = lane >> 4;
-    const int n0 = blockIdx.x * kTallBN, m0 = blockIdx.z * kTallBM;
+    const int n0 = blockIdx.x * kTallBN, m0 = blockIdx.z * BM;
     const int rounds_total = K / kTallRoundK;
     const int r_begin = blockIdx.y * rounds_per_block;
     const int n_rounds = min(rounds_per_block, rounds_total - r_begin);
@@ -111,18 +129,18 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const int4_t none = tall_rsrc(x, 0u);  // zero records: no traffic, zeros returned
 
     // ---- what a lane fetches per round
-    // activations: of the stage's 32 pieces of 1 KiB (half h, rows 8p .. 8p+7) this wave loads h = wave / 4,
-    // p = (wave % 4) * 4 + i; lane l lands at row 8p + l / 8, chunk position l % 8, which holds the
+    // activations: of the stage's 4 MT pieces of 1 KiB (half h, rows 8p .. 8p+7) this wave loads h = wave / 4,
+    // p = (wave % 4) * PW + i; lane l lands at row 8p + l / 8, chunk position l % 8, which holds the
     // chunk (l % 8) ^ swizzle(row); rows past M are past the end of the buffer and read as zero
-    int x_off[4];
+    int x_off[PW];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = ((wave & 3) * 4 + i) * 8 + (lane >> 3);
+    for (int i = 0; i < PW; ++i) {
+        const int row = ((wave & 3) * PW + i) * 8 + (lane >> 3);
         const int chunk = (lane & 7) ^ ((row >> 1) & 7);
         x_off[i] = ((m0 + row) * K + r_begin * kTallRoundK + (wave >> 2) * 64 + chunk * 8) * 2;
     }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)smem);
-    const uint32_t lds_wave = lds0 + (uint32_t)((wave >> 2) * 16 + (wave & 3) * 4) * 1024u;
+    const uint32_t lds_wave = lds0 + (uint32_t)(wave >> 2) * kHalfBytes + (uint32_t)((wave & 3) * PW) * 1024u;
     const int w_off = ((k_wave / 8 + o) * N + col) * 4;
     const int s_off = col * 2, z_off = (col >> 3) * 4;
     const int z_shift = (j & 1) * 16;  // the lane's four zero points: nibbles 4 (j & 1) .. + 3 of the word
@@ -134,8 +152,8 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     int load_group = __builtin_amdgcn_readfirstlane(k_wave / group_size);
     int load_in_group = __builtin_amdgcn_readfirstlane(k_wave % group_size);
     int use_in_group = load_in_group;
-    // The seven loads that go with step `step`, in their fixed order: piece 0 the packed words, 1 the scales,
-    // 2 the zero points (all into ring slot S), 3..6 the four 1 KiB pieces of the activation stage of round
+    // The LR loads that go with step `step`, in their fixed order: piece 0 the packed words, 1 the scales,
+    // 2 the zero points (all into ring slot S), 3.. the wave's 1 KiB pieces of the activation stage of round
     // step - 1 (into buffer (step - 1) % 4).  The main loop spreads the pieces over the round's MFMAs: issued
     // back to back by all eight waves right after the barrier they fill the vector memory queue, and the
     // waves stall in issue with the matrix pipes idle.
@@ -155,7 +173,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         }
         if constexpr (I >= 3) {
             const int stage = step - 1;
-            const uint32_t base = lds_wave + (uint32_t)((S + 3) & 3) * kTallStageBytes;
+            const uint32_t base = lds_wave + (uint32_t)((S + 3) & 3) * kStageBytes;
             tall_load_to_lds(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], stage < n_rounds ? x_rsrc : none, stage * 256);
         }
     };
@@ -163,12 +181,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         issue_piece(slot, std::integral_constant<int, 0>{}, step);
         issue_piece(slot, std::integral_constant<int, 1>{}, step);
         issue_piece(slot, std::integral_constant<int, 2>{}, step);
-        if (with_stage) {
-            issue_piece(slot, std::integral_constant<int, 3>{}, step);
-            issue_piece(slot, std::integral_constant<int, 4>{}, step);
-            issue_piece(slot, std::integral_constant<int, 5>{}, step);
-            issue_piece(slot, std::integral_constant<int, 6>{}, step);
-        }
+        if (with_stage) tall_static_for<3, LR>([&](auto piece) { issue_piece(slot, piece, step); });
     };
 
     DequantRegs regs;
@@ -189,9 +202,9 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     // A operand of row tile rt: row rt*16 + j, chunk (ks & 1)*4 + o of the wave's half; the swizzle of
     // row rt*16 + j does not depend on rt
     const int a_off = tall_swz(j, (ks & 1) * 4 + o);
-    float4_t acc[8][4];
+    float4_t acc[MT][4];
 #pragma unroll
-    for (int rt = 0; rt < 8; ++rt)
+    for (int rt = 0; rt < MT; ++rt)
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[rt][c] = float4_t{0.f, 0.f, 0.f, 0.f};
     half8_t b[2][4];
@@ -210,8 +223,8 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     auto round = [&](auto slot, int r) {
         constexpr int S = decltype(slot)::value, P = S & 1, S1 = (S + 1) & 3;
         // done after this wait: everything up to the stage of round r, which includes the words and
-        // constants of step r + 1; still in flight: the 2 x 7 loads of the last two rounds
-        tall_wait<14>(rq[S1], rs[S1], rz[S1]);
+        // constants of step r + 1; still in flight: the 2 x LR loads of the last two rounds
+        tall_wait<2 * LR>(rq[S1], rs[S1], rz[S1]);
         __syncthreads();
         // from here on slot S is free (step r was dequantised last round) and so is the stage buffer of
         // round r - 1: the loads of step r + 4 and stage r + 3 go out between the MFMAs below
@@ -220,27 +233,26 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             do use_in_group -= group_size; while (use_in_group >= group_size);
             make_consts(rs[S1], rz[S1]);
         }
-        const int8_t* stage = smem + S * kTallStageBytes + (ks >> 1) * 16384 + a_off;
-        half8_t a[8];
+        const int8_t* stage = smem + S * kStageBytes + (ks >> 1) * kHalfBytes + a_off;
+        half8_t a[MT];
 #pragma unroll
-        for (int rt = 0; rt < 8; ++rt) a[rt] = *reinterpret_cast<const half8_t*>(stage + rt * 2048);
+        for (int rt = 0; rt < MT; ++rt) a[rt] = *reinterpret_cast<const half8_t*>(stage + rt * 2048);
         __builtin_amdgcn_sched_barrier(0);
+        // 2 MT pairs of MFMAs; after pair s one of the round's loads and / or the dequantisation of one packed
+        // word of step r + 1: every second pair at eight row tiles (a load) and every fourth (a word), every
+        // pair and every second at four, every pair at two
+        tall_static_for<0, 2 * MT>([&](auto pair) {
+            constexpr int s = decltype(pair)::value;
 #pragma unroll
-        for (int rt = 0; rt < 8; ++rt) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                acc[rt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[rt], b[P][c], acc[rt][c], 0, 0, 0);
+            for (int m = 2 * s; m < 2 * s + 2; ++m)
+                acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m >> 2], b[P][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (rt == 0) issue_piece(slot, std::integral_constant<int, 0>{}, r + 4);
-            if (rt == 1) issue_piece(slot, std::integral_constant<int, 1>{}, r + 4);
-            if (rt == 2) issue_piece(slot, std::integral_constant<int, 2>{}, r + 4);
-            if (rt == 3) issue_piece(slot, std::integral_constant<int, 3>{}, r + 4);
-            if (rt == 4) issue_piece(slot, std::integral_constant<int, 4>{}, r + 4);
-            if (rt == 5) issue_piece(slot, std::integral_constant<int, 5>{}, r + 4);
-            if (rt == 6) issue_piece(slot, std::integral_constant<int, 6>{}, r + 4);
-            if (rt & 1) dequant_piece(b[P ^ 1][rt >> 1], rq[S1][rt >> 1], rt >> 1);
+            constexpr int load = MT == 8 ? ((s & 1) ? s >> 1 : -1) : s;
+            if constexpr (load >= 0 && load < LR) issue_piece(slot, std::integral_constant<int, load>{}, r + 4);
+            constexpr int word = MT == 8 ? (s % 4 == 3 ? s / 4 : -1) : MT == 4 ? ((s & 1) ? s >> 1 : -1) : s;
+            if constexpr (word >= 0) dequant_piece(b[P ^ 1][word], rq[S1][word], word);
             __builtin_amdgcn_sched_barrier(0);
-        }
+        });
     };
     for (int r = 0; r < n_rounds; r += 4) {
         round(std::integral_constant<int, 0>{}, r);
@@ -255,18 +267,18 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     __syncthreads();
 
     // ---- the four quarters of K, added in a fixed order: (0 + 1) + (2 + 3)
-    // a wave's accumulators as 32 blocks of 1 KiB, lane-linear on both sides
+    // a wave's accumulators as 4 MT blocks of 1 KiB, lane-linear on both sides
     auto put = [&](int region) {
-        float4_t* dst = reinterpret_cast<float4_t*>(smem + region * 32768) + lane;
+        float4_t* dst = reinterpret_cast<float4_t*>(smem + region * kRegion) + lane;
 #pragma unroll
-        for (int rt = 0; rt < 8; ++rt)
+        for (int rt = 0; rt < MT; ++rt)
 #pragma unroll
             for (int c = 0; c < 4; ++c) dst[(rt * 4 + c) * 64] = acc[rt][c];
     };
     auto add = [&](int region) {
-        const float4_t* src = reinterpret_cast<const float4_t*>(smem + region * 32768) + lane;
+        const float4_t* src = reinterpret_cast<const float4_t*>(smem + region * kRegion) + lane;
 #pragma unroll
-        for (int rt = 0; rt < 8; ++rt)
+        for (int rt = 0; rt < MT; ++rt)
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[rt][c] += src[(rt * 4 + c) * 64];
     };
@@ -284,7 +296,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         constexpr int kRow = 256 + 16;  // bytes per tile row in LDS
         if (ks == 0) {
 #pragma unroll
-            for (int rt = 0; rt < 8; ++rt)
+            for (int rt = 0; rt < MT; ++rt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const half4_t h = {(half_t)acc[rt][0][e], (half_t)acc[rt][1][e], (half_t)acc[rt][2][e], (half_t)acc[rt][3][e]};
@@ -296,9 +308,9 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             // out[m, b*128 + h*64 + c] = silu(gate) * up of the fp16-rounded sums, b = blockIdx.x / 2, h = blockIdx.x % 2
             half_t* dst = out + (blockIdx.x >> 1) * 128 + (blockIdx.x & 1) * 64;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < (MT + 3) / 4; ++i) {
                 const int id = i * kTallThreads + tid, row = id >> 3, ch = id & 7;
-                if (m0 + row >= M) continue;
+                if (row >= BM || m0 + row >= M) continue;
                 const half8_t g = *reinterpret_cast<const half8_t*>(smem + row * kRow + ch * 16);
                 const half8_t u = *reinterpret_cast<const half8_t*>(smem + row * kRow + 128 + ch * 16);
                 half8_t h;
@@ -309,7 +321,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             return;
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < MT / 2; ++i) {
             const int id = i * kTallThreads + tid, row = id >> 4, ch = id & 15;
             const int m = m0 + row, n = n0 + ch * 8;
             if (m >= M || n >= N) continue;
@@ -321,7 +333,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         constexpr int kRow = 512 + 16;
         if (ks == 0) {
 #pragma unroll
-            for (int rt = 0; rt < 8; ++rt)
+            for (int rt = 0; rt < MT; ++rt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float4_t v = {acc[rt][0][e], acc[rt][1][e], acc[rt][2][e], acc[rt][3][e]};
@@ -330,7 +342,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < MT; ++i) {
             const int id = i * kTallThreads + tid, row = id >> 5, ch = id & 31;
             const int m = m0 + row, n = n0 + ch * 4;
             if (m >= M || n >= N) continue;
@@ -343,19 +355,22 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
 // ---- host side ---------------------------------------------------------------------------
 
 struct TallPlan {
-    int tiles_n, row_blocks, split_k, rounds_per_block;
+    int mt, tiles_n, row_blocks, split_k, rounds_per_block;
 };
 
 static TallPlan plan_tall(int M, int N, int K) {
     TallPlan p;
+    p.mt = M <= 32 ? 2 : M <= 64 ? 4 : 8;
+    const int bm = 16 * p.mt;
     p.tiles_n = (N + kTallBN - 1) / kTallBN;
-    p.row_blocks = (M + kTallBM - 1) / kTallBM;
+    p.row_blocks = (M + bm - 1) / bm;
     const int rounds = K / kTallRoundK;
-    // one workgroup per CU (eight waves, 128 KiB of LDS); a workgroup keeps at least four rounds, and
-    // the fp32 partial sums (8 M N bytes per split, written and read) stay below the packed weights' bytes
+    // one workgroup per CU (eight waves; 128 KiB of LDS at eight row tiles); a workgroup keeps at least four
+    // rounds, and the fp32 partial sums (8 M N bytes per split, written and read) stay below the packed
+    // weights' bytes
     long split = (long)compute_units() / ((long)p.tiles_n * p.row_blocks);
     if (split > rounds / 4) split = rounds / 4;
-    const long traffic_cap = (long)K / (16L * (M < kTallBM ? M : kTallBM));
+    const long traffic_cap = (long)K / (16L * (M < bm ? M : bm));
     if (split > traffic_cap) split = traffic_cap;
     if (split < 1) split = 1;
     p.rounds_per_block = (int)((rounds + split - 1) / split);
@@ -366,7 +381,7 @@ static TallPlan plan_tall(int M, int N, int K) {
 static int tall_min_m() {
     static const int v = [] {
         const char* e = getenv("MH_GEMM_TALL_MIN_M");
-        return e && *e ? atoi(e) : 65;
+        return e && *e ? atoi(e) : 33;
     }();
     return v;
 }
@@ -376,7 +391,12 @@ static int tall_min_m() {
 // rows 38.7 / 58.6, 41.2 / 62.3, 75.2 / 80.5, 561 / 567; 4096 x 14336: 29.1 / 33.0, 36.5 / 35.9, 40.1 /
 // 55.3, 278 / 310; 14336 x 4096: 28.3 / 33.8, 32.2 / 33.1, 43.1 / 60.0, 242 / 283; 8192 x 8192 at 512 rows
 // 72.0 / 113.5.  Never slower by more than 2 %, so every 4-bit product of more than 64 rows whose K is a
-// multiple of 128 comes here.  The kernel runs at the power limit of the part (15-20 % faster on all-zero
+// multiple of 128 comes here.  With four row tiles (33 to 64 rows) against the small-M kernel's single block
+// of 64 rows, at 64 rows: 8192 x 10240 29.0 / 41.6, 28672 x 8192 55.7 / 62.3, 4096 x 14336 23.9 / 26.3, 8192 x
+// 57344 109 / 112; with two row tiles at 32 rows it loses (8192 x 57344 77.8 / 67.9, 28672 x 8192 48.6 / 43.5:
+// there the weight stream dominates and the small-M kernel's ring of eight loads per wave hides more
+// latency than this kernel's three rounds), so the switch is at 33 rows (MH_GEMM_TALL_MIN_M moves it).
+// The kernel runs at the power limit of the part (15-20 % faster on all-zero
 // activations); ablations of the main loop at 128 x 8192 x 28672: MFMAs alone 0.58 us per round, loads
 // alone 0.64, together 1.1-1.2.
 bool gemm_tall_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
@@ -408,9 +428,17 @@ int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qwei
         return fail(MH_ERR_WORKSPACE, "mh_gptq_gemm: workspace of %zu bytes required, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
     float* partial = need ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes) : nullptr;
-    hipLaunchKernelGGL(gptq_gemm_tall_kernel, dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, stream,
-                       (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales,
-                       (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block, p.split_k, bias, epilogue);
+#define MH_LAUNCH_TALL(MT)                                                                                            \
+    hipLaunchKernelGGL(gptq_gemm_tall_kernel<MT>, dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, \
+                       stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,                  \
+                       (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block,        \
+                       p.split_k, bias, epilogue)
+    switch (p.mt) {
+        case 2: MH_LAUNCH_TALL(2); break;
+        case 4: MH_LAUNCH_TALL(4); break;
+        default: MH_LAUNCH_TALL(8); break;
+    }
+#undef MH_LAUNCH_TALL
     MH_CHECK_LAUNCH();
     if (p.split_k > 1) {
         SmallFuse fuse;

@@ -52,12 +52,13 @@ def test_static_scratch_rejects_what_does_not_fit(hip):
     from minit_amd.hip.tensor import HIPTensor
     limit = hip.call("mh_gptq_static_scratch_bytes")
     assert limit == 24 << 20
-    # a product whose split-K partial sums exceed the built-in buffer (the plan depends on the CU count)
-    shapes = [(64, 8192, 57344), (48, 16384, 57344), (128, 28672, 8192), (32, 8192, 57344), (64, 16384, 28672)]
-    needs = [hip.call("mh_gptq_workspace_bytes", m, n, k, GROUP, BITS) for m, k, n in shapes]
+    # a product whose split-K partial sums exceed the built-in buffer (the plan depends on the CU count and
+    # on the kernel: 8-bit weights at 64 rows run as one block of 64 rows with K split over workgroups)
+    shapes = [(64, 8192, 57344, 8), (48, 16384, 57344, 8), (64, 8192, 57344, 4), (32, 8192, 57344, 4)]
+    needs = [hip.call("mh_gptq_workspace_bytes", m, n, k, GROUP, bits) for m, k, n, bits in shapes]
     assert max(needs) > limit, f"no shape exceeds the built-in buffer: {needs}"
-    (m, k, n), need = max(zip(shapes, needs), key=lambda t: t[1])
+    (m, k, n, bits), need = max(zip(shapes, needs), key=lambda t: t[1])
     dummy = HIPTensor.allocate((16,), "float16")     # never dereferenced: the size check comes first
     with pytest.raises(hip.HipError, match="scratch"):
         hip.call("mh_gptq_matmul_static", None, dummy.data_ptr, dummy.data_ptr, dummy.data_ptr, dummy.data_ptr, None,
-                 dummy.data_ptr, m, n, k, GROUP, BITS)
+                 dummy.data_ptr, m, n, k, GROUP, bits)
