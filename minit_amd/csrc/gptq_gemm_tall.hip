@@ -43,7 +43,6 @@ namespace mh {
 constexpr int kTallBN = 128;
 constexpr int kTallRoundK = 128;                 // four waves x one 32-k step
 constexpr int kTallThreads = 512;
-constexpr int kTallStages = 4;
 
 // A compile-time loop: f(integral_constant<int, S>) for S = BEGIN .. END - 1.
 template <int BEGIN, int END, class F>
@@ -92,7 +91,11 @@ __device__ __forceinline__ void tall_wait(uint4_t& q, uint2_t& s, uint32_t& z) {
 
 // MT: 16-row MFMA tiles per block of rows (8: blocks of 128 rows; 4: one block of up to 64 rows; 2: up to 32
 // rows, reached only when MH_GEMM_TALL_MIN_M is lowered), the same walk with fewer MFMAs per dequantised word.
-template <int MT>
+// NS: rounds in flight = slots of the register ring = activation stages in LDS.  Four everywhere: eight (the
+// LDS allows them below eight row tiles) measured slower, 32 x 8192 x 57344 90.3 against 77.8 us and 64 x 8192 x
+// 10240 30.3 against 29.0 -- what holds the kernel back at few rows is its ~105 vector instructions per
+// round, not latency.
+template <int MT, int NS>
 __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
@@ -104,7 +107,8 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     constexpr int LR = 3 + PW;                     // loads per wave and round
     constexpr int kRegion = MT * 4096;             // a wave's accumulators in LDS
     static_assert(MT == 2 || MT == 4 || MT == 8, "two, four or eight row tiles");
-    __shared__ __attribute__((aligned(1024))) int8_t smem[kTallStages * kStageBytes];
+    __shared__ __attribute__((aligned(1024))) int8_t smem[NS * kStageBytes];
+    static_assert(NS * kStageBytes >= 4 * kRegion, "the reduction reuses the stages");
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -145,16 +149,16 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const int s_off = col * 2, z_off = (col >> 3) * 4;
     const int z_shift = (j & 1) * 16;  // the lane's four zero points: nibbles 4 (j & 1) .. + 3 of the word
 
-    uint4_t rq[4];   // packed words of steps r .. r + 3
-    uint2_t rs[4];   // their scales
-    uint32_t rz[4];  // their zero-point words
+    uint4_t rq[NS];   // packed words of steps r .. r + NS - 1
+    uint2_t rs[NS];   // their scales
+    uint32_t rz[NS];  // their zero-point words
     // group of the step whose loads are issued next / whose constants are built next
     int load_group = __builtin_amdgcn_readfirstlane(k_wave / group_size);
     int load_in_group = __builtin_amdgcn_readfirstlane(k_wave % group_size);
     int use_in_group = load_in_group;
     // The LR loads that go with step `step`, in their fixed order: piece 0 the packed words, 1 the scales,
     // 2 the zero points (all into ring slot S), 3.. the wave's 1 KiB pieces of the activation stage of round
-    // step - 1 (into buffer (step - 1) % 4).  The main loop spreads the pieces over the round's MFMAs: issued
+    // step - 1 (into buffer (step - 1) % NS).  The main loop spreads the pieces over the round's MFMAs: issued
     // back to back by all eight waves right after the barrier they fill the vector memory queue, and the
     // waves stall in issue with the matrix pipes idle.
     auto issue_piece = [&](auto slot, auto piece, int step) {
@@ -173,7 +177,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         }
         if constexpr (I >= 3) {
             const int stage = step - 1;
-            const uint32_t base = lds_wave + (uint32_t)((S + 3) & 3) * kStageBytes;
+            const uint32_t base = lds_wave + (uint32_t)((S + NS - 1) % NS) * kStageBytes;
             tall_load_to_lds(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], stage < n_rounds ? x_rsrc : none, stage * 256);
         }
     };
@@ -209,25 +213,23 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         for (int c = 0; c < 4; ++c) acc[rt][c] = float4_t{0.f, 0.f, 0.f, 0.f};
     half8_t b[2][4];
 
-    // ---- prologue: the loads of the virtual rounds -4 .. -1, then the operands of step 0
-    issue(std::integral_constant<int, 0>{}, 0, false);
-    issue(std::integral_constant<int, 1>{}, 1, true);
-    issue(std::integral_constant<int, 2>{}, 2, true);
-    issue(std::integral_constant<int, 3>{}, 3, true);
+    // ---- prologue: the loads of the virtual rounds -NS .. -1, then the operands of step 0
+    tall_static_for<0, NS>([&](auto slot) { issue(slot, decltype(slot)::value, decltype(slot)::value != 0); });
     tall_wait<0>(rq[0], rs[0], rz[0]);
     make_consts(rs[0], rz[0]);
 #pragma unroll
     for (int c = 0; c < 4; ++c) dequant_piece(b[0][c], rq[0][c], c);
 
-    // ---- one round: S = r % 4 (ring slot, stage buffer), P = r % 2 (B operand set)
+    // ---- one round: S = r % NS (ring slot, stage buffer), P = r % 2 (B operand set; NS is even)
+    static_assert(NS % 2 == 0, "the B operand sets alternate with the rounds");
     auto round = [&](auto slot, int r) {
-        constexpr int S = decltype(slot)::value, P = S & 1, S1 = (S + 1) & 3;
+        constexpr int S = decltype(slot)::value, P = S & 1, S1 = (S + 1) % NS;
         // done after this wait: everything up to the stage of round r, which includes the words and
-        // constants of step r + 1; still in flight: the 2 x LR loads of the last two rounds
-        tall_wait<2 * LR>(rq[S1], rs[S1], rz[S1]);
+        // constants of step r + 1; still in flight: the LR loads of each of the last NS - 2 rounds
+        tall_wait<(NS - 2) * LR>(rq[S1], rs[S1], rz[S1]);
         __syncthreads();
         // from here on slot S is free (step r was dequantised last round) and so is the stage buffer of
-        // round r - 1: the loads of step r + 4 and stage r + 3 go out between the MFMAs below
+        // round r - 1: the loads of step r + NS and stage r + NS - 1 go out between the MFMAs below
         use_in_group += kTallRoundK;
         if (use_in_group >= group_size) {  // step r + 1 lies in another group than step r
             do use_in_group -= group_size; while (use_in_group >= group_size);
@@ -248,18 +250,16 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
                 acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m >> 2], b[P][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             constexpr int load = MT == 8 ? ((s & 1) ? s >> 1 : -1) : s;
-            if constexpr (load >= 0 && load < LR) issue_piece(slot, std::integral_constant<int, load>{}, r + 4);
+            if constexpr (load >= 0 && load < LR) issue_piece(slot, std::integral_constant<int, load>{}, r + NS);
             constexpr int word = MT == 8 ? (s % 4 == 3 ? s / 4 : -1) : MT == 4 ? ((s & 1) ? s >> 1 : -1) : s;
             if constexpr (word >= 0) dequant_piece(b[P ^ 1][word], rq[S1][word], word);
             __builtin_amdgcn_sched_barrier(0);
         });
     };
-    for (int r = 0; r < n_rounds; r += 4) {
-        round(std::integral_constant<int, 0>{}, r);
-        if (r + 1 < n_rounds) round(std::integral_constant<int, 1>{}, r + 1);
-        if (r + 2 < n_rounds) round(std::integral_constant<int, 2>{}, r + 2);
-        if (r + 3 < n_rounds) round(std::integral_constant<int, 3>{}, r + 3);
-    }
+    for (int r = 0; r < n_rounds; r += NS)
+        tall_static_for<0, NS>([&](auto slot) {
+            if (r + decltype(slot)::value < n_rounds) round(slot, r + decltype(slot)::value);
+        });
 
     // the loads requested past the end are still in flight: their registers are dead to the compiler
     // and their stages would land in LDS that the reduction is about to use
@@ -429,7 +429,7 @@ int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qwei
                     workspace ? workspace_bytes : (size_t)0);
     float* partial = need ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes) : nullptr;
 #define MH_LAUNCH_TALL(MT)                                                                                            \
-    hipLaunchKernelGGL(gptq_gemm_tall_kernel<MT>, dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, \
+    hipLaunchKernelGGL((gptq_gemm_tall_kernel<MT, 4>), dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, \
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,                  \
                        (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block,        \
                        p.split_k, bias, epilogue)
