@@ -191,10 +191,19 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     DequantRegs regs;
     regs.init(4);
     ColumnConst cc[4];
+    // The constants of make_column_const() without conversions, four instructions per column: for a zero
+    // point z <= 15 the fp16 values 1024 + (z + 1) and 64 + (z + 1) are 0x6400 + (z + 1) and 0x5400 +
+    // 16 (z + 1) as bit patterns (one unit, one sixteenth per mantissa step), so both pairs are one
+    // 24-bit multiply-add of z each.
     auto make_consts = [&](const uint2_t& s, uint32_t z) {
-        const half4_t sv = __builtin_bit_cast(half4_t, s);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) cc[c] = make_column_const(sv[c], (z >> (z_shift + 4 * c)) & 0xFu);
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t zc = (z >> (z_shift + 4 * c)) & 0xFu;
+            const uint32_t sw = s[c >> 1];
+            cc[c].scale = as_half2((c & 1) ? __builtin_amdgcn_perm(sw, sw, 0x07060706u) : __builtin_amdgcn_perm(sw, sw, 0x05040504u));
+            cc[c].zero_lo = as_half2(zc * 0x00010001u + 0x64016401u);
+            cc[c].zero_hi = as_half2(zc * 0x00100010u + 0x54105410u);
+        }
     };
     // one packed word -> the B operand of MFMA tile c: k0 .. k7 of column 4j + c
     auto dequant_piece = [&](half8_t& b, uint32_t word, int c) {
