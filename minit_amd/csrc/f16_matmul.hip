@@ -223,6 +223,12 @@ int f16_gemv_prepare() {
 
 }  // namespace mh
 
+namespace mh {
+// f16_matmul_lds.hip
+bool f16_matmul_lds_supported(int M, int N, int K);
+int f16_matmul_lds_launch(hipStream_t stream, const void* a, const void* b, void* out, int M, int N, int K);
+}  // namespace mh
+
 using namespace mh;
 
 extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out, int M, int N,
@@ -267,6 +273,8 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
         MH_CHECK_LAUNCH();
         return MH_OK;
     }
+    // more rows against a long weight: the weight streamed through LDS in whole lines
+    if (f16_matmul_lds_supported(M, N, K)) return f16_matmul_lds_launch(st, a, b, out, M, N, K);
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     const int nt = mt == 1 ? 1 : 2;  // columns per wave: 16 or 32
     dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt));

@@ -194,7 +194,11 @@ def test_sigmoid_multiply_compose_to_silu(hip):
                                    # one to four rows and a tall weight: the dot-product kernel (row groups of
                                    # four, ragged last group, waves with one group more than others)
                                    (1, 128256, 1024), (2, 8193, 2048), (3, 9001, 1024), (4, 8192, 8192), (8, 8200, 8192), (5, 16390, 1024),
-                                   (1, 8190, 4096)])
+                                   (1, 8190, 4096),
+                                   # more than eight rows and a tall weight: the weight streamed through LDS (ragged
+                                   # last tile, seven rounds for six stages; exactly six rounds, four row tiles; two
+                                   # blocks of 64 rows, the second ragged)
+                                   (9, 16390, 448), (33, 16384, 384), (64, 20000, 1024), (70, 16400, 512), (32, 32768, 2048)])
 def test_dense_matmul_nk(hip, m, n, k):
     import minit_amd.functional as F
     rng = np.random.default_rng(10)
