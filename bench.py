@@ -314,6 +314,9 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
+    ap.add_argument("--calibrate-barrier", action="store_true",
+                    help="time a device-wide barrier (agent-scope counter, bounded polls) of one and two workgroups "
+                         "per CU against a boundary between two dependent launches, then exit")
     ap.add_argument("--calibrate-issue", action="store_true",
                     help="run only the register-resident vector + MFMA instruction mix at 1, 2 and 4 waves per "
                          "SIMD (do vector and matrix instructions of one SIMD's waves overlap?), then exit")
@@ -391,6 +394,47 @@ def main():
             res.append({"operands": label, "ms": round(ms, 2), "tops": round(tops, 1),
                         "frac_of_datasheet": round(tops / INT8_PEAK_TOPS, 4)})
         print(json.dumps({"kernel": "i8_mfma_probe_kernel", "waves_per_simd": 2, "results": res}))
+        return
+
+    if args.calibrate_barrier:
+        cus = info["compute_units"]
+        words = HIPTensor.allocate((32 * 18,), "int32")   # counters on lines of their own, error word last
+        err_ptr = words.data_ptr + 32 * 17 * 4
+        rows = []
+        for per_cu in (1, 2):
+            for groups in (1, 8):
+                blocks, rounds = cus * per_cu, 2000
+                words.memory.reset()
+                lib.call("mh_grid_barrier_probe", None, words.data_ptr, err_ptr, blocks, 10, 1 << 16, groups)
+                memory.synchronize()
+                words.memory.reset()
+                memory.synchronize()
+                e0, e1 = memory.Event(), memory.Event()
+                e0.record()
+                lib.call("mh_grid_barrier_probe", None, words.data_ptr, err_ptr, blocks, rounds, 1 << 16, groups)
+                e1.record()
+                e1.synchronize()
+                gave_up = int(words.numpy()[32 * 17])
+                ns = e0.elapsed_ms(e1) * 1e6 / rounds
+                rows.append({"workgroups": blocks, "arrival_groups": groups, "rounds": rounds,
+                             "ns_per_barrier": round(ns, 1), "gave_up": gave_up})
+                log(f"device-wide barrier, {blocks} workgroups, {groups} arrival group(s): {ns:.0f} ns per round "
+                    f"(gave up: {gave_up})")
+        launches = 2000
+        for blocks in (cus, 2 * cus):
+            for i in range(20):
+                lib.call("mh_empty_probe", None, None, blocks)
+            memory.synchronize()
+            e0, e1 = memory.Event(), memory.Event()
+            e0.record()
+            for i in range(launches):
+                lib.call("mh_empty_probe", None, None, blocks)
+            e1.record()
+            e1.synchronize()
+            ns = e0.elapsed_ms(e1) * 1e6 / launches
+            rows.append({"workgroups": blocks, "launches": launches, "ns_per_empty_launch": round(ns, 1)})
+            log(f"empty launch of {blocks} workgroups, back to back in one stream: {ns:.0f} ns per launch")
+        print(json.dumps({"kernel": "grid_barrier_probe_kernel", "results": rows}))
         return
 
     if args.calibrate_issue:

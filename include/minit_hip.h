@@ -208,6 +208,17 @@ int mh_i8_mfma_probe(mh_stream_t stream, const int8_t* operands, int32_t* out, i
  * whether vector and matrix instructions of the waves of one SIMD overlap. */
 int mh_issue_probe(mh_stream_t stream, float* out, int blocks, int iters, int n_valu, int n_mfma,
                    int dependent);
+/* Calibration, no counterpart in the reference: `blocks` workgroups of 256 threads meet `rounds`
+ * times at a device-wide barrier (agent-scope counters that only grow: counter[0] and, with groups > 1,
+ * one per group at counter[32 * (1 + g)], 32 * 17 words zeroed by the caller; every wait gives up
+ * after spin_limit polls and sets *error, after which no workgroup waits any more, so every wave
+ * exits).  groups = 1: every workgroup arrives at counter[0]; groups = 8: per-XCD arrival, then one
+ * arrival per group.  blocks must not exceed two per CU.  Used by bench.py
+ * --calibrate-barrier to price a phase barrier of a persistent kernel against a kernel boundary
+ * (mh_empty_probe: an empty launch of `blocks` workgroups). */
+int mh_grid_barrier_probe(mh_stream_t stream, unsigned* counter, unsigned* error, int blocks, int rounds,
+                          int spin_limit, int groups);
+int mh_empty_probe(mh_stream_t stream, unsigned* sink, int blocks);
 /* out[n, k] = in[k, n]: one-time layout conversion for weights stored [K, N]. */
 int mh_i8_transpose(mh_stream_t stream, const int8_t* in, int8_t* out, int rows, int cols);
 

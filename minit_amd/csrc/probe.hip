@@ -43,9 +43,77 @@ __global__ void __launch_bounds__(256) issue_probe_kernel(float* __restrict__ ou
     out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// Cost of a device-wide barrier between the phases of a would-be persistent kernel, against the cost
+// of a kernel boundary: every workgroup bumps one agent-scope counter and polls it until all have
+// arrived, `rounds` times.  The counter only grows (round r waits for (r + 1) * workgroups), so no
+// reset races with a late reader.  Every wait is bounded: after spin_limit polls a workgroup sets
+// the error word and, like every workgroup that sees it set, stops waiting for the rest of the
+// launch, so all waves exit whether or not the workgroups were resident together.
+// groups > 1: two levels.  Workgroup b arrives at counter[32 * (1 + b % groups)] (a line of its own per
+// group; consecutive workgroups go to different XCDs, so a group is the workgroups of one XCD when
+// groups is 8), and the one that completes its group's round bumps counter[0], which everybody polls:
+// the arrivals at one address, which serialise, drop from all workgroups to the group size plus groups.
+__global__ void __launch_bounds__(256) grid_barrier_probe_kernel(unsigned* __restrict__ counter,
+                                                                 unsigned* __restrict__ error, int rounds,
+                                                                 int spin_limit, int groups) {
+    __shared__ int give_up;
+    if (threadIdx.x == 0) give_up = 0;
+    __syncthreads();
+    const unsigned group = blockIdx.x % groups;
+    const unsigned group_size = gridDim.x / groups + (group < gridDim.x % groups ? 1u : 0u);
+    for (int r = 0; r < rounds; ++r) {
+        if (threadIdx.x == 0 && !give_up) {
+            if (groups > 1) {
+                const unsigned prev = __hip_atomic_fetch_add(counter + 32 * (1 + group), 1u, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT);
+                if (prev + 1 == (unsigned)(r + 1) * group_size)
+                    __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            const unsigned target = (unsigned)(r + 1) * (groups > 1 ? (unsigned)groups : gridDim.x);
+            int spins = 0;
+            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+                if (++spins > spin_limit || __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+                    __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    give_up = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__global__ void __launch_bounds__(256) empty_probe_kernel(unsigned* __restrict__ sink) {
+    if (sink == nullptr) return;
+    if (threadIdx.x == 0 && blockIdx.x == 0x7fffffffu) *sink = 1u;  // never true: keeps the argument alive
+}
+
 }  // namespace mh
 
 using namespace mh;
+
+extern "C" int mh_grid_barrier_probe(mh_stream_t stream, unsigned* counter, unsigned* error, int blocks, int rounds,
+                                     int spin_limit, int groups) {
+    MH_REQUIRE(counter != nullptr && error != nullptr && blocks > 0 && rounds > 0 && spin_limit > 0 && groups >= 1 &&
+                   groups <= 16 && groups <= blocks,
+               "mh_grid_barrier_probe: bad argument");
+    MH_REQUIRE(blocks <= compute_units() * 2, "mh_grid_barrier_probe: %d workgroups cannot be resident together on %d CUs",
+               blocks, compute_units());
+    MH_REQUIRE((long)blocks * rounds < (1L << 31), "mh_grid_barrier_probe: counter would overflow");
+    grid_barrier_probe_kernel<<<blocks, 256, 0, as_stream(stream)>>>(counter, error, rounds, spin_limit, groups);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+extern "C" int mh_empty_probe(mh_stream_t stream, unsigned* sink, int blocks) {
+    MH_REQUIRE(blocks > 0, "mh_empty_probe: bad argument");
+    empty_probe_kernel<<<blocks, 256, 0, as_stream(stream)>>>(sink);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
 
 extern "C" int mh_issue_probe(mh_stream_t stream, float* out, int blocks, int iters, int n_valu, int n_mfma,
                               int dependent) {

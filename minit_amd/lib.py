@@ -58,6 +58,8 @@ PROTOTYPES = {
     "mh_i8_transpose": (c_int, [_P, _P, _P, c_int, c_int]),
     "mh_i8_mfma_probe": (c_int, [_P, _P, _P, c_int, c_int]),
     "mh_issue_probe": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mh_grid_barrier_probe": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int]),
+    "mh_empty_probe": (c_int, [_P, _P, c_int]),
     "mh_rms_norm": (c_int, [_P, _P, _P, _P, c_size_t, c_size_t, c_size_t, c_double, c_int]),
     "mh_rope": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_softmax": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
