@@ -387,6 +387,18 @@ def test_silu_pairs_epilogue(hip, m, k, ffn):
     assert (np.abs(got.astype(np.float64) - ref) <= 1.0 * ulp + slack + 1e-7).all()
     # and the product itself is the oracle's
     assert_fp16_close(y.reshape(m, 2 * ffn), O.matmul_f64(x, qweight, qzeros, scales, None, 4, g), what="gate|up")
+    # one-hot activations: the sums are rows of the dequantised matrix whatever the summation order, so the
+    # epilogue must return silu(W[k, gate(j)]) * W[k, up(j)] to one fp16 step -- no slack for a wrong pairing
+    rows = np.random.default_rng(m).integers(0, k, m)
+    onehot = np.zeros((m, k), dtype=np.float16)
+    onehot[np.arange(m), rows] = 1.0
+    dh = _dev(hip, onehot)
+    hip.call("mh_gptq_matmul_silu_pairs", None, dh.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, out.data_ptr,
+             m, 2 * ffn, k, g, 4, ws._pointer, ws._size)
+    w = O.dequantize_packed(qweight, qzeros, scales, None, 4, g)[rows].reshape(m, ffn // 128, 2, 128)
+    ref = O.silu_mul_f64(w[:, :, 0], w[:, :, 1]).reshape(m, ffn)
+    ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64)
+    assert (np.abs(out.numpy().astype(np.float64) - ref) <= ulp + 1e-9).all()
 
 
 def _random_cases(count, seed):
