@@ -117,22 +117,30 @@ def bench_int8(lib, HIPTensor, memory, n, iters=20):
     def go(i):
         lib.call("mh_i8_gemm", None, a.data_ptr, ws[i % 4].data_ptr, sa.data_ptr, sw.data_ptr, out.data_ptr,
                  None, m, n, k)
-    for i in range(3):
-        go(i)
-    memory.synchronize()
-    e0, e1 = memory.Event(), memory.Event()
-    e0.record()
-    for i in range(iters):
-        go(i)
-    e1.record()
-    e1.synchronize()
-    us = e0.elapsed_ms(e1) * 1e3 / iters
+    us = _time_launches(memory, go, iters=iters, warmup=4)
     tops = 2.0 * m * n * k / us / 1e6
     return {"M": m, "N": n, "K": k, "us": round(us, 2), "tops": round(tops, 1),
             "frac_of_peak": round(tops / INT8_PEAK_TOPS, 4)}
 
 
+def _settle(memory, fn, ms):
+    """Runs fn(0), fn(1), ... for at least `ms` milliseconds, untimed: the part needs some tens of
+    milliseconds of load to reach its steady clocks (the headline step measures 99.7 us when timed
+    right after 20 warm-up steps and 92.1-92.7 us after 0.3 s of the same work)."""
+    t0, i = time.perf_counter(), 0
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(16):
+            fn(i)
+            i += 1
+        memory.synchronize()
+    return i
+
+
+SETTLE_MS = 150.0   # untimed load before every timed section (--settle-ms)
+
+
 def _time_launches(memory, fn, iters=200, warmup=10):
+    _settle(memory, fn, SETTLE_MS)
     for i in range(warmup):
         fn(i)
     memory.synchronize()
@@ -299,8 +307,8 @@ def bench_int8_library(n, iters=50):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--layers", type=int, default=6, help="distinct weight sets cycled through")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
@@ -314,9 +322,15 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
     ap.add_argument("--calibrate-mfma", action="store_true",
                     help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed load (the step itself) before the warm-up steps, so that the timed steps run at the "
+                         "part's steady clocks; half of it before every timed section of the extras; 0 switches it off")
     ap.add_argument("--calibrate-barrier", action="store_true",
                     help="time a device-wide barrier (agent-scope counter, bounded polls) of one and two workgroups "
                          "per CU against a boundary between two dependent launches, then exit")
+    ap.add_argument("--calibrate-stream", action="store_true",
+                    help="read the packed words of gate|up (8192 x 57344, six sets) with the small-M kernel's load "
+                         "footprint and no arithmetic, and the same shape at other K, then exit")
     ap.add_argument("--calibrate-issue", action="store_true",
                     help="run only the register-resident vector + MFMA instruction mix at 1, 2 and 4 waves per "
                          "SIMD (do vector and matrix instructions of one SIMD's waves overlap?), then exit")
@@ -337,6 +351,8 @@ def main():
         print(json.dumps({"int8_gemm_vendor_library": [bench_int8_library(n) for n in (4096, 11008)]}))
         return
     ENTRY = args.entry
+    global SETTLE_MS
+    SETTLE_MS = args.settle_ms / 2
     if args.gpus != 1:
         log(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
             "(no collectives or sharding in this path).")
@@ -437,6 +453,24 @@ def main():
         print(json.dumps({"kernel": "grid_barrier_probe_kernel", "results": rows}))
         return
 
+    if args.calibrate_stream:
+        n, sets = 57344, 6
+        rows_max = 2048
+        words = [HIPTensor.allocate((rows_max, n), "int32") for _ in range(sets)]
+        for i, w in enumerate(words):
+            lib.call("mh_synth_u32", None, w.data_ptr, rows_max * n, 77 + i)
+        sink = HIPTensor.allocate((256,), "int32")
+        rows_out = []
+        for k, parts in ((8192, 2), (8192, 4), (16384, 2)):
+            rows = k // 8
+            us = _time_launches(memory, lambda i: lib.call("mh_weight_stream_probe", None, words[i % sets].data_ptr,
+                                                           sink.data_ptr, rows, n, parts), iters=120, warmup=12)
+            nbytes = rows * n * 4
+            rows_out.append({"K": k, "N": n, "parts": parts, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1)})
+            log(f"weight stream {k}x{n}, {parts} K parts: {us:.1f} us, {nbytes / us / 1e3:.0f} GB/s")
+        print(json.dumps({"kernel": "weight_stream_probe_kernel", "results": rows_out}))
+        return
+
     if args.calibrate_issue:
         cus = info["compute_units"]
         iters = 20000
@@ -499,6 +533,9 @@ def main():
         for lin in layers[i % args.layers]:
             run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
 
+    if args.settle_ms > 0:
+        settled = _settle(memory, step, args.settle_ms)
+        log(f"settled the clocks with {settled} untimed steps ({args.settle_ms:.0f} ms)")
     for i in range(args.warmup):
         step(i)
     memory.synchronize()
@@ -519,12 +556,31 @@ def main():
     log(f"{args.steps} steps: {dev_ms:.2f} ms on device ({wall * 1e3:.2f} ms wall), "
         f"{ms_per_step * 1e3:.1f} us/step, {gbps:.0f} GB/s")
 
-    # ---- the dominant kernel (gate|up: 55 % of the step's bytes), timed launch by launch with an
-    # event pair around it inside a second pass over the same steps, same launch sequence
+    # ---- the dominant kernel (gate|up: 55 % of the step's bytes): its average launch duration inside the
+    # layer sequence = what the same K steps lose when that launch is left out (HIP events around both
+    # passes).  An event pair around every launch, also reported, brackets the launch with two more
+    # packets on the stream and reads 2-3 us more than the kernel trace of the same command; the
+    # difference of the two passes agrees with it.
     dom = max(range(len(LINEARS)), key=lambda j: linear_bytes(1, LINEARS[j][1], LINEARS[j][2]))
     dom_name, dom_k, dom_n = LINEARS[dom]
-    pairs = [(memory.Event(), memory.Event()) for _ in range(args.steps)]
+
+    def step_without(i):
+        for j, lin in enumerate(layers[i % args.layers]):
+            if j != dom:
+                run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
+
+    for i in range(max(args.warmup, 20)):
+        step_without(i)
+    memory.synchronize()
+    s0, s1 = memory.Event(), memory.Event()
+    s0.record()
     for i in range(args.steps):
+        step_without(i)
+    s1.record()
+    s1.synchronize()
+    dom_us = (dev_ms - s0.elapsed_ms(s1)) * 1e3 / args.steps
+    pairs = [(memory.Event(), memory.Event()) for _ in range(min(args.steps, 400))]
+    for i in range(len(pairs)):
         for j, lin in enumerate(layers[i % args.layers]):
             if j == dom:
                 pairs[i][0].record()
@@ -532,11 +588,12 @@ def main():
             if j == dom:
                 pairs[i][1].record()
     memory.synchronize()
-    dom_us = float(np.mean([a.elapsed_ms(b) for a, b in pairs])) * 1e3
+    dom_pair_us = float(np.mean([a.elapsed_ms(b) for a, b in pairs])) * 1e3
     dom_bytes = linear_bytes(1, dom_k, dom_n)
     dom_gbps = dom_bytes / dom_us / 1e3
     traffic, traffic_commit = measured_traffic(ENTRY)
-    log(f"dominant kernel ({dom_name} {dom_k}x{dom_n}): {dom_us:.2f} us per launch in the layer sequence, {dom_gbps:.0f} GB/s")
+    log(f"dominant kernel ({dom_name} {dom_k}x{dom_n}): {dom_us:.2f} us per launch in the layer sequence "
+        f"({dom_pair_us:.2f} us between an event pair per launch), {dom_gbps:.0f} GB/s")
 
     result = {
         "metric": "w4a16_gemv_hbm_gbps",
@@ -556,6 +613,7 @@ def main():
                         "o 8192x8192, gate_up 8192x57344, down 28672x8192; one step = one layer",
             "layers_cycled": args.layers,
             "bytes_per_step": step_bytes,
+            "settle_ms": args.settle_ms,
             "device": info["name"].strip(),
         },
         "roofline": {
@@ -568,6 +626,7 @@ def main():
             "unit": "GB/s",
             "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
             "avg_launch_us": round(dom_us, 3),
+            "avg_launch_us_event_pair_per_launch": round(dom_pair_us, 3),
             "bytes_per_launch": dom_bytes,
             "traffic": traffic,
             "traffic_measured_at_commit": traffic_commit,

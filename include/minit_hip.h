@@ -219,6 +219,12 @@ int mh_issue_probe(mh_stream_t stream, float* out, int blocks, int iters, int n_
 int mh_grid_barrier_probe(mh_stream_t stream, unsigned* counter, unsigned* error, int blocks, int rounds,
                           int spin_limit, int groups);
 int mh_empty_probe(mh_stream_t stream, unsigned* sink, int blocks);
+/* Calibration, no counterpart in the reference: reads `rows` packed rows of N 32-bit words with the
+ * footprint of the small-M GPTQ kernel's weight stream (N / 256 x parts workgroups of four waves, a wave
+ * load = four rows x 256 bytes, eight loads in flight per wave) and does nothing with them.  sink: 256
+ * words, never written in practice.  Used by bench.py --calibrate-stream: the rate the memory system
+ * delivers to that footprint. */
+int mh_weight_stream_probe(mh_stream_t stream, const uint32_t* words, uint32_t* sink, int rows, int N, int parts);
 /* out[n, k] = in[k, n]: one-time layout conversion for weights stored [K, N]. */
 int mh_i8_transpose(mh_stream_t stream, const int8_t* in, int8_t* out, int rows, int cols);
 

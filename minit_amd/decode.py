@@ -278,7 +278,7 @@ def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=pr
     for b in batches:
         toks = np.arange(b, dtype=np.int32) * 17 + 5
         pos = np.full(b, context, np.int32)
-        dec.decode(toks, pos, 2, graph=graph)          # warm-up (and the recording of the step)
+        dec.decode(toks, pos, 12, graph=graph)         # warm-up: the recording of the step, and the part's clocks
         memory.synchronize()
         # host clock around a call that ends in a device synchronisation: the graph
         # variant runs on the decoder's own stream, where null-stream events do not see it

@@ -60,6 +60,7 @@ PROTOTYPES = {
     "mh_issue_probe": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int]),
     "mh_grid_barrier_probe": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int]),
     "mh_empty_probe": (c_int, [_P, _P, c_int]),
+    "mh_weight_stream_probe": (c_int, [_P, _P, _P, c_int, c_int, c_int]),
     "mh_rms_norm": (c_int, [_P, _P, _P, _P, c_size_t, c_size_t, c_size_t, c_double, c_int]),
     "mh_rope": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_softmax": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),
