@@ -44,7 +44,7 @@ __device__ __forceinline__ int4_t lds_rsrc(const void* base, uint32_t bytes) {
 // 16 bytes per lane, global -> LDS at m0 + lane * 16; out-of-range records write zeros.
 __device__ __forceinline__ void lds_load(uint32_t lds_addr, int voffset, const int4_t& rsrc, int soffset) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
 
 // MT: 16-row tiles of activations per workgroup (2: up to 32 rows, 4: up to 64).

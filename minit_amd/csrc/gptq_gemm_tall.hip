@@ -80,7 +80,7 @@ __device__ __forceinline__ void tall_load_b32(uint32_t& dst, int voffset, const 
 // 16 bytes per lane, global -> LDS at m0 + lane * 16.
 __device__ __forceinline__ void tall_load_to_lds(uint32_t lds_addr, int voffset, const int4_t& rsrc, int soffset) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
 // Everything but the newest NEWEST loads has arrived; the registers read next pass through the
 // wait, so that no use can be scheduled above it.

@@ -31,7 +31,7 @@ constexpr int kDmaStagePitch = 144;                         // epilogue: 64 fp16
 // soffset: the scalar (k) offset; out-of-range records read as zero.
 __device__ __forceinline__ void load_to_lds(uint32_t lds_addr, int voffset, const int4_t& rsrc, int soffset) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
 
 __device__ __forceinline__ int4_t make_rsrc(const void* base, uint32_t bytes) {
