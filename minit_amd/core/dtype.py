@@ -1,21 +1,20 @@
-"""dtype registry; names and sizes as in the reference (minit/core/dtype.py:36-49)."""
-from typing import Dict, Optional
+"""dtype registry: the reference's names with their python type and size
+(minit/core/dtype.py:36-49)."""
+from typing import Dict, NamedTuple, Optional
 
 
-class DataTypeInfo:
-    __slots__ = ["name", "python_type", "size_in_bytes"]
-
-    def __init__(self, name: str, python_type: Optional[type], size_in_bytes: int) -> None:
-        self.name = name
-        self.python_type = python_type
-        self.size_in_bytes = size_in_bytes
+class DataTypeInfo(NamedTuple):
+    name: str
+    python_type: Optional[type]
+    size_in_bytes: int
 
 
 DATA_TYPES: Dict[str, DataTypeInfo] = {}
 
 
-def register_dtype(name: str, python_type: Optional[type], size_in_bytes: int):
-    assert name not in DATA_TYPES
+def register_dtype(name: str, python_type: Optional[type], size_in_bytes: int) -> None:
+    if name in DATA_TYPES:
+        raise AssertionError(f"dtype {name} is registered already")
     DATA_TYPES[name] = DataTypeInfo(name, python_type, size_in_bytes)
 
 
@@ -23,9 +22,14 @@ def dtype_info(name: str) -> DataTypeInfo:
     return DATA_TYPES[name]
 
 
-for _name, _py, _size in [
-    ("float64", float, 8), ("float32", float, 4), ("float16", float, 2), ("bfloat16", float, 2),
-    ("int64", int, 8), ("int32", int, 4), ("int16", int, 2), ("int8", int, 1),
-    ("uint64", int, 8), ("uint32", int, 4), ("uint16", int, 2), ("uint8", int, 1),
-]:
-    register_dtype(_name, _py, _size)
+def _register_builtin() -> None:
+    # floating types by bit width (bfloat16 shares float16's size), then the integers of 8 to 64 bits
+    for bits in (64, 32, 16):
+        register_dtype(f"float{bits}", float, bits // 8)
+    register_dtype("bfloat16", float, 2)
+    for prefix in ("int", "uint"):
+        for bits in (64, 32, 16, 8):
+            register_dtype(f"{prefix}{bits}", int, bits // 8)
+
+
+_register_builtin()

@@ -1,7 +1,7 @@
-"""``rms_norm`` / ``rope`` / ``softmax`` / ``sigmoid`` entry points with the
-reference's signatures and argument checks (minit/functional/special.py:6-26).
-``rope`` and ``softmax`` take optional keyword extensions (per-row positions; a
-fused causal mask); the reference forms are the defaults."""
+"""``rms_norm`` / ``rope`` / ``softmax`` / ``sigmoid``: the functional face of the
+operators in ``minit_amd.operator`` with the reference's names, argument order and
+argument checks (minit/functional/special.py:6-26).  ``rope`` takes an optional fourth
+tensor (per-row positions); without it the call is the reference's."""
 from typing import Optional
 
 from ..core.dispatch import dispatch
@@ -9,27 +9,26 @@ from ..core.tensor import Tensor
 from ..operator import RMSNorm, RoPE, Sigmoid, Softmax
 
 
-def sigmoid(x: Tensor):
-    (z,) = dispatch(Sigmoid(), x)
-    return z
+def _single(outputs):
+    """Every rule returns a tuple; these operators have one result."""
+    assert len(outputs) == 1, f"expected one output, got {len(outputs)}"
+    return outputs[0]
+
+
+def sigmoid(x: Tensor) -> Tensor:
+    return _single(dispatch(Sigmoid(), x))
 
 
 def rms_norm(x: Tensor, weight: Tensor, axis: int, eps: float) -> Tensor:
-    assert isinstance(eps, float)
-    assert eps > 0
-    assert eps < 0.5
-    (z,) = dispatch(RMSNorm(axis=axis, eps=eps), x, weight)
-    return z
+    # the reference insists on a python float in (0, 0.5): an int or an array here is a slipped argument
+    assert isinstance(eps, float) and 0.0 < eps < 0.5, f"eps must be a float in (0, 0.5), got {eps!r}"
+    return _single(dispatch(RMSNorm(axis=axis, eps=eps), x, weight))
 
 
 def rope(x: Tensor, freqs_cos: Tensor, freqs_sin: Tensor, positions: Optional[Tensor] = None) -> Tensor:
-    if positions is None:
-        (z,) = dispatch(RoPE(), x, freqs_cos, freqs_sin)
-    else:
-        (z,) = dispatch(RoPE(), x, freqs_cos, freqs_sin, positions)
-    return z
+    operands = (x, freqs_cos, freqs_sin) if positions is None else (x, freqs_cos, freqs_sin, positions)
+    return _single(dispatch(RoPE(), *operands))
 
 
 def softmax(x: Tensor, axis: int) -> Tensor:
-    (z,) = dispatch(Softmax(axis=axis), x)
-    return z
+    return _single(dispatch(Softmax(axis=axis), x))
