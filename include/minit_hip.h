@@ -71,6 +71,12 @@ int mh_copy_kernel(mh_stream_t stream, const void* src, void* dst, size_t bytes)
  * (4 or 8).  packed is int32 [rows, cols]; out is uint8
  * [rows * (32/bits), cols] for axis 0, [rows, cols * (32/bits)] for axis 1.
  */
+/* out row j = qweight row perm[j] of the K unpacked rows, both packed along K ([K/P, N] int32):
+ * the one-time repack of an act-order checkpoint whose rows are sorted by group
+ * (examples/qwen1_5_int8.py:283-285 keeps g_idx and gathers per element at every product instead).
+ * perm int32 [K] holds every row once (not checked on the device); not in place. */
+int mh_gptq_permute_rows(mh_stream_t stream, const int32_t* qweight, const int32_t* perm, int32_t* out, int N,
+                         int K, int bits);
 int mh_gptq_unpack(mh_stream_t stream, const int32_t* packed, uint8_t* out,
                    size_t rows, size_t cols, int axis, int bits);
 

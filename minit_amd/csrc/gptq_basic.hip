@@ -121,11 +121,51 @@ int gptq_generic_launch(hipStream_t stream, const void* x, const int32_t* qweigh
     return MH_OK;
 }
 
+// Rows of a packed weight in another order: out row j = in row perm[j], sub-word by sub-word
+// (the one-time repack of an act-order checkpoint, rows sorted by group, so that the kernels
+// that read sequential groups serve it).  One thread per output word.
+template <int BITS>
+__global__ void permute_rows_kernel(const uint32_t* __restrict__ packed, const int32_t* __restrict__ perm,
+                                    uint32_t* __restrict__ out, size_t packed_rows, size_t cols) {
+    constexpr int P = Packing<BITS>::kPerWord;
+    constexpr uint32_t MASK = Packing<BITS>::kMask;
+    const size_t total = packed_rows * cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t row = i / cols, col = i % cols;
+        uint32_t word = 0;
+#pragma unroll
+        for (int e = 0; e < P; ++e) {
+            const size_t src = (size_t)perm[row * P + e];
+            word |= ((packed[src / P * cols + col] >> (src % P * BITS)) & MASK) << (e * BITS);
+        }
+        out[i] = word;
+    }
+}
+
 }  // namespace mh
 
 using namespace mh;
 
 extern "C" {
+
+int mh_gptq_permute_rows(mh_stream_t stream, const int32_t* qweight, const int32_t* perm, int32_t* out, int N,
+                         int K, int bits) {
+    MH_REQUIRE(bits == 4 || bits == 8, "mh_gptq_permute_rows: bits must be 4 or 8, got %d", bits);
+    MH_REQUIRE(N > 0 && K > 0 && K % (32 / bits) == 0, "mh_gptq_permute_rows: bad shape N=%d K=%d", N, K);
+    MH_REQUIRE(qweight && perm && out && qweight != out, "mh_gptq_permute_rows: null pointer, or in place");
+    const size_t packed_rows = (size_t)K / (32 / bits), total = packed_rows * N;
+    size_t blocks = (total + 255) / 256;
+    const size_t cap = (size_t)compute_units() * 16;
+    if (blocks > cap) blocks = cap;
+    if (bits == 4)
+        hipLaunchKernelGGL(permute_rows_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           (const uint32_t*)qweight, perm, (uint32_t*)out, packed_rows, (size_t)N);
+    else
+        hipLaunchKernelGGL(permute_rows_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           (const uint32_t*)qweight, perm, (uint32_t*)out, packed_rows, (size_t)N);
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
 
 int mh_gptq_unpack(mh_stream_t stream, const int32_t* packed, uint8_t* out, size_t rows, size_t cols,
                    int axis, int bits) {

@@ -57,6 +57,7 @@ PROTOTYPES = {
     "mh_i8_gemm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int]),
     "mh_i8_transpose": (c_int, [_P, _P, _P, c_int, c_int]),
     "mh_i8_mfma_probe": (c_int, [_P, _P, _P, c_int, c_int]),
+    "mh_gptq_permute_rows": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
     "mh_issue_probe": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int]),
     "mh_grid_barrier_probe": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int]),
     "mh_empty_probe": (c_int, [_P, _P, c_int]),

@@ -10,6 +10,7 @@ one group, ``P = 32 / bits``.
 import numpy
 
 from ..hip.tensor import HIPTensor
+from ..lib import call
 from .tensor import QuantizedTensor
 
 
@@ -46,14 +47,33 @@ def sort_rows_by_group(qweight: numpy.ndarray, g_idx: numpy.ndarray, bits: int, 
     ``None`` when some group does not hold exactly ``group_size`` rows: such a
     weight stays on the per-element path.
     """
+    perm = group_order(g_idx, group_size)
+    if perm is None:
+        return None
+    rows = unpack_subwords(qweight, 0, bits)          # [K, N] uint8
+    return pack_subwords(rows[perm], 0, bits), perm
+
+
+def group_order(g_idx: numpy.ndarray, group_size: int):
+    """``perm`` with ``g_idx[perm[j]] == j // group_size`` (rows stably sorted by group), or
+    ``None`` when some group does not hold exactly ``group_size`` rows."""
     g = numpy.asarray(g_idx, dtype=numpy.int64)
     k = g.shape[0]
     counts = numpy.bincount(g, minlength=k // group_size)
     if counts.shape[0] != k // group_size or (counts != group_size).any():
         return None
-    perm = numpy.argsort(g, kind="stable").astype(numpy.int32)
-    rows = unpack_subwords(qweight, 0, bits)          # [K, N] uint8
-    return pack_subwords(rows[perm], 0, bits), perm
+    return numpy.argsort(g, kind="stable").astype(numpy.int32)
+
+
+def sort_rows_by_group_on_device(qweight: HIPTensor, perm: HIPTensor, bits: int) -> HIPTensor:
+    """The repack of :func:`sort_rows_by_group` as one kernel over the packed words on the
+    device (``mh_gptq_permute_rows``), with ``perm`` from :func:`group_order`."""
+    packed_rows, n = qweight._shape
+    k = packed_rows * (32 // bits)
+    assert tuple(perm._shape) == (k,) and perm.dtype == "int32"
+    out = HIPTensor.allocate((packed_rows, n), "int32")
+    call("mh_gptq_permute_rows", None, qweight.data_ptr, perm.data_ptr, out.data_ptr, n, k, bits)
+    return out
 
 
 def quantized_tensor_from_host(qweight, qzeros, scales, g_idx=None) -> QuantizedTensor:

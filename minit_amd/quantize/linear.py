@@ -12,7 +12,7 @@ from typing import Optional
 from ..lib import DTYPE_CODES, call
 from ..hip import memory
 from ..hip.tensor import HIPTensor
-from .gptq import quantized_tensor_from_host, sort_rows_by_group
+from .gptq import group_order, quantized_tensor_from_host, sort_rows_by_group_on_device
 from .tensor import QuantizedTensor
 
 
@@ -34,19 +34,20 @@ class QLinear:
     def from_host(cls, w, reorder: bool = True) -> "QLinear":
         """From :class:`minit_amd.quantize.checkpoint.GPTQLinearWeights`.
 
-        An act-order weight (``g_idx`` not sequential) is repacked once, rows sorted
-        by group, so that the product runs on the MFMA kernels with the activations
-        gathered to match; ``reorder=False`` (or groups of uneven size) keeps the
+        An act-order weight (``g_idx`` not sequential) is repacked once on the device,
+        rows sorted by group, so that the product runs on the MFMA kernels with the
+        activations gathered to match; ``reorder=False`` (or groups of uneven size) keeps the
         checkpoint layout and the per-element kernel.
         """
         bias = None if w.bias is None else HIPTensor.from_numpy(w.bias)
         if w.g_idx is not None and reorder:
             geo = w.geometry
-            packed = sort_rows_by_group(w.qweight, w.g_idx, geo.bits, geo.group_size)
-            if packed is not None:
-                qweight, perm = packed
-                return cls(quantized_tensor_from_host(qweight, w.qzeros, w.scales, None), bias,
-                           HIPTensor.from_numpy(perm))
+            perm = group_order(w.g_idx, geo.group_size)
+            if perm is not None:
+                order = HIPTensor.from_numpy(perm)
+                weight = quantized_tensor_from_host(w.qweight, w.qzeros, w.scales, None)
+                weight._data = sort_rows_by_group_on_device(weight._data, order, geo.bits)
+                return cls(weight, bias, order)
         return cls(quantized_tensor_from_host(w.qweight, w.qzeros, w.scales, w.g_idx), bias)
 
     def forward(self, x):

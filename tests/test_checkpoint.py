@@ -153,6 +153,28 @@ def test_sort_rows_by_group_is_a_row_permutation_with_sequential_groups():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("k,n,g,bits", [(512, 24, 128, 4), (256, 16, 64, 8), (4096, 1000, 128, 4), (1024, 12, 32, 8)])
+def test_device_repack_equals_the_host_repack(hip, k, n, g, bits):
+    """mh_gptq_permute_rows against the numpy repack, word for word; a random permutation
+    (not only a sort by group) as well, and the identity returns the input."""
+    from minit_amd.hip.tensor import HIPTensor
+    from minit_amd.quantize.gptq import (group_order, sort_rows_by_group, sort_rows_by_group_on_device,
+                                         unpack_subwords)
+    rng = np.random.default_rng(k + n)
+    t = _linear(rng, k, n, g, bits, act_order=True)
+    qsorted, perm = sort_rows_by_group(t["qweight"], t["g_idx"], bits, g)
+    np.testing.assert_array_equal(perm, group_order(t["g_idx"], g))
+    words = HIPTensor.from_numpy(t["qweight"])
+    got = sort_rows_by_group_on_device(words, HIPTensor.from_numpy(perm), bits).numpy()
+    np.testing.assert_array_equal(got, qsorted)
+    shuffle = rng.permutation(k).astype(np.int32)
+    got = sort_rows_by_group_on_device(words, HIPTensor.from_numpy(shuffle), bits).numpy()
+    np.testing.assert_array_equal(got, pack_subwords(unpack_subwords(t["qweight"], 0, bits)[shuffle], 0, bits))
+    same = sort_rows_by_group_on_device(words, HIPTensor.from_numpy(np.arange(k, dtype=np.int32)), bits).numpy()
+    np.testing.assert_array_equal(same, t["qweight"])
+
+
+@pytest.mark.gpu
 def test_act_order_repacked_and_per_element_paths_agree(hip):
     """The same act-order checkpoint with and without the one-time repack, against
     the oracle; one-hot activations return rows of the dequantized matrix bit for
