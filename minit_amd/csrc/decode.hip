@@ -229,8 +229,8 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
 // alternate chunks and are merged through LDS; splits are merged by the last
 // block to arrive.
 
-template <int G, int D>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
+template <int G, int D, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
     const half_t* __restrict__ q, const half_t* __restrict__ k_cache, const half_t* __restrict__ vt_cache,
     const int32_t* __restrict__ positions, half_t* __restrict__ out, float* partial, unsigned* counters,
     int kvh, int max_seq, float scale, int splits) {
@@ -244,9 +244,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int span = ((len + splits - 1) / splits + 63) / 64 * 64;
     const int t0 = split * span, t1 = min(len, t0 + span);
 
-    __shared__ __attribute__((aligned(16))) half_t p_s[4][16 * PP];
-    __shared__ float m_s[4][16], l_s[4][16];
-    __shared__ float acc_s[4][G][D];
+    __shared__ __attribute__((aligned(16))) half_t p_s[WAVES][16 * PP];
+    __shared__ float m_s[WAVES][16], l_s[WAVES][16];
+    __shared__ float acc_s[WAVES][G][D];
 
     // A operand of S = Q K^T: row = head i16, k = dims s*32 + kq*8 .. +8
     uint4 qf[4];
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int c0 = t0 + wave * 64; c0 < t1; c0 += 256) {
+    for (int c0 = t0 + wave * 64; c0 < t1; c0 += WAVES * 64) {
         // all loads of the chunk are issued before the first use (refilling K after
         // Q K^T and V after P V for the wave's next chunk, so that loads stay in flight
         // under the arithmetic, measured no faster at batch 1 and 32 and slower at 8)
@@ -381,17 +381,19 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
     __syncthreads();
 
-    // merge the four waves: thread -> (head, four dims)
+    // merge the waves: thread -> (head, four dims)
     constexpr int REC = D + 4;        // floats per (head, split) record: acc[D], m, l, two unused
     constexpr int ITEMS = G * D / 4;  // <= 256
     const size_t head0 = ((size_t)b * kvh + g) * G;
     const int h = tid / (D / 4), d = tid % (D / 4) * 4;
     if (tid < ITEMS) {
-        const float mm = fmaxf(fmaxf(m_s[0][h], m_s[1][h]), fmaxf(m_s[2][h], m_s[3][h]));
+        float mm = m_s[0][h];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) mm = fmaxf(mm, m_s[w][h]);
         float ll = 0.f;
         float4_t a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             const float f = (m_s[w][h] == -INFINITY) ? 0.f : expf(m_s[w][h] - mm);
             ll += l_s[w][h] * f;
             a += *reinterpret_cast<const float4_t*>(&acc_s[w][h][d]) * f;
@@ -483,8 +485,13 @@ struct Scratch {
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
 
+// With a (row, KV head) pair per CU or more, a pair is one block of eight waves and nothing is merged
+// across blocks (the merge of two splits costs 3.5 us of a 56 us launch at 32 rows).
+static bool attn_unsplit(int n_kv_heads, int batch) { return batch * n_kv_heads >= compute_units(); }
+
 static int attn_splits(int n_kv_heads, int max_seq, int batch) {
     const int pairs = batch * n_kv_heads;
+    if (attn_unsplit(n_kv_heads, batch)) return 1;
     // two blocks per CU: 0.5, 1, 1.5, 4 and 8 measured no faster at any batch size (context 2048)
     int splits = (2 * compute_units() + pairs - 1) / pairs;
     // a block walks 256 positions per pass of its four waves
@@ -507,8 +514,13 @@ template <int G>
 static void launch_attn_raw(hipStream_t st, const half_t* q, const half_t* k_cache, const half_t* vt_cache,
                             const int32_t* positions, half_t* out, float* partial, unsigned* counters, int batch,
                             int n_kv_heads, int max_seq, int splits) {
-    hipLaunchKernelGGL((attn_decode_kernel<G, 128>), dim3(splits, n_kv_heads, batch), dim3(256), 0, st, q, k_cache,
-                       vt_cache, positions, out, partial, counters, n_kv_heads, max_seq, 1.0f / sqrtf(128.f), splits);
+    if (splits == 1 && attn_unsplit(n_kv_heads, batch))
+        hipLaunchKernelGGL((attn_decode_kernel<G, 128, 8>), dim3(1, n_kv_heads, batch), dim3(512), 0, st, q, k_cache,
+                           vt_cache, positions, out, partial, counters, n_kv_heads, max_seq, 1.0f / sqrtf(128.f), 1);
+    else
+        hipLaunchKernelGGL((attn_decode_kernel<G, 128, 4>), dim3(splits, n_kv_heads, batch), dim3(256), 0, st, q,
+                           k_cache, vt_cache, positions, out, partial, counters, n_kv_heads, max_seq,
+                           1.0f / sqrtf(128.f), splits);
 }
 
 static Scratch carve(const Llama& m, int batch, char* base) {

@@ -57,6 +57,9 @@ def _t(arr):
     (2, 64, 8, 2112, [2047, 1000]),         # the 70B head geometry, several splits
     (5, 4, 4, 128, [17, 64, 63, 127, 1]),   # one query head per KV head
     (2, 4, 2, 576, [300, 575]),             # two query heads per KV head
+    # a (row, KV head) pair per CU: one block of eight waves per pair, no merge across blocks;
+    # rows shorter than one pass of the block, a ragged end, the last slot
+    (32, 16, 8, 640, [(7 * i * i + 3) % 640 for i in range(29)] + [0, 511, 639]),
 ])
 def test_attention_entry_points_match_oracle(hip, batch, qh, kvh, max_seq, positions):
     from minit_amd.hip.tensor import HIPTensor
