@@ -74,7 +74,7 @@ int mh_copy_kernel(mh_stream_t stream, const void* src, void* dst, size_t bytes)
 /* out row j = qweight row perm[j] of the K unpacked rows, both packed along K ([K/P, N] int32):
  * the one-time repack of an act-order checkpoint whose rows are sorted by group
  * (examples/qwen1_5_int8.py:283-285 keeps g_idx and gathers per element at every product instead).
- * perm int32 [K] holds every row once (not checked on the device); not in place. */
+ * perm int32 [K] holds every row once (not checked; entries outside [0, K) are clamped); not in place. */
 int mh_gptq_permute_rows(mh_stream_t stream, const int32_t* qweight, const int32_t* perm, int32_t* out, int N,
                          int K, int bits);
 int mh_gptq_unpack(mh_stream_t stream, const int32_t* packed, uint8_t* out,

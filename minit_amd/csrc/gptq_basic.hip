@@ -135,7 +135,8 @@ __global__ void permute_rows_kernel(const uint32_t* __restrict__ packed, const i
         uint32_t word = 0;
 #pragma unroll
         for (int e = 0; e < P; ++e) {
-            const size_t src = (size_t)perm[row * P + e];
+            // an index outside [0, K) reads the nearest row instead of memory outside the matrix
+            const size_t src = (size_t)min(max(perm[row * P + e], 0), (int)(packed_rows * P) - 1);
             word |= ((packed[src / P * cols + col] >> (src % P * BITS)) & MASK) << (e * BITS);
         }
         out[i] = word;
