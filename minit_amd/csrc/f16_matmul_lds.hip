@@ -19,9 +19,11 @@
 // either operand past the end of its matrix are past the end of its buffer and read as zero.
 //
 // Measured, lm_head 128256 x 8192: 467-494 us at 9 to 64 rows (4.3-4.5 TB/s), flat in the row count,
-// against 581-636 us before.  The rate is that of 128-byte pieces of rows 16 KiB apart (a read-only
-// kernel with this footprint reaches 4.7 TB/s where 1 KiB runs reach 6.1-6.8); longer runs per row
-// and round need fewer rows per workgroup and a reduction over K inside it, and were not tried.
+// against 581-636 us before.  A read-only kernel with this footprint (128-byte pieces of rows 16 KiB
+// apart) reaches 4.7 TB/s where 1 KiB runs reach 6.1-6.8; rounds of 128 k (256-byte pieces, four
+// stages of 40 KiB) measured slower, 494 against 472 us at 32 rows.  Runs of 1 KiB per row and round
+// need 32 rows per workgroup (four times the activation traffic out of L2) and a reduction over K
+// inside it, and were not tried.
 #include "common.h"
 
 namespace mh {
