@@ -315,9 +315,10 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  *   qkv      fused q|k|v projection, GPTQ, [hidden] -> [(QH + 2 KVH) * D]
  *   gate_up  fused gate|up projection, [hidden] -> [2 * ffn], columns interleaved in
  *            blocks of 128 gate / 128 up as for mh_gptq_matmul_silu_pairs (ffn % 128 == 0)
- *   k_cache  fp16 [batch_max, KVH, max_seq, D], v_cache fp16 [batch_max, KVH, D, max_seq]
- *            (V is kept transposed for the P.V matrix product); both appended in place;
- *            max_seq is a multiple of 8
+ *   k_cache  fp16 [batch_max, KVH, max_seq, D], v_cache fp16 [batch_max, KVH, max_seq / 64, D, 64]
+ *            (V is kept with positions contiguous, in tiles of 64, for the P.V matrix product:
+ *            value d of position p sits at ((p / 64) * D + d) * 64 + p % 64 of its row and KV
+ *            head); both appended in place; max_seq is a multiple of 64
  *   embed, lm_head     fp16 [vocab, hidden]; norms fp16 [hidden]
  *   freqs_cos / sin    fp32 [max_seq, D / 2]
  */
@@ -328,8 +329,9 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  *   mh_rope_kv_append   qkv fp16 [batch, (QH + 2 KVH) * D] (q heads, then k heads, then
  *                       v heads): q and k rotated at positions[b] with the interleaved
  *                       pairs of mh_rope, q to q_out [batch, QH, D], k into k_cache
- *                       [batch, KVH, max_seq, D] and v into vt_cache [batch, KVH, D,
- *                       max_seq] at that position (clamped to the cache)
+ *                       [batch, KVH, max_seq, D] and v into vt_cache [batch, KVH,
+ *                       max_seq / 64, D, 64] (the tiled layout of v_cache above) at that
+ *                       position (clamped to the cache); max_seq a multiple of 64
  *   mh_attn_decode      out[b, h] = softmax(q[b, h] . K[b, h / (QH / KVH), 0..positions[b]] / sqrt(D)) . V,
  *                       fp32 inside, one rounding; D == 128, QH / KVH in {1, 2, 4, 8};
  *                       positions[b] is the index of the newest cache entry.  The

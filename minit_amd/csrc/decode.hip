@@ -102,7 +102,7 @@ __global__ void add_kernel(half_t* __restrict__ h, const half_t* __restrict__ de
 }
 
 // qkv [B, (QH + 2 KVH) * D]: rotate q heads into q_out [B, QH, D]; rotate k
-// heads and copy v heads into the caches at positions[b] (V transposed).  One 64-thread block
+// heads and copy v heads into the caches at positions[b] (V tiled, vt_offset).  One 64-thread block
 // per (head, batch row); thread i owns the interleaved pair i
 // (minit/cuda/kernel/cuda/rope.py:58-73).
 __global__ __launch_bounds__(64) void rope_kv_append_kernel(
@@ -116,10 +116,10 @@ __global__ __launch_bounds__(64) void rope_kv_append_kernel(
     for (int i = threadIdx.x; i < half_dim; i += blockDim.x) {
         const float re = (float)src[2 * i], im = (float)src[2 * i + 1];
         if (head >= qh + kvh) {  // v: plain copy
-            // the V cache is dim-major, [B, KVH, D, T]: see attn_decode_kernel
-            half_t* dst = v_cache + ((size_t)b * kvh + (head - qh - kvh)) * head_dim * max_seq + pos;
-            dst[(size_t)(2 * i) * max_seq] = src[2 * i];
-            dst[(size_t)(2 * i + 1) * max_seq] = src[2 * i + 1];
+            // the V cache is tiled, [B, KVH, T / 64, D, 64]: see vt_offset
+            half_t* dst = v_cache + ((size_t)b * kvh + (head - qh - kvh)) * head_dim * max_seq + vt_offset(2 * i, pos, head_dim);
+            dst[0] = src[2 * i];
+            dst[kVTile] = src[2 * i + 1];
             continue;
         }
         const float c = freqs_cos[(size_t)pos * half_dim + i], s = freqs_sin[(size_t)pos * half_dim + i];
@@ -225,7 +225,8 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
 // max / sum softmax on the accumulator layout, passes P through LDS to turn it
 // into an A operand, and accumulates O += P V with 16 more MFMAs.  For that
 // product the B operand needs eight consecutive positions of one dim per lane,
-// so V is cached transposed, [B, KVH, D, T] (positions contiguous).  Waves own
+// so V is cached with positions contiguous, in tiles of 64, [B, KVH, T / 64, D, 64]
+// (vt_offset: a chunk of a wave is one tile).  Waves own
 // alternate chunks and are merged through LDS; splits are merged by the last
 // block to arrive.
 
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i16 = lane & 15, kq = lane >> 4;
     const int len = min(max(positions[b], 0), max_seq - 1) + 1;  // the new token has been appended
-    // chunk starts stay multiples of 64 so that the transposed V reads are 16-byte aligned
+    // chunk starts stay multiples of 64: a chunk is one tile of the V cache
     const int span = ((len + splits - 1) / splits + 63) / 64 * 64;
     const int t0 = split * span, t1 = min(len, t0 + span);
 
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
             const int p0 = min(c0 + ks * 32 + kq * 8, max_seq - 8);
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
-                vf[dt][ks] = *reinterpret_cast<const uint4*>(vbase + (size_t)(dt * 16 + i16) * max_seq + p0);
+                vf[dt][ks] = *reinterpret_cast<const uint4*>(vbase + vt_offset(dt * 16 + i16, p0));
         }
 
         // S tile pt: rows = heads kq*4 + r, column = position c0 + pt*16 + i16
@@ -591,7 +592,7 @@ int mh_attn_decode(mh_stream_t stream, const void* q, const void* k_cache, const
                n_kv_heads);
     const int g = n_q_heads / n_kv_heads;
     MH_REQUIRE(g == 1 || g == 2 || g == 4 || g == 8, "mh_attn_decode: %d query heads per KV head unsupported", g);
-    MH_REQUIRE(max_seq >= 8 && max_seq % 8 == 0, "mh_attn_decode: max_seq must be a multiple of 8, got %d", max_seq);
+    MH_REQUIRE(max_seq >= kVTile && max_seq % kVTile == 0, "mh_attn_decode: max_seq must be a multiple of 64, got %d", max_seq);
     MH_REQUIRE(((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)vt_cache | (uintptr_t)out) % 16 == 0,
                "mh_attn_decode: operands must be 16-byte aligned");
     const size_t need = attn_workspace_bytes(batch, n_q_heads, n_kv_heads, head_dim, max_seq);
@@ -649,8 +650,9 @@ int mh_rope_kv_append(mh_stream_t stream, const void* qkv, const float* freqs_co
     if (batch == 0) return MH_OK;
     MH_REQUIRE(qkv && freqs_cos && freqs_sin && positions && q_out && k_cache && vt_cache,
                "mh_rope_kv_append: null pointer");
-    MH_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && n_q_heads > 0 && n_kv_heads > 0 && max_seq > 0,
-               "mh_rope_kv_append: bad sizes");
+    MH_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && n_q_heads > 0 && n_kv_heads > 0, "mh_rope_kv_append: bad sizes");
+    MH_REQUIRE(max_seq >= kVTile && max_seq % kVTile == 0, "mh_rope_kv_append: max_seq must be a multiple of 64, got %d",
+               max_seq);
     hipLaunchKernelGGL(rope_kv_append_kernel, dim3(n_q_heads + 2 * n_kv_heads, batch), dim3(64), 0, as_stream(stream),
                        (const half_t*)qkv, freqs_cos, freqs_sin, positions, (half_t*)q_out, (half_t*)k_cache,
                        (half_t*)vt_cache, n_q_heads, n_kv_heads, head_dim, max_seq);
@@ -665,7 +667,8 @@ int mh_llama_create(void** handle, const mh_llama_config* cfg) {
     MH_REQUIRE(cfg->n_kv_heads > 0 && cfg->n_q_heads % cfg->n_kv_heads == 0, "mh_llama_create: bad head counts");
     const int g = cfg->n_q_heads / cfg->n_kv_heads;
     MH_REQUIRE(g == 1 || g == 2 || g == 4 || g == 8, "mh_llama_create: %d query heads per KV head unsupported", g);
-    MH_REQUIRE(cfg->max_seq >= 8 && cfg->max_seq % 8 == 0, "mh_llama_create: max_seq must be a multiple of 8, got %d", cfg->max_seq);
+    MH_REQUIRE(cfg->max_seq >= kVTile && cfg->max_seq % kVTile == 0, "mh_llama_create: max_seq must be a multiple of 64, got %d",
+               cfg->max_seq);
     MH_REQUIRE(cfg->hidden % 8 == 0 && cfg->hidden <= 8192, "mh_llama_create: hidden must be <= 8192 and a multiple of 8");
     MH_REQUIRE(cfg->ffn % 128 == 0, "mh_llama_create: ffn must be a multiple of 128 (gate/up interleave)");
     {

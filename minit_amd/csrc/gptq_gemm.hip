@@ -667,11 +667,11 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 }
                 const float4_t sum = sum_splits(partial + (size_t)m * N + c);
                 const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
-                if (!rotated) {  // value head: copied, cache is dim-major
-                    half_t* dst = fuse.vt_cache + (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) *
-                                                      fuse.max_seq + pos;
+                if (!rotated) {  // value head: copied, cache is tiled
+                    half_t* dst = fuse.vt_cache + ((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 * fuse.max_seq +
+                                  vt_offset(d, pos);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
+                    for (int e = 0; e < 4; ++e) dst[e * kVTile] = y[e];
                     continue;
                 }
                 half4_t o;

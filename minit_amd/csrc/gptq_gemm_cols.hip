@@ -355,11 +355,11 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         // the two columns are one interleaved pair of a head of 128 dims (gptq_common.h)
         const int head = col / 128, d = col % 128;
         const int pos = ep_pos;  // clamped to the cache at the start
-        if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
-            half_t* dst = fuse.vt_cache +
-                          (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;
+        if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is tiled
+            half_t* dst = fuse.vt_cache + ((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 * fuse.max_seq +
+                          vt_offset(d, pos);
             dst[0] = y[0];
-            dst[fuse.max_seq] = y[1];
+            dst[kVTile] = y[1];
             return;
         }
         const float cs = ep_cos, sn = ep_sin;

@@ -232,11 +232,11 @@ __global__ __launch_bounds__(256) void splitk_finalize_rope_kernel(const float* 
     const int m = (int)(i / N), c = (int)(i % N);
     const int head = c / 128, d = c % 128;
     const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
-    if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is dim-major
-        half_t* dst = fuse.vt_cache +
-                      (((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 + d) * fuse.max_seq + pos;
+    if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is tiled
+        half_t* dst = fuse.vt_cache + ((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 * fuse.max_seq +
+                      vt_offset(d, pos);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[(size_t)e * fuse.max_seq] = y[e];
+        for (int e = 0; e < 4; ++e) dst[e * kVTile] = y[e];
         return;
     }
     const float* cr = fuse.rope_cos + (size_t)pos * 64 + d / 2;

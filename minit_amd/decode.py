@@ -55,12 +55,30 @@ def interleave_gate_up(qweight, qzeros, scales, bits=4):
     return qweight[:, cols], qzeros[:, words], scales[:, cols]
 
 
+V_TILE = 64
+
+
+def tile_v_cache(v: np.ndarray) -> np.ndarray:
+    """``[B, KVH, T, D]`` (T a multiple of 64) to the layout the attention kernel reads,
+    ``[B, KVH, T / 64, D, 64]``: positions contiguous, in tiles of 64, so that the 64
+    positions x D values of one step of a wave are one piece of memory."""
+    b, h, t, d = v.shape
+    assert t % V_TILE == 0, f"cache length {t} must be a multiple of {V_TILE}"
+    return np.ascontiguousarray(v.reshape(b, h, t // V_TILE, V_TILE, d).transpose(0, 1, 2, 4, 3))
+
+
+def untile_v_cache(vt: np.ndarray) -> np.ndarray:
+    """Inverse of :func:`tile_v_cache`: ``[B, KVH, T / 64, D, 64]`` to ``[B, KVH, T, D]``."""
+    b, h, tiles, d, w = vt.shape
+    return np.ascontiguousarray(vt.transpose(0, 1, 2, 4, 3).reshape(b, h, tiles * w, d))
+
+
 def decode_attention(q, k_cache, vt_cache, positions, max_seq: int):
     """Attention of one new token per row over a preallocated cache (the core of
     examples/llama3_70b.py:77-113 for a decode step) through ``mh_attn_decode``.
 
-    ``q [B, QH, 128]``, ``k_cache [B, KVH, max_seq, 128]``, ``vt_cache [B, KVH, 128,
-    max_seq]`` (V transposed), ``positions [B]`` int32 = index of the newest entry;
+    ``q [B, QH, 128]``, ``k_cache [B, KVH, max_seq, 128]``, ``vt_cache [B, KVH, max_seq / 64,
+    128, 64]`` (:func:`tile_v_cache`), ``positions [B]`` int32 = index of the newest entry;
     all :class:`HIPTensor`.  Returns ``[B, QH, 128]``.
     """
     batch, qh, d = q._shape
@@ -92,7 +110,7 @@ class LlamaDecoder:
 
     def __init__(self, config: dict, batch_max: int, max_seq: int):
         self.config = dict(config)
-        # the transposed V cache is read 8 positions (16 bytes) at a time; rows of whole 128-byte lines keep those reads inside one line
+        # the V cache is kept in tiles of 64 positions
         max_seq = (max_seq + 63) // 64 * 64
         self.batch_max, self.max_seq = batch_max, max_seq
         c = self.config
@@ -118,9 +136,10 @@ class LlamaDecoder:
     # ---- weights ------------------------------------------------------------------------------
     def _alloc_cache(self):
         c = self.config
-        # K is [B, KVH, T, D]; V is kept transposed, [B, KVH, D, T], for the P.V matrix product
+        # K is [B, KVH, T, D]; V is kept with positions contiguous, in tiles of 64 (tile_v_cache), for the
+        # P.V matrix product
         k_shape = (self.batch_max, c["n_kv_heads"], self.max_seq, c["head_dim"])
-        v_shape = (self.batch_max, c["n_kv_heads"], c["head_dim"], self.max_seq)
+        v_shape = (self.batch_max, c["n_kv_heads"], self.max_seq // V_TILE, c["head_dim"], V_TILE)
         kc, vc = HIPTensor.allocate(k_shape, "float16"), HIPTensor.allocate(v_shape, "float16")
         kc._memory.reset()
         vc._memory.reset()
@@ -199,10 +218,10 @@ class LlamaDecoder:
                 t = k_cache[l].shape[2]
                 kpad = np.zeros(kc._shape, np.float16)
                 kpad[:, :, :t] = k_cache[l]
-                vpad = np.zeros(vc._shape, np.float16)
-                vpad[:, :, :, :t] = np.transpose(v_cache[l], (0, 1, 3, 2))
+                vpad = np.zeros(kc._shape, np.float16)
+                vpad[:, :, :t] = v_cache[l]
                 kc.copy_from_numpy(kpad)
-                vc.copy_from_numpy(vpad)
+                vc.copy_from_numpy(tile_v_cache(vpad))
             self._set_layer(l, linears, HIPTensor.from_numpy(layer["input_norm"]),
                             HIPTensor.from_numpy(layer["post_norm"]), kc, vc)
         self._set_globals(HIPTensor.from_numpy(model["embed"]), HIPTensor.from_numpy(model["lm_head"]),

@@ -18,6 +18,7 @@ import pytest
 from oracle import cport
 from oracle import decode as OD
 from oracle import special as OS
+from minit_amd.decode import untile_v_cache
 
 pytestmark = pytest.mark.gpu
 
@@ -94,12 +95,12 @@ def test_two_layers_at_70b_widths(hip, wide_model, batch):
     # appended keys and values, each row at its own position: layer 0 sees only the q|k|v product and RoPE,
     # layer 1 everything the first layer computed (attention, o + residual, gate|up + SiLU, down + residual, norm)
     for layer in range(CFG["n_layers"]):
-        kc, vc = dec.k_cache[layer].numpy(), dec.v_cache[layer].numpy()      # V is kept [B, KVH, D, T]
+        kc, vc = dec.k_cache[layer].numpy(), untile_v_cache(dec.v_cache[layer].numpy())   # both [B, KVH, T, D]
         tol = 2e-2 if layer == 0 else 6e-2
         for b in range(batch):
             p = int(positions[b])
             ek = np.abs(kc[b, :, p].astype(np.float64) - ref_k[layer][b, :, p].astype(np.float64)).max()
-            ev = np.abs(vc[b, :, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max()
+            ev = np.abs(vc[b, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max()
             assert ek <= tol and ev <= tol, f"layer {layer} row {b}: appended k/v off by {ek:.3g} / {ev:.3g}"
         # what was already in the cache stays (row 0, below its position)
         p0 = int(positions[0])

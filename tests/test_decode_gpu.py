@@ -11,6 +11,7 @@ import pytest
 
 from oracle import decode as OD
 from oracle import special as OS
+from minit_amd.decode import untile_v_cache
 
 pytestmark = pytest.mark.gpu
 
@@ -186,12 +187,12 @@ def test_decode_wide_qkv_on_cut_tiles(hip, batch):
     assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
     # the appended keys and values of both layers, each row at its own position
     for layer in range(cfg["n_layers"]):
-        kc, vc = dec.k_cache[layer].numpy(), dec.v_cache[layer].numpy()  # V is kept [B, KVH, D, T]
+        kc, vc = dec.k_cache[layer].numpy(), untile_v_cache(dec.v_cache[layer].numpy())  # both [B, KVH, T, D]
         for b in range(batch):
             p = int(positions[b])
             tol = 2e-2 if layer == 0 else 6e-2  # layer 1 sees layer 0's rounding differences
             assert np.abs(kc[b, :, p].astype(np.float64) - ref_k[layer][b, :, p].astype(np.float64)).max() <= tol
-            assert np.abs(vc[b, :, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max() <= tol
+            assert np.abs(vc[b, :, p].astype(np.float64) - ref_v[layer][b, :, p].astype(np.float64)).max() <= tol
 
 
 @pytest.mark.parametrize("batch", [1, 3, 9])
@@ -279,8 +280,8 @@ def test_positions_are_kept_inside_the_cache(hip):
     for l in range(CFG["n_layers"]):
         kb, ka = before[l], after[l]                      # [B, KVH, T, D]
         assert np.array_equal(kb[:, :, :max_seq - 1].view(np.uint16), ka[:, :, :max_seq - 1].view(np.uint16))
-        vb, va = before[CFG["n_layers"] + l], after[CFG["n_layers"] + l]   # [B, KVH, D, T]
-        assert np.array_equal(vb[..., :max_seq - 1].view(np.uint16), va[..., :max_seq - 1].view(np.uint16))
+        vb, va = (untile_v_cache(c[CFG["n_layers"] + l]) for c in (before, after))   # [B, KVH, T, D]
+        assert np.array_equal(vb[:, :, :max_seq - 1].view(np.uint16), va[:, :, :max_seq - 1].view(np.uint16))
 
 
 @pytest.mark.parametrize("batch", [1, 4])

@@ -81,14 +81,16 @@ def test_attention_entry_points_match_oracle(hip, batch, qh, kvh, max_seq, posit
         v_ref[i, :, pos[i]] = v_new[i]
     ref = OD.attention(q_ref, k_ref, v_ref, pos)
 
-    dk, dvt = _t(k_cache), _t(np.transpose(v_cache, (0, 1, 3, 2)))
+    from minit_amd.decode import tile_v_cache, untile_v_cache
+    dk, dvt = _t(k_cache), _t(tile_v_cache(v_cache))
     dq = HIPTensor.allocate((batch, qh, d), "float16")
     dpos, dqkv, dcos, dsin = _t(pos), _t(qkv), _t(cos), _t(sin)   # named: the buffers must outlive the launch
     hip.call("mh_rope_kv_append", None, dqkv.data_ptr, dcos.data_ptr, dsin.data_ptr, dpos.data_ptr,
              dq.data_ptr, dk.data_ptr, dvt.data_ptr, batch, qh, kvh, d, max_seq)
     # the copy of v is exact; the rotation is fp32 on the device against float64 here, one
     # rounding each: equal except where the fp32 value sits on a rounding boundary (one step)
-    np.testing.assert_array_equal(dvt.numpy().view(np.uint16), np.transpose(v_ref, (0, 1, 3, 2)).view(np.uint16))
+    np.testing.assert_array_equal(dvt.numpy().view(np.uint16), tile_v_cache(v_ref).view(np.uint16))
+    np.testing.assert_array_equal(untile_v_cache(dvt.numpy()).view(np.uint16), v_ref.view(np.uint16))
     for got, want in ((dq.numpy(), q_ref), (dk.numpy(), k_ref)):
         step = np.spacing(np.abs(want)).astype(np.float64)
         assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= step).all()
@@ -175,7 +177,7 @@ def test_one_step_composed_from_the_operator_api(hip):
     and the stand-alone entry points, against the oracle's step and against the
     native loop's logits."""
     import minit_amd.functional as F
-    from minit_amd.decode import LlamaDecoder, decode_attention
+    from minit_amd.decode import LlamaDecoder, decode_attention, tile_v_cache
     from minit_amd.hip.tensor import HIPTensor
     from minit_amd.quantize.gptq import quantized_tensor_from_host
     from test_decode_gpu import CFG, _host_model
@@ -206,7 +208,7 @@ def test_one_step_composed_from_the_operator_api(hip):
     h = _t(model["embed"][tokens])
     xn = F.rms_norm(h, _t(model["layers"][0]["input_norm"]), 1, eps)
     for l, layer in enumerate(model["layers"]):
-        kc, vt = _t(k_cache[l]), _t(np.transpose(v_cache[l], (0, 1, 3, 2)))
+        kc, vt = _t(k_cache[l]), _t(tile_v_cache(v_cache[l]))
         qkv = F.matrix_multiply(xn, qt(layer["qkv"]))
         q = HIPTensor.allocate((batch, qh, d), "float16")
         hip.call("mh_rope_kv_append", None, qkv.data_ptr, cos.data_ptr, sin.data_ptr, pos.data_ptr, q.data_ptr,
