@@ -155,6 +155,24 @@ def test_interleave_gate_up_moves_whole_columns():
         np.testing.assert_array_equal(wi[:, t * 256 + 128:(t + 1) * 256], w[:, ffn + t * 128:ffn + (t + 1) * 128])
 
 
+def test_v_cache_tiling_follows_the_kernels_offset_rule():
+    """tile_v_cache puts value d of position p at ((p // 64) * D + d) * 64 + p % 64 of its row and
+    KV head (vt_offset in csrc/gptq_common.h), and untile_v_cache is its inverse."""
+    import numpy as np
+    from minit_amd.decode import tile_v_cache, untile_v_cache
+    b, h, t, d = 2, 3, 192, 128
+    v = np.arange(b * h * t * d, dtype=np.int64).reshape(b, h, t, d).astype(np.float32)
+    tiled = tile_v_cache(v)
+    assert tiled.shape == (b, h, t // 64, d, 64) and tiled.flags["C_CONTIGUOUS"]
+    flat = tiled.reshape(b, h, -1)
+    for p, dim in ((0, 0), (1, 0), (63, 127), (64, 5), (130, 77), (191, 127)):
+        np.testing.assert_array_equal(flat[:, :, ((p // 64) * d + dim) * 64 + p % 64], v[:, :, p, dim])
+    np.testing.assert_array_equal(untile_v_cache(tiled), v)
+    import pytest
+    with pytest.raises(AssertionError):
+        tile_v_cache(v[:, :, :100])
+
+
 def test_prototypes_match_header_argument_counts():
     """ctypes converts surplus arguments by default rules (a pointer becomes a
     truncated int), so a prototype that is one entry short corrupts a call
