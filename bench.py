@@ -278,6 +278,34 @@ def bench_small_configs(lib, HIPTensor, memory, ws):
         nbytes = 2 * (vocab * hid + m * hid + m * vocab)
         head.append({"M": m, "us": round(us, 1), "gbps": round(nbytes / us / 1e3, 1)})
     res["lm_head_f16"] = head
+    del w
+    # the decode attention on its own at the 70B head geometry, cache filled to 2048 positions
+    # (K and V read once per launch; six cache sets cycled, more than the 256 MB of the last-level cache
+    # from 8 rows on)
+    qh, kvh, d, ctx, max_seq, sets = 64, 8, 128, 2048, 2112, 6
+    attn = []
+    for batch in (1, 8, 32):
+        n = batch * kvh * max_seq * d
+        ks = [HIPTensor.allocate((batch, kvh, max_seq, d), "float16") for _ in range(sets)]
+        vs = [HIPTensor.allocate((batch, kvh, max_seq // 64, d, 64), "float16") for _ in range(sets)]
+        for i in range(sets):
+            lib.call("mh_synth_normal", None, ks[i].data_ptr, n, 0.0, 1.0, 0, 0.0, 50 + i, 0)
+            lib.call("mh_synth_normal", None, vs[i].data_ptr, n, 0.0, 1.0, 0, 0.0, 60 + i, 0)
+        q = HIPTensor.allocate((batch, qh, d), "float16")
+        lib.call("mh_synth_normal", None, q.data_ptr, batch * qh * d, 0.0, 1.0, 0, 0.0, 70, 0)
+        pos = HIPTensor.from_numpy(np.full(batch, ctx - 1, np.int32))
+        out = HIPTensor.allocate((batch, qh, d), "float16")
+        nws = lib.call("mh_attn_decode_workspace_bytes", batch, qh, kvh, d, max_seq)
+        aws = HIPTensor.allocate((nws,), "int8")
+        aws._memory.reset()
+        memory.synchronize()
+        us = _time_launches(memory, lambda i: lib.call("mh_attn_decode", None, q.data_ptr, ks[i % sets].data_ptr,
+                                                       vs[i % sets].data_ptr, pos.data_ptr, out.data_ptr, batch, qh,
+                                                       kvh, d, max_seq, aws.data_ptr, nws), iters=200, warmup=10)
+        nbytes = batch * 2 * ctx * kvh * d * 2
+        attn.append({"batch": batch, "context": ctx, "us": round(us, 1), "gbps": round(nbytes / us / 1e3, 1)})
+        del ks, vs
+    res["attention_70b"] = attn
     return res
 
 
