@@ -371,7 +371,7 @@ def main():
                     help="time only the row-wise kernels (RMSNorm, RoPE, softmax, row sum) and print their lines")
     ap.add_argument("--small-configs-only", action="store_true",
                     help="run only config 0 (GEMV 4096x4096), config 1 (Mistral-shape MLP block at 1 to 128 rows) and "
-                         "the lm_head lines, then exit")
+                         "the lm_head and decode-attention lines, then exit")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the W8A8 GEMM lines (M=2048, K=4096, N in {4096, 11008}), then exit")
     args = ap.parse_args()
