@@ -199,7 +199,7 @@ def test_sigmoid_multiply_compose_to_silu(hip):
                                    # last tile, seven rounds for six stages; exactly six rounds, four row tiles; two
                                    # blocks of 64 rows, the second ragged)
                                    (9, 16390, 448), (33, 16384, 384), (64, 20000, 1024), (70, 16400, 512), (32, 32768, 2048),
-                                   # K a multiple of 128: rounds of 128 k (five rounds for four stages, ragged tile; three stages)
+                                   # 17 rows (two row tiles, the second ragged) on a ragged last tile of columns; 48 rows (four row tiles, one empty)
                                    (17, 16390, 640), (48, 16384, 512)])
 def test_dense_matmul_nk(hip, m, n, k):
     import minit_amd.functional as F
