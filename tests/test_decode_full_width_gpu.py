@@ -105,3 +105,30 @@ def test_two_layers_at_70b_widths(hip, wide_model, batch):
         # what was already in the cache stays (row 0, below its position)
         p0 = int(positions[0])
         assert np.array_equal(kc[0, :, :p0].view(np.uint16), k_cache[layer][0, :, :p0].view(np.uint16))
+
+
+def test_recorded_step_at_70b_widths_replays_like_the_eager_loop(hip, wide_model):
+    """Three tokens at batch 32 (one unsplit attention block per row and KV head, second-stage kernels
+    for q|k|v, gate|up and down): the recorded step, replayed, gives the eager loop's tokens, logits and
+    caches bit for bit."""
+    from minit_amd.decode import LlamaDecoder
+    batch, steps = 32, 3
+    rng = np.random.default_rng(732)
+    shape = (batch, CFG["n_kv_heads"], MAX_SEQ, CFG["head_dim"])
+    k_cache = [rng.standard_normal(shape, np.float32).astype(np.float16) for _ in range(CFG["n_layers"])]
+    v_cache = [rng.standard_normal(shape, np.float32).astype(np.float16) for _ in range(CFG["n_layers"])]
+    tokens = rng.integers(0, CFG["vocab"], batch).astype(np.int32)
+    positions = (CONTEXT - (np.arange(batch) % 7) * 11).astype(np.int32)
+    runs = []
+    for graph in (False, True):
+        print(f"[70B widths] batch {batch}, {steps} steps, graph={graph}", flush=True)
+        dec = LlamaDecoder(CFG, batch, MAX_SEQ)
+        dec.load_host(wide_model, k_cache, v_cache)
+        out, logits = dec.decode(tokens, positions, steps, want_logits=True, graph=graph)
+        runs.append((out, logits, [t.numpy() for t in dec.k_cache + dec.v_cache]))
+        del dec
+    (out_e, logits_e, cache_e), (out_g, logits_g, cache_g) = runs
+    np.testing.assert_array_equal(out_g, out_e)
+    np.testing.assert_array_equal(logits_g.view(np.uint16), logits_e.view(np.uint16))
+    for a, b in zip(cache_g, cache_e):
+        np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
