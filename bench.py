@@ -348,23 +348,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel (1 GiB read + 1 GiB write per launch) that the "
                          "FETCH_SIZE / WRITE_SIZE counters are scaled against, then exit")
-    ap.add_argument("--calibrate-mfma", action="store_true",
-                    help="run only the register-resident int8 MFMA stream (zero and random operands), then exit")
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="untimed load (the step itself) before the warm-up steps, so that the timed steps run at the "
                          "part's steady clocks; half of it before every timed section of the extras; 0 switches it off")
-    ap.add_argument("--calibrate-barrier", action="store_true",
-                    help="time a device-wide barrier (agent-scope counter, bounded polls) of one and two workgroups "
-                         "per CU against a boundary between two dependent launches, then exit")
-    ap.add_argument("--calibrate-stream", action="store_true",
-                    help="read the packed words of gate|up (8192 x 57344, six sets) with the small-M kernel's load "
-                         "footprint and no arithmetic, and the same shape at other K, then exit")
-    ap.add_argument("--calibrate-issue", action="store_true",
-                    help="run only the register-resident vector + MFMA instruction mix at 1, 2 and 4 waves per "
-                         "SIMD (do vector and matrix instructions of one SIMD's waves overlap?), then exit")
-    ap.add_argument("--issue-case", default="",
-                    help="with --calibrate-issue: run one case only, 'valu,mfma,dependent,waves_per_simd' "
-                         "(for a counter run under rocprofv3)")
     ap.add_argument("--int8-library", action="store_true",
                     help="time the vendor library's int8 GEMM (torch._int_mm) on the W8A8 shapes, then exit")
     ap.add_argument("--rowwise-only", action="store_true",
@@ -414,120 +400,6 @@ def main():
                           "us": round(us, 1), "gbps_read_plus_write": round(2 * nbytes / us / 1e3, 1)}))
         return
 
-    if args.calibrate_mfma:
-        # what the int8 matrix pipes sustain from registers alone, all-zero vs random operands
-        blocks, iters = 256 * 2, 40000          # two waves per SIMD
-        nbytes = blocks * 512 * 96
-        res = []
-        for label in ("zero", "random"):
-            ops_buf = HIPTensor.allocate((nbytes,), "int8")
-            if label == "zero":
-                ops_buf._memory.reset()
-            else:
-                lib.call("mh_synth_i8", None, ops_buf.data_ptr, nbytes, -127, 127, 99)
-            sink = HIPTensor.allocate((blocks * 512,), "int32")
-            lib.call("mh_i8_mfma_probe", None, ops_buf.data_ptr, sink.data_ptr, blocks, 1000)
-            memory.synchronize()
-            e0, e1 = memory.Event(), memory.Event()
-            e0.record()
-            lib.call("mh_i8_mfma_probe", None, ops_buf.data_ptr, sink.data_ptr, blocks, iters)
-            e1.record()
-            e1.synchronize()
-            ms = e0.elapsed_ms(e1)
-            tops = iters * 8 * 65536.0 * (blocks * 512 / 64) / (ms * 1e9)
-            res.append({"operands": label, "ms": round(ms, 2), "tops": round(tops, 1),
-                        "frac_of_datasheet": round(tops / INT8_PEAK_TOPS, 4)})
-        print(json.dumps({"kernel": "i8_mfma_probe_kernel", "waves_per_simd": 2, "results": res}))
-        return
-
-    if args.calibrate_barrier:
-        cus = info["compute_units"]
-        words = HIPTensor.allocate((32 * 18,), "int32")   # counters on lines of their own, error word last
-        err_ptr = words.data_ptr + 32 * 17 * 4
-        rows = []
-        for per_cu in (1, 2):
-            for groups in (1, 8):
-                blocks, rounds = cus * per_cu, 2000
-                words.memory.reset()
-                lib.call("mh_grid_barrier_probe", None, words.data_ptr, err_ptr, blocks, 10, 1 << 16, groups)
-                memory.synchronize()
-                words.memory.reset()
-                memory.synchronize()
-                e0, e1 = memory.Event(), memory.Event()
-                e0.record()
-                lib.call("mh_grid_barrier_probe", None, words.data_ptr, err_ptr, blocks, rounds, 1 << 16, groups)
-                e1.record()
-                e1.synchronize()
-                gave_up = int(words.numpy()[32 * 17])
-                ns = e0.elapsed_ms(e1) * 1e6 / rounds
-                rows.append({"workgroups": blocks, "arrival_groups": groups, "rounds": rounds,
-                             "ns_per_barrier": round(ns, 1), "gave_up": gave_up})
-                log(f"device-wide barrier, {blocks} workgroups, {groups} arrival group(s): {ns:.0f} ns per round "
-                    f"(gave up: {gave_up})")
-        launches = 2000
-        for blocks in (cus, 2 * cus):
-            for i in range(20):
-                lib.call("mh_empty_probe", None, None, blocks)
-            memory.synchronize()
-            e0, e1 = memory.Event(), memory.Event()
-            e0.record()
-            for i in range(launches):
-                lib.call("mh_empty_probe", None, None, blocks)
-            e1.record()
-            e1.synchronize()
-            ns = e0.elapsed_ms(e1) * 1e6 / launches
-            rows.append({"workgroups": blocks, "launches": launches, "ns_per_empty_launch": round(ns, 1)})
-            log(f"empty launch of {blocks} workgroups, back to back in one stream: {ns:.0f} ns per launch")
-        print(json.dumps({"kernel": "grid_barrier_probe_kernel", "results": rows}))
-        return
-
-    if args.calibrate_stream:
-        n, sets = 57344, 6
-        rows_max = 2048
-        words = [HIPTensor.allocate((rows_max, n), "int32") for _ in range(sets)]
-        for i, w in enumerate(words):
-            lib.call("mh_synth_u32", None, w.data_ptr, rows_max * n, 77 + i)
-        sink = HIPTensor.allocate((256,), "int32")
-        rows_out = []
-        for k, parts in ((8192, 2), (8192, 4), (16384, 2)):
-            rows = k // 8
-            us = _time_launches(memory, lambda i: lib.call("mh_weight_stream_probe", None, words[i % sets].data_ptr,
-                                                           sink.data_ptr, rows, n, parts), iters=120, warmup=12)
-            nbytes = rows * n * 4
-            rows_out.append({"K": k, "N": n, "parts": parts, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1)})
-            log(f"weight stream {k}x{n}, {parts} K parts: {us:.1f} us, {nbytes / us / 1e3:.0f} GB/s")
-        print(json.dumps({"kernel": "weight_stream_probe_kernel", "results": rows_out}))
-        return
-
-    if args.calibrate_issue:
-        cus = info["compute_units"]
-        iters = 20000
-        cases = [(52, 0, 0), (0, 4, 0), (52, 4, 0), (52, 4, 1), (26, 4, 1), (104, 4, 1), (0, 8, 0)]
-        waves = (1, 2, 4)
-        if args.issue_case:
-            nv, nm, dep, w = (int(v) for v in args.issue_case.split(","))
-            cases, waves = [(nv, nm, dep)], (w,)
-        rows = []
-        for wps in waves:
-            blocks = cus * wps                      # 256 threads = 4 waves = one per SIMD and block
-            sink = HIPTensor.allocate((blocks * 256,), "float32")
-            for nv, nm, dep in cases:
-                lib.call("mh_issue_probe", None, sink.data_ptr, blocks, 200, nv, nm, dep)
-                memory.synchronize()
-                e0, e1 = memory.Event(), memory.Event()
-                e0.record()
-                lib.call("mh_issue_probe", None, sink.data_ptr, blocks, iters, nv, nm, dep)
-                e1.record()
-                e1.synchronize()
-                ns = e0.elapsed_ms(e1) * 1e6 / iters           # per iteration of every wave of a SIMD
-                rows.append({"waves_per_simd": wps, "valu": nv, "mfma": nm, "dependent": bool(dep),
-                             "ns_per_iteration_per_simd": round(ns / wps, 1),
-                             "ns_per_iteration_per_wave": round(ns, 1)})
-                log(f"waves/SIMD {wps}: {nv:3d} vector + {nm} MFMA (dependent={dep}): "
-                    f"{ns / wps:7.1f} ns per iteration per SIMD")
-        print(json.dumps({"kernel": "issue_probe_kernel", "iterations": iters, "results": rows}))
-        return
-
     if args.rowwise_only:
         print(json.dumps({"rowwise_cfg3": bench_rowwise(lib, HIPTensor, memory)}))
         return
@@ -561,53 +433,73 @@ def main():
         for lin in layers[i % args.layers]:
             run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
 
+    def timed_steps(fn, count):
+        e0, e1 = memory.Event(), memory.Event()
+        e0.record()                      # null stream: the stream the kernels run on
+        for i in range(count):
+            fn(i)
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_ms(e1)
+
+    step_bytes = sum(linear_bytes(1, k, n) for _, k, n in LINEARS)
+    # the same K steps right after the warm-up, before the clocks have settled: the figure earlier
+    # versions of this benchmark reported as `value`, kept so that results stay comparable
+    for i in range(args.warmup):
+        step(i)
+    memory.synchronize()
+    unsettled_ms = timed_steps(step, args.steps)
+    gbps_unsettled = step_bytes / (unsettled_ms / args.steps * 1e-3) / 1e9
     if args.settle_ms > 0:
         settled = _settle(memory, step, args.settle_ms)
         log(f"settled the clocks with {settled} untimed steps ({args.settle_ms:.0f} ms)")
     for i in range(args.warmup):
         step(i)
     memory.synchronize()
-    e0, e1 = memory.Event(), memory.Event()
     wall0 = time.perf_counter()
-    e0.record()                      # null stream: the stream the kernels run on
-    for i in range(args.steps):
-        step(i)
-    e1.record()
-    e1.synchronize()
+    dev_ms = timed_steps(step, args.steps)
     memory.synchronize()
     wall = time.perf_counter() - wall0
-    dev_ms = e0.elapsed_ms(e1)
     ms_per_step = dev_ms / args.steps
-    step_bytes = sum(linear_bytes(1, k, n) for _, k, n in LINEARS)
     gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
     launches = args.steps * len(LINEARS)
     log(f"{args.steps} steps: {dev_ms:.2f} ms on device ({wall * 1e3:.2f} ms wall), "
-        f"{ms_per_step * 1e3:.1f} us/step, {gbps:.0f} GB/s")
+        f"{ms_per_step * 1e3:.1f} us/step, {gbps:.0f} GB/s ({gbps_unsettled:.0f} GB/s before the clocks settled)")
 
-    # ---- the dominant kernel (gate|up: 55 % of the step's bytes): its average launch duration inside the
-    # layer sequence = what the same K steps lose when that launch is left out (HIP events around both
-    # passes).  An event pair around every launch, also reported, brackets the launch with two more
-    # packets on the stream and reads 2-3 us more than the kernel trace of the same command; the
-    # difference of the two passes agrees with it.
+    # ---- the dominant kernel (gate|up: 55 % of the step's bytes).  Its average launch duration is measured
+    # directly: max(K, 200) launches of it back to back over the cycled weight sets between one pair of HIP
+    # events on the stream it runs on (the gaps between the launches, well under a microsecond, are part of
+    # the figure, so it reads slightly above the kernel trace of the same command, never below).  Two other
+    # readings are reported beside it and are not the roofline figure: what the step loses when that launch
+    # is left out (`marginal_us_in_step`: a difference of two passes, which also drops one launch boundary),
+    # and the mean of an event pair around every such launch inside the step (two more packets per launch,
+    # 2-3 us above the trace).
     dom = max(range(len(LINEARS)), key=lambda j: linear_bytes(1, LINEARS[j][1], LINEARS[j][2]))
     dom_name, dom_k, dom_n = LINEARS[dom]
+    dom_count = max(args.steps, 200)
+
+    def dom_only(i):
+        lin = layers[i % args.layers][dom]
+        run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
 
     def step_without(i):
         for j, lin in enumerate(layers[i % args.layers]):
             if j != dom:
                 run_gemv(lib, xs[lin.k], lin, outs[lin.n], ws, entry=ENTRY)
 
-    for i in range(max(args.warmup, 20)):
+    for i in range(20):
+        dom_only(i)
+    memory.synchronize()
+    dom_us = timed_steps(dom_only, dom_count) * 1e3 / dom_count
+    for i in range(20):
+        step(i)
+    memory.synchronize()
+    with_ms = timed_steps(step, dom_count)
+    for i in range(20):
         step_without(i)
     memory.synchronize()
-    s0, s1 = memory.Event(), memory.Event()
-    s0.record()
-    for i in range(args.steps):
-        step_without(i)
-    s1.record()
-    s1.synchronize()
-    dom_us = (dev_ms - s0.elapsed_ms(s1)) * 1e3 / args.steps
-    pairs = [(memory.Event(), memory.Event()) for _ in range(min(args.steps, 400))]
+    marginal_us = (with_ms - timed_steps(step_without, dom_count)) * 1e3 / dom_count
+    pairs = [(memory.Event(), memory.Event()) for _ in range(min(dom_count, 400))]
     for i in range(len(pairs)):
         for j, lin in enumerate(layers[i % args.layers]):
             if j == dom:
@@ -620,8 +512,8 @@ def main():
     dom_bytes = linear_bytes(1, dom_k, dom_n)
     dom_gbps = dom_bytes / dom_us / 1e3
     traffic, traffic_commit = measured_traffic(ENTRY)
-    log(f"dominant kernel ({dom_name} {dom_k}x{dom_n}): {dom_us:.2f} us per launch in the layer sequence "
-        f"({dom_pair_us:.2f} us between an event pair per launch), {dom_gbps:.0f} GB/s")
+    log(f"dominant kernel ({dom_name} {dom_k}x{dom_n}): {dom_us:.2f} us per launch back to back ({dom_count} launches), "
+        f"{dom_gbps:.0f} GB/s; marginal in the step {marginal_us:.2f} us, event pair per launch {dom_pair_us:.2f} us")
 
     result = {
         "metric": "w4a16_gemv_hbm_gbps",
@@ -636,6 +528,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
+        # the same steps timed before the untimed settle_ms of load (clocks not yet steady)
+        "value_unsettled": round(gbps_unsettled, 1),
+        "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
         "config": {
             "workload": "llama3-70b-shape GPTQ w4a16 decode GEMVs, M=1, group 128: qkv 8192x10240, "
                         "o 8192x8192, gate_up 8192x57344, down 28672x8192; one step = one layer",
@@ -654,13 +549,16 @@ def main():
             "unit": "GB/s",
             "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
             "avg_launch_us": round(dom_us, 3),
+            "launches_timed": dom_count,
+            "marginal_us_in_step": round(marginal_us, 3),
             "avg_launch_us_event_pair_per_launch": round(dom_pair_us, 3),
             "bytes_per_launch": dom_bytes,
             "traffic": traffic,
             "traffic_measured_at_commit": traffic_commit,
-            # the whole step (four launches, two kernels, launch gaps included) on the same scale
-            "step": {"achieved": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "avg_launch_us": round(dev_ms * 1e3 / launches, 3), "bytes_per_launch": step_bytes // len(LINEARS)},
+            # the whole step (four launches, launch gaps included) on the same scale: the headline value
+            "step_achieved": round(gbps, 1),
+            "step_frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "step_avg_launch_us": round(dev_ms * 1e3 / launches, 3),
         },
     }
 

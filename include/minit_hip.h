@@ -144,7 +144,10 @@ int mh_gptq_linear(mh_stream_t stream, const void* x, const int32_t* qweight, co
 
 /* mh_gptq_matmul for callers that cannot allocate device memory or pass a
  * workspace: code under HIP graph capture, tight serving loops, harnesses that
- * forbid hipMalloc.  No counterpart in the reference (its fused product
+ * forbid hipMalloc.  The first call on a device looks up the address of the
+ * built-in buffer (hipGetSymbolAddress), which a stream capture must not record:
+ * make that call outside any capture (a call under capture before it fails with
+ * MH_ERR_INVALID and records nothing); every later call may be captured.  No counterpart in the reference (its fused product
  * accumulates with atomics into a zeroed output and needs no scratch,
  * examples/qwen1_5_int8.py:198,263).  Same arguments and results as
  * mh_gptq_matmul without the workspace pair: the split-K counters and partial
@@ -169,10 +172,13 @@ int mh_gptq_matmul_static(mh_stream_t stream, const void* x, const int32_t* qwei
  * is up column t*128 + c; qzeros and scales permuted alike -- a load-time
  * permutation of whole 8-column words).  out is [M, N / 2]:
  *   out[m, t*128 + c] = fp16( silu(y[m, t*256 + c]) * y[m, t*256 + 128 + c] ),
- * y the fp16-rounded product, silu and the multiply in fp32.  N % 256 == 0.  Up to
- * 32 rows with group_size in {32, 64, 128, 256} it is one launch (the epilogue
- * runs in the product's reduction); otherwise the product goes to the workspace
- * and one more pass applies the epilogue.  The workspace is always required:
+ * y the fp16-rounded product, silu and the multiply in fp32.  N % 256 == 0.  It is
+ * one launch up to 32 rows with group_size in {32, 64, 128, 256} (the epilogue runs
+ * in the product's reduction) and, above 32 rows, for 4-bit weights with K a
+ * multiple of 128 and at least 512 whose column tiles fill the GPU without a split
+ * of K (the epilogue runs in the store of the 64- or 128-row blocks); otherwise the
+ * product goes to the workspace and one more pass applies the epilogue.  The
+ * workspace is always required:
  * mh_gptq_silu_pairs_workspace_bytes(M, N, K, ...) bytes, zero-filled once. */
 size_t mh_gptq_silu_pairs_workspace_bytes(int M, int N, int K, int group_size, int bits);
 int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* qweight,
@@ -187,6 +193,12 @@ int mh_gptq_matmul_silu_pairs(mh_stream_t stream, const void* x, const int32_t* 
  */
 int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out,
                      int M, int N, int K);
+/* BatchMatrixMultiply (minit/cuda/dispatch.py:82-101: the whole batch in one strided library call,
+ * e.g. the q.k^T and p.v products of a prefill, `einsum("bsnd,btnd->bnst")`): out[i] = a[i] @ b[i]^T
+ * for i < batch with a [batch, M, K], b [batch, N, K], out [batch, M, N], all dense.  One launch
+ * for the whole batch (at most 65535 matrices). */
+int mh_f16_matmul_nk_batched(mh_stream_t stream, const void* a, const void* b, void* out,
+                             int batch, int M, int N, int K);
 
 /* ---- W8A8 int8 GEMM --------------------------------------------------------------
  * No counterpart in the reference (its "int8" model is weight-only,
@@ -200,37 +212,6 @@ int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out
 int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w,
                const float* a_scale, const float* w_scale, void* out_f16,
                int32_t* acc_i32, int M, int N, int K);
-/* Calibration, no counterpart in the reference: blocks x 512 threads each run
- * iters x 8 register-resident v_mfma_i32_32x32x32_i8 (2 * 32*32*32 operations
- * per wave each) on operands read once from `operands` (blocks * 512 * 96 bytes);
- * out receives blocks * 512 int32.  Used by bench.py --calibrate-mfma to find the
- * int8 rate the matrix pipes sustain on this box for given operand values. */
-int mh_i8_mfma_probe(mh_stream_t stream, const int8_t* operands, int32_t* out, int blocks, int iters);
-/* Calibration, no counterpart in the reference: blocks x 256 threads each run iters
- * times n_valu packed-fp16 vector instructions and n_mfma v_mfma_f32_16x16x32_f16 from
- * registers (dependent != 0: the MFMA operands come from the vector results of the same
- * iteration).  Instances: (52,0,0) (0,4,0) (52,4,0) (52,4,1) (26,4,1) (104,4,1) (0,8,0).
- * out receives blocks * 256 floats.  Used by bench.py --calibrate-issue to measure
- * whether vector and matrix instructions of the waves of one SIMD overlap. */
-int mh_issue_probe(mh_stream_t stream, float* out, int blocks, int iters, int n_valu, int n_mfma,
-                   int dependent);
-/* Calibration, no counterpart in the reference: `blocks` workgroups of 256 threads meet `rounds`
- * times at a device-wide barrier (agent-scope counters that only grow: counter[0] and, with groups > 1,
- * one per group at counter[32 * (1 + g)], 32 * 17 words zeroed by the caller; every wait gives up
- * after spin_limit polls and sets *error, after which no workgroup waits any more, so every wave
- * exits).  groups = 1: every workgroup arrives at counter[0]; groups = 8: per-XCD arrival, then one
- * arrival per group.  blocks must not exceed two per CU.  Used by bench.py
- * --calibrate-barrier to price a phase barrier of a persistent kernel against a kernel boundary
- * (mh_empty_probe: an empty launch of `blocks` workgroups). */
-int mh_grid_barrier_probe(mh_stream_t stream, unsigned* counter, unsigned* error, int blocks, int rounds,
-                          int spin_limit, int groups);
-int mh_empty_probe(mh_stream_t stream, unsigned* sink, int blocks);
-/* Calibration, no counterpart in the reference: reads `rows` packed rows of N 32-bit words with the
- * footprint of the small-M GPTQ kernel's weight stream (N / 256 x parts workgroups of four waves, a wave
- * load = four rows x 256 bytes, eight loads in flight per wave) and does nothing with them.  sink: 256
- * words, never written in practice.  Used by bench.py --calibrate-stream: the rate the memory system
- * delivers to that footprint. */
-int mh_weight_stream_probe(mh_stream_t stream, const uint32_t* words, uint32_t* sink, int rows, int N, int parts);
 /* out[n, k] = in[k, n]: one-time layout conversion for weights stored [K, N]. */
 int mh_i8_transpose(mh_stream_t stream, const int8_t* in, int8_t* out, int rows, int cols);
 

@@ -25,6 +25,10 @@ template <int MT, int NT>
 __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __restrict__ a,
                                                             const half_t* __restrict__ b,
                                                             half_t* __restrict__ out, int M, int N, int K) {
+    // blockIdx.z: the matrix of a batch (a [batch, M, K], b [batch, N, K], out [batch, M, N])
+    a += (size_t)blockIdx.z * M * K;
+    b += (size_t)blockIdx.z * N * K;
+    out += (size_t)blockIdx.z * M * N;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i16 = lane & 15, kq = lane >> 4;
     // a wave owns NT groups of 16 output columns: above 16 rows two groups share every
@@ -197,6 +201,9 @@ __global__ __launch_bounds__(512) void f16_gemv_nk_kernel(const half_t* __restri
 // Any K (no divisibility or alignment assumptions): one thread per output.
 __global__ void f16_matmul_nk_generic_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
                                              half_t* __restrict__ out, int M, int N, int K) {
+    a += (size_t)blockIdx.y * M * K;  // blockIdx.y: the matrix of a batch
+    b += (size_t)blockIdx.y * N * K;
+    out += (size_t)blockIdx.y * M * N;
     const size_t total = (size_t)M * N;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
@@ -278,6 +285,46 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     const int nt = mt == 1 ? 1 : 2;  // columns per wave: 16 or 32
     dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt));
+#define MH_DENSE(MT, NT)                                                                                            \
+    hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT>), grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, \
+                       (half_t*)out, M, N, K)
+    switch (mt) {
+        case 1: MH_DENSE(1, 1); break;
+        case 2: MH_DENSE(2, 2); break;
+        default: MH_DENSE(4, 2); break;
+    }
+#undef MH_DENSE
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
+// One launch for a batch of independent products: blockIdx.z (blockIdx.y of the generic kernel)
+// walks the matrices, each with the tiling of a single product.
+extern "C" int mh_f16_matmul_nk_batched(mh_stream_t stream, const void* a, const void* b, void* out, int batch,
+                                        int M, int N, int K) {
+    MH_REQUIRE(batch >= 0 && M >= 0 && N >= 0 && K >= 0, "mh_f16_matmul_nk_batched: bad shape batch=%d M=%d N=%d K=%d",
+               batch, M, N, K);
+    if (batch == 0 || M == 0 || N == 0) return MH_OK;
+    if (batch == 1) return mh_f16_matmul_nk(stream, a, b, out, M, N, K);
+    MH_REQUIRE(a && b && out, "mh_f16_matmul_nk_batched: null pointer");
+    MH_REQUIRE(batch <= 65535, "mh_f16_matmul_nk_batched: at most 65535 matrices per call, got %d", batch);
+    hipStream_t st = as_stream(stream);
+    // every matrix of the batch must start on a 16-byte boundary for the vector loads
+    const bool fast = K > 0 && K % 32 == 0 && ((uintptr_t)a | (uintptr_t)b) % 16 == 0 &&
+                      ((size_t)M * K * 2) % 16 == 0 && ((size_t)N * K * 2) % 16 == 0;
+    if (!fast) {
+        size_t blocks = ((size_t)M * N + 255) / 256;
+        const size_t cap = (size_t)compute_units() * 16;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(f16_matmul_nk_generic_kernel, dim3((unsigned)blocks, batch), dim3(256), 0, st,
+                           (const half_t*)a, (const half_t*)b, (half_t*)out, M, N, K);
+        MH_CHECK_LAUNCH();
+        return MH_OK;
+    }
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    const int nt = mt == 1 ? 1 : 2;
+    dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt), batch);
+    MH_REQUIRE(grid.y <= 65535, "mh_f16_matmul_nk_batched: M=%d is too large for one launch", M);
 #define MH_DENSE(MT, NT)                                                                                            \
     hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT>), grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, \
                        (half_t*)out, M, N, K)

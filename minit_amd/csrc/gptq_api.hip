@@ -79,8 +79,9 @@ __global__ void static_scratch_clear_kernel(uint4* p, int n16) {
     if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
-// The current device's copy of `scratch` (looked up on first use on that device).
-static int static_scratch_pointer(void** out) {
+// The current device's copy of `scratch` (looked up on first use on that device).  The lookup loads
+// the code object's symbol table: not something to do while `stream` is being captured.
+static int static_scratch_pointer(hipStream_t stream, void** out) {
     int dev = 0;
     MH_CHECK_HIP(hipGetDevice(&dev));
     MH_REQUIRE(dev >= 0 && dev < kStaticMaxDevices, "mh_gptq_matmul_static: device index %d out of range", dev);
@@ -88,6 +89,13 @@ static int static_scratch_pointer(void** out) {
     void* ptr = g_static_scratch[dev];
     hipError_t err = hipSuccess;
     if (ptr == nullptr) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (stream != nullptr && hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+            capturing != hipStreamCaptureStatusNone) {
+            pthread_mutex_unlock(&g_static_lock);
+            return fail(MH_ERR_INVALID, "mh_gptq_matmul_static: the first call on a device must be made outside a "
+                                        "stream capture (it looks up the built-in buffer's address)");
+        }
         err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (err == hipSuccess) g_static_scratch[dev] = ptr;
     }
@@ -119,7 +127,7 @@ int mh_gptq_matmul_static(mh_stream_t stream, const void* x, const int32_t* qwei
                     M, N, K, need, kStaticScratchBytes);
     void* ws = nullptr;
     if (need != 0) {
-        rc = static_scratch_pointer(&ws);
+        rc = static_scratch_pointer(as_stream(stream), &ws);
         if (rc) return rc;
         // the arrival counters must start at zero; the buffer keeps whatever the previous call (or a call
         // that was interrupted) left, so clear them with a kernel (no memset node, safe under graph capture)

@@ -768,7 +768,11 @@ static int env_int_gemm(const char* name, int fallback) {
 
 constexpr int kSmallMaxM = 32;     // rows of one launch with epilogues / norm fusion
 constexpr int kSmallBlockM = 64;   // rows per pass of a plain product above kSmallMaxM rows
-static const int kFusedReduceMaxM = env_int_gemm("MH_GEMM_FUSED_REDUCE_MAX_M", 8);
+// (an A/B switch; workspace sizes and the row-blocked path assume at most kSmallMaxM)
+static const int kFusedReduceMaxM = [] {
+    const int v = env_int_gemm("MH_GEMM_FUSED_REDUCE_MAX_M", 8);
+    return v < 1 ? 1 : v > kSmallMaxM ? kSmallMaxM : v;
+}();
 
 // Plan of the small-M kernel: column tiles x K splits sized so the GPU holds
 // about MH_GEMM_SMALL_WAVES_PER_CU waves per CU; a block walks whole stages.

@@ -490,34 +490,6 @@ __global__ __launch_bounds__(kI8Threads) void i8_gemm_k128_kernel(
     }
 }
 
-// Calibration: a register-resident stream of v_mfma_i32_32x32x32_i8 (eight
-// independent accumulators, operands read once from memory), to find what the
-// matrix pipe sustains on a given box with given operand values -- under dense
-// int8 work the part is power-limited and the rate depends on how many operand
-// bits toggle.
-__global__ __launch_bounds__(512) void i8_mfma_probe_kernel(const int4_t* __restrict__ operands, int32_t* __restrict__ out,
-                                                            int iters) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    int4_t a[4], b[2];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = operands[(size_t)t * 6 + i];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) b[i] = operands[(size_t)t * 6 + 4 + i];
-    int16_t_v c[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) c[j][i] = 0;
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) c[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j & 1], a[j >> 1], c[j], 0, 0, 0);
-    }
-    int32_t s = 0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) s += c[j][j];
-    out[t] = s;
-}
-
 // out[c, r] = in[r, c] through a 64 x 64 LDS tile.
 __global__ __launch_bounds__(256) void i8_transpose_kernel(const int8_t* __restrict__ in,
                                                            int8_t* __restrict__ out, int rows, int cols) {
@@ -593,15 +565,6 @@ int mh_i8_gemm(mh_stream_t stream, const int8_t* a, const int8_t* w, const float
         MH_I8_LAUNCH(1);
     }
 #undef MH_I8_LAUNCH
-    MH_CHECK_LAUNCH();
-    return MH_OK;
-}
-
-int mh_i8_mfma_probe(mh_stream_t stream, const int8_t* operands, int32_t* out, int blocks, int iters) {
-    MH_REQUIRE(operands && out && blocks > 0 && iters > 0, "mh_i8_mfma_probe: bad argument");
-    MH_REQUIRE((uintptr_t)operands % 16 == 0, "mh_i8_mfma_probe: operands must be 16-byte aligned");
-    hipLaunchKernelGGL(i8_mfma_probe_kernel, dim3(blocks), dim3(512), 0, as_stream(stream),
-                       reinterpret_cast<const int4_t*>(operands), out, iters);
     MH_CHECK_LAUNCH();
     return MH_OK;
 }

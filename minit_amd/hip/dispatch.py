@@ -85,16 +85,17 @@ def dispatch_matmul(op: MatrixMultiply, a: HIPTensor, b: HIPTensor):
 @register_dispatch()
 def dispatch_batch_matmul(op: BatchMatrixMultiply, a: HIPTensor, b: HIPTensor):
     # minit/cuda/dispatch.py:82-101: c[i] = a[i] @ b[i]^T for i < batch, b stored [batch, N, K];
-    # the reference hands the whole batch to one strided library call, here one launch per matrix
+    # one strided launch for the whole batch, like the reference's library call
     b0, m, k0 = a._shape
     b1, n, k1 = b._shape
     assert b0 == b1
     assert k0 == k1
     assert a.dtype == b.dtype == "float16"
     c = HIPTensor.allocate((b0, m, n), a.dtype)
-    for i in range(b0):
-        call("mh_f16_matmul_nk", None, a.data_ptr + i * m * k0 * 2, b.data_ptr + i * n * k0 * 2,
-             c.data_ptr + i * m * n * 2, m, n, k0)
+    for i0 in range(0, b0, 65535):   # the launch takes at most 65535 matrices
+        nb = min(65535, b0 - i0)
+        call("mh_f16_matmul_nk_batched", None, a.data_ptr + i0 * m * k0 * 2, b.data_ptr + i0 * n * k0 * 2,
+             c.data_ptr + i0 * m * n * 2, nb, m, n, k0)
     return (c,)
 
 

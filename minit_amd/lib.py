@@ -54,14 +54,10 @@ PROTOTYPES = {
     "mh_gptq_silu_pairs_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "mh_gptq_matmul_silu_pairs": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, c_size_t]),
     "mh_f16_matmul_nk": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
+    "mh_f16_matmul_nk_batched": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mh_i8_gemm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int]),
     "mh_i8_transpose": (c_int, [_P, _P, _P, c_int, c_int]),
-    "mh_i8_mfma_probe": (c_int, [_P, _P, _P, c_int, c_int]),
     "mh_gptq_permute_rows": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int]),
-    "mh_issue_probe": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int]),
-    "mh_grid_barrier_probe": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int]),
-    "mh_empty_probe": (c_int, [_P, _P, c_int]),
-    "mh_weight_stream_probe": (c_int, [_P, _P, _P, c_int, c_int, c_int]),
     "mh_rms_norm": (c_int, [_P, _P, _P, _P, c_size_t, c_size_t, c_size_t, c_double, c_int]),
     "mh_rope": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_size_t, c_size_t, c_size_t, c_int]),
     "mh_softmax": (c_int, [_P, _P, _P, c_size_t, c_size_t, c_size_t, c_int]),

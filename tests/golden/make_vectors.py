@@ -42,6 +42,17 @@ def round_fraction_to_f16(fr: Fraction) -> int:
     return f16_bits(as_double)
 
 
+def round_signed_sqrt_to_f16(sign: int, square: Fraction) -> float:
+    """The fp16 value nearest to sign * sqrt(square), decided exactly: the candidate from double
+    arithmetic is accepted only if the squares of the two midpoints to its fp16 neighbours
+    bracket `square` (compared as rationals)."""
+    cand = np.float16(float(square) ** 0.5)
+    lo = Fraction(float(np.nextafter(cand, np.float16(0)))) + Fraction(float(cand))
+    hi = Fraction(float(np.nextafter(cand, np.float16(np.inf)))) + Fraction(float(cand))
+    assert (lo / 2) ** 2 < square < (hi / 2) ** 2, "candidate is not the nearest fp16 value"
+    return sign * float(cand)
+
+
 def pack_words(values, bits):
     """values: list of 32 // bits sub-words -> one signed 32-bit word."""
     word = 0
@@ -107,6 +118,16 @@ def special_cases():
     cases["rms_norm_constant_rows"] = {
         "x": [[3.0] * 8, [-0.25] * 8], "weight": w, "eps": 1e-6,
         "out": [w, [-v for v in w]],
+    }
+    # RMSNorm where eps decides the answer: a constant row c with eps = c^2 normalises to sign(c) * w / sqrt(2),
+    # and c = 3 * 2^-10 with the same eps to w * 3 / sqrt(10); eps left out gives +-w, eps added outside the
+    # square root gives w * c / (|c| + eps) = 0.999 w.  out^2 = w^2 c^2 / (c^2 + eps), rounded to fp16 exactly.
+    c0, eps = Fraction(1, 1024), Fraction(1, 1 << 20)
+    rows = [c0, -c0, 3 * c0]
+    cases["rms_norm_eps_rows"] = {
+        "x": [[float(c)] * 8 for c in rows], "weight": w, "eps": float(eps),
+        "out": [[round_signed_sqrt_to_f16((1 if c > 0 else -1) * (1 if v > 0 else -1),
+                                          Fraction(v) ** 2 * c * c / (c * c + eps)) for v in w] for c in rows],
     }
     # softmax: uniform row of 8 -> 1/8; -inf entries -> exactly 0, the rest uniform
     ninf = "-inf"

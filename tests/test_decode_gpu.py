@@ -350,3 +350,47 @@ def test_large_residual_channels(hip, batch):
     dec2.load_host(model, k_cache, v_cache)
     _, got2 = dec2.decode(tokens, positions, 1, want_logits=True)
     assert np.isfinite(got2.astype(np.float64)).all(), "a saturated h * w must not turn the step into NaN"
+
+
+@pytest.mark.parametrize("batch", [2, 9])
+def test_norm_eps_in_the_fused_norms(hip, batch):
+    """A residual stream whose mean square is of the order of eps (embedding rows around 2^-10, eps
+    2^-20), kept that small through layer 0 by o and down weights equal to their zero point: eps
+    then decides layer 0's post-attention norm (residual epilogue of o -> prologue of gate|up) and
+    layer 1's input norm (epilogue of down -> prologue of q|k|v; at 9 rows both ride on the second
+    stage).  An eps outside the square root, or none, moves every normalised value by 30 to 40 %."""
+    from minit_amd.decode import LlamaDecoder
+    from oracle import gptq as OG
+    cfg = dict(CFG, hidden=1024, ffn=256, rms_eps=2.0 ** -20)
+    model = _host_model(cfg, seed=130 + batch)
+    rng = np.random.default_rng(1300 + batch)
+    model["embed"] = (rng.choice([-1.0, 1.0], model["embed"].shape) * rng.uniform(0.5, 1.5, model["embed"].shape)
+                      * 2.0 ** -10).astype(np.float16)
+    for name in ("o", "down"):   # q == z + 1: the projection is exactly zero
+        qw, qz, sc, g = model["layers"][0][name]
+        z = OG.unpack(qz, 1, 4)                                    # [K / g, N]
+        model["layers"][0][name] = (OG.pack(np.repeat(z + 1, g, axis=0).astype(np.uint8), 0, 4), qz, sc, g)
+    context, max_seq = 9, 64
+    shape = (batch, cfg["n_kv_heads"], max_seq, 128)
+    k_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    v_cache = [np.zeros(shape, np.float16) for _ in range(cfg["n_layers"])]
+    for c in k_cache + v_cache:
+        c[:, :, :context] = rng.normal(0, 1, (batch, cfg["n_kv_heads"], context, 128))
+    tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
+    positions = np.full(batch, context, np.int32)
+    dec = LlamaDecoder(cfg, batch, max_seq)
+    dec.load_host(model, k_cache, v_cache)
+    _, got = dec.decode(tokens, positions, 1, want_logits=True)
+    ref_k, ref_v = [c.copy() for c in k_cache], [c.copy() for c in v_cache]
+    ref = OD.decode_step(model, tokens, positions, ref_k, ref_v)
+    # the oracle with eps dropped must be far away, or this model would not test what it says
+    wrong = OD.decode_step(dict(model, config=dict(cfg, rms_eps=1e-12)), tokens, positions,
+                           [c.copy() for c in k_cache], [c.copy() for c in v_cache])
+    g, r = got.astype(np.float64), ref.astype(np.float64)
+    assert np.linalg.norm(wrong.astype(np.float64) - r) / np.linalg.norm(r) > 5e-2
+    assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
+    # layer 1's appended keys and values are linear in its input norm's output
+    kc, vc = dec.k_cache[1].numpy(), untile_v_cache(dec.v_cache[1].numpy())
+    for got_c, ref_c in ((kc, ref_k[1]), (vc, ref_v[1])):
+        a, b = got_c[:, :, context].astype(np.float64), ref_c[:, :, context].astype(np.float64)
+        assert np.linalg.norm(a - b) <= 1e-2 * np.linalg.norm(b)

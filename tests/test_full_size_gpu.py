@@ -78,6 +78,57 @@ def test_mistral_mlp_block(hip, mistral_weights, m):
     assert_fp16_close(y.numpy(), h_host.astype(np.float64) @ dense["down"], what=f"down M={m}")
 
 
+@pytest.mark.parametrize("m", [1, 8, 32, 128])
+def test_mistral_mlp_block_fused_entry_points(hip, mistral_weights, m):
+    """The same block through the two calls the benchmark times: mh_gptq_matmul_silu_pairs on
+    the interleaved gate|up weight (4096 -> 2 x 14336, SiLU*up inside the product: in the
+    reduction of the small-M kernel up to 32 rows, in the store of the 128-row blocks above),
+    then mh_gptq_matmul 14336 -> 4096, each stage against the float64 oracle."""
+    from minit_amd import synthetic
+    from minit_amd.decode import interleave_gate_up
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    host, dense = mistral_weights
+    hidden, ffn = 4096, 14336
+    x = synthetic.activations("cfg1", f"x{m}", (m, hidden))
+    fused = interleave_gate_up(*(np.concatenate([g, u], axis=1) for g, u in zip(host["gate"], host["up"])))
+    dq, dz, ds = (_dev(t) for t in fused)
+    dx = _dev(x)
+    h = HIPTensor.allocate((m, ffn), "float16")
+    ws = memory.workspace(max(hip.call("mh_gptq_silu_pairs_workspace_bytes", m, 2 * ffn, hidden, GROUP, BITS),
+                              hip.call("mh_gptq_workspace_bytes", m, hidden, ffn, GROUP, BITS), 256))
+    hip.call("mh_gptq_matmul_silu_pairs", None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, h.data_ptr,
+             m, 2 * ffn, hidden, GROUP, BITS, ws._pointer, ws._size)
+    h_host = h.numpy()
+    assert np.isfinite(h_host.astype(np.float64)).all()
+    x64 = x.astype(np.float64)
+    gate = (x64 @ dense["gate"]).astype(np.float16)
+    up = (x64 @ dense["up"]).astype(np.float16)
+    ref = O.silu_mul_f64(gate, up)
+    # gate and up are rounded to fp16 before the epilogue; the device's fp32 sums may round to the
+    # neighbouring fp16 value, which moves the result by |d silu / d gate| <= 1.1 times a step of
+    # gate times |up|, and by |silu(gate)| times a step of up
+    g64, u64 = gate.astype(np.float64), up.astype(np.float64)
+    step_h = fp16_spacing(ref)
+    # (sums that nearly cancel differ between fp32 and float64 accumulation by far more than their own
+    # fp16 spacing: an absolute term for that, `hidden` terms of unit size in fp32)
+    order = 4.0 * hidden * 2.0 ** -24
+    slack = (1.1 * np.abs(u64) * (fp16_spacing(gate) + order)
+             + np.abs(g64 / (1.0 + np.exp(-g64))) * (fp16_spacing(up) + order))
+    err = np.abs(h_host.astype(np.float64) - ref)
+    assert (err <= step_h + slack + 1e-7).all(), f"SiLU*up M={m}: worst {(err - slack).max():.4g}"
+    # and that allowance is the exception: nearly all outputs sit within one step of their own
+    share = float((err > step_h).mean())
+    assert share < 0.02, f"SiLU*up M={m}: {share:.2%} of the outputs needed the operand-step allowance"
+    assert np.linalg.norm(h_host.astype(np.float64) - ref) <= 1e-3 * np.linalg.norm(ref)
+
+    y = HIPTensor.allocate((m, hidden), "float16")
+    dd = tuple(_dev(t) for t in host["down"])
+    hip.call("mh_gptq_matmul", None, h.data_ptr, dd[0].data_ptr, dd[1].data_ptr, dd[2].data_ptr, None, y.data_ptr,
+             m, hidden, ffn, GROUP, BITS, ws._pointer, ws._size)
+    assert_fp16_close(y.numpy(), h_host.astype(np.float64) @ dense["down"], what=f"down after fused gate|up M={m}")
+
+
 LLAMA70B_LINEARS = [("qkv", 8192, 10240), ("o", 8192, 8192), ("gate_up", 8192, 57344), ("down", 28672, 8192)]
 
 

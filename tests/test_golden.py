@@ -66,6 +66,9 @@ def test_oracle_special_known_answers():
     c = s["rms_norm_constant_rows"]
     got = OS.rms_norm(np.asarray(c["x"], np.float16), np.asarray(c["weight"], np.float16), 1, c["eps"])
     np.testing.assert_array_equal(got, np.asarray(c["out"], np.float16))
+    c = s["rms_norm_eps_rows"]   # eps as large as the mean square: its place in the formula decides the answer
+    got = OS.rms_norm(np.asarray(c["x"], np.float16), np.asarray(c["weight"], np.float16), 1, c["eps"])
+    np.testing.assert_array_equal(got, np.asarray(c["out"], np.float16))
     c = s["softmax_rows"]
     np.testing.assert_array_equal(OS.softmax(_inf(c["x"]), 1), np.asarray(c["out"], np.float16))
     c = s["softmax_causal"]
@@ -143,6 +146,20 @@ def test_hip_special_known_answers(hip):
     c = s["rms_norm_constant_rows"]
     got = F.rms_norm(_t(np.asarray(c["x"], np.float16)), _t(np.asarray(c["weight"], np.float16)), 1, c["eps"]).numpy()
     np.testing.assert_array_equal(got, np.asarray(c["out"], np.float16))
+    c = s["rms_norm_eps_rows"]
+    x, w, ref = (np.asarray(c[key], np.float16) for key in ("x", "weight", "out"))
+    step = np.spacing(np.abs(ref)).astype(np.float64)
+    got = F.rms_norm(_t(x), _t(w), 1, c["eps"]).numpy()
+    assert (np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= step).all(), "mh_rms_norm: eps term"
+    # the same rows through the fused residual add + norm, without and with a delta that sums to the row
+    for delta in (None, x / 2):
+        h = _t(x if delta is None else x / 2)
+        d = None if delta is None else _t(np.ascontiguousarray(delta))
+        out, dw = HIPTensor.allocate(x.shape, "float16"), _t(w)
+        hip.call("mh_add_rms_norm", None, h.data_ptr, d.data_ptr if d else None, dw.data_ptr, out.data_ptr,
+                 x.shape[0], x.shape[1], c["eps"])
+        assert (np.abs(out.numpy().astype(np.float64) - ref.astype(np.float64)) <= step).all(), "mh_add_rms_norm: eps term"
+        np.testing.assert_array_equal(h.numpy(), x)
     c = s["softmax_rows"]
     np.testing.assert_array_equal(F.softmax(_t(_inf(c["x"])), 1).numpy(), np.asarray(c["out"], np.float16))
     c = s["softmax_causal"]

@@ -351,7 +351,8 @@ def test_operator_api_drop_in(hip):
 
 
 @pytest.mark.parametrize("m,k,ffn", [(1, 512, 256), (3, 1024, 384), (8, 256, 128), (16, 512, 256), (32, 768, 512),
-                                     (40, 512, 256),     # 33 to 64 rows: product, then one pass
+                                     (40, 512, 256),     # 33 to 64 rows, K >= 512: one block of 64 rows, SiLU*up in its store
+                                     (40, 384, 256), (64, 256, 128),      # ... K < 512: product, then one pass
                                      (130, 1024, 384), (200, 512, 640),   # 128-row blocks, SiLU*up in their store
                                      (128, 4096, 512)])  # ... K split over workgroups: product, then one pass
 def test_silu_pairs_epilogue(hip, m, k, ffn):

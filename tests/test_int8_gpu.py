@@ -42,6 +42,17 @@ def test_i8_gemm_bit_exact(hip, m, n, k):
     np.testing.assert_array_equal(out.view(np.uint16), ref_out.view(np.uint16))
 
 
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 4096), (130, 260, 192)])
+def test_i8_gemm_fp16_output_only(hip, m, n, k):
+    """acc_i32 == NULL, the call the benchmark times: the fp16 output alone, bit for bit."""
+    from minit_amd import synthetic
+    a, w, a_scale, w_scale = synthetic.int8_operands(f"i8-{m}-{n}-{k}", m, n, k)
+    out, acc = _run(hip, a, w, a_scale, w_scale, want_acc=False)
+    assert acc is None
+    ref_out, _ = O.gemm(a, w, a_scale, w_scale)
+    np.testing.assert_array_equal(out.view(np.uint16), ref_out.view(np.uint16))
+
+
 def _sweep(count, seed):
     rng = np.random.default_rng(seed)
     return [(int(rng.integers(1, 400)), int(rng.integers(1, 700)), 64 * int(rng.integers(1, 13)))

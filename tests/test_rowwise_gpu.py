@@ -221,3 +221,29 @@ def test_batch_matrix_multiply(hip):
     assert got.shape == (2, 3, 5, 40)
     ref = np.einsum("bhsd,bhtd->bhst", a.astype(np.float64), b.astype(np.float64))
     assert_fp16_close(got.reshape(-1, 40), ref.reshape(-1, 40), what="batched nk")
+
+
+@pytest.mark.parametrize("batch,m,n,k", [(6, 5, 40, 128),      # q.k^T of a short prefill, one 16-row tile
+                                         (64, 70, 70, 128),    # 64 heads, four row tiles, ragged
+                                         (3, 33, 129, 64),     # two row tiles, ragged columns
+                                         (4, 7, 9, 20),        # K not a multiple of 32: the generic kernel
+                                         (1, 12, 300, 96)])    # a batch of one
+def test_batched_dense_product_is_one_launch_per_batch(hip, batch, m, n, k):
+    """mh_f16_matmul_nk_batched against the oracle's dense product matrix by matrix, and bit for bit
+    against the same matrices through mh_f16_matmul_nk one by one."""
+    from minit_amd.hip.tensor import HIPTensor
+    rng = np.random.default_rng(batch * 1000 + m)
+    a = rng.normal(0, 1, size=(batch, m, k)).astype(np.float16)
+    b = rng.normal(0, 0.2, size=(batch, n, k)).astype(np.float16)
+    da, db = _t(a), _t(b)
+    out = HIPTensor.allocate((batch, m, n), "float16")
+    hip.call("mh_f16_matmul_nk_batched", None, da.data_ptr, db.data_ptr, out.data_ptr, batch, m, n, k)
+    got = out.numpy()
+    one = HIPTensor.allocate((m, n), "float16")
+    for i in range(batch):
+        ref = OG.dense_matmul(a[i], np.ascontiguousarray(b[i].T))
+        assert_fp16_close(got[i], ref.astype(np.float64), what=f"batched nk, matrix {i}")
+        if k % 32 == 0 and m <= 64:   # same kernel, same tiling: same bits
+            hip.call("mh_f16_matmul_nk", None, da.data_ptr + i * m * k * 2, db.data_ptr + i * n * k * 2,
+                     one.data_ptr, m, n, k)
+            np.testing.assert_array_equal(one.numpy().view(np.uint16), got[i].view(np.uint16))
