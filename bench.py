@@ -585,6 +585,35 @@ def main():
             cached[name] = {"us": round(us, 2), "gbps": round(linear_bytes(1, k, n) / us / 1e3, 1),
                             "weight_mb": round(linear_bytes(1, k, n) / 1e6, 1)}
         result["extra"] = {"gemv_per_shape": per_shape, "gemv_per_shape_cache_resident": cached}
+        # What the launch boundaries cost: the same step with its four launches alternated over two
+        # streams (a workspace each).  The four products of the benchmark step do not depend on each
+        # other, so the launches overlap freely, which the products of a decode layer cannot: a figure
+        # for comparison, not a way the hot path is run.
+        two = [memory.create_stream() for _ in range(2)]
+        ws2 = [memory.HIPMemory(max(ws_bytes, 256)) for _ in range(2)]
+        for mem in ws2:
+            mem.reset()
+        memory.synchronize()
+
+        def step_two_streams(i):
+            for j, lin in enumerate(layers[i % args.layers]):
+                t = (i * len(LINEARS) + j) & 1
+                lib.call(ENTRY, two[t], xs[lin.k].data_ptr, lin.qweight.data_ptr, lin.qzeros.data_ptr,
+                         lin.scales.data_ptr, None, outs[lin.n].data_ptr, 1, lin.n, lin.k, GROUP, BITS,
+                         ws2[t]._pointer, ws2[t]._size)
+        for i in range(200):
+            step_two_streams(i)
+        memory.synchronize()
+        t0 = time.perf_counter()
+        for i in range(1000):
+            step_two_streams(i)
+        memory.synchronize()
+        two_us = (time.perf_counter() - t0) * 1e3
+        for st in two:
+            lib.call("mh_stream_destroy", st)
+        result["extra"]["gemv_step_two_independent_streams"] = {
+            "us": round(two_us, 2), "gbps": round(step_bytes / two_us / 1e3, 1),
+            "note": "host clock around 1000 steps; launches of a step overlap, which dependent products cannot"}
         if not args.shapes_only:
             # the same four shapes on 8-bit weights (the bit width the reference's own example ships,
             # examples/qwen1_5_int8.py): half the arithmetic per byte
