@@ -295,7 +295,9 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  * pointers are device pointers owned by the caller.
  *   qkv      fused q|k|v projection, GPTQ, [hidden] -> [(QH + 2 KVH) * D]
  *   gate_up  fused gate|up projection, [hidden] -> [2 * ffn], columns interleaved in
- *            blocks of 128 gate / 128 up as for mh_gptq_matmul_silu_pairs (ffn % 128 == 0)
+ *            blocks of 128 gate / 128 up as for mh_gptq_matmul_silu_pairs (ffn % 128 == 0);
+ *            the activation is silu(gate) * up (for examples/qwen1_5_int8.py:376-385 gate is w2
+ *            and up is w1)
  *   k_cache  fp16 [batch_max, KVH, max_seq, D], v_cache fp16 [batch_max, KVH, max_seq / 64, D, 64]
  *            (V is kept with positions contiguous, in tiles of 64, for the P.V matrix product:
  *            value d of position p sits at ((p / 64) * D + d) * 64 + p % 64 of its row and KV
@@ -341,10 +343,19 @@ typedef struct {
     int group_size, bits, max_seq;
     float rms_eps;
 } mh_llama_config;
+/* One quantized linear of the model.  bias: fp16 [N] or NULL, added to the fp16-rounded product before
+ * anything else sees it (QLinearWithBias.forward, examples/qwen1_5_int8.py:311-317; every linear of that
+ * file's model has one); for gate_up it is interleaved like the columns.  perm: NULL for sequential
+ * groups; for an act-order checkpoint (g_idx a permutation, :283-285) the caller sorts the rows of
+ * qweight by group once at load time (mh_gptq_permute_rows) and passes the row order here, int32 [K]
+ * with row j of qweight = row perm[j] of the checkpoint's: the loop then gathers the activations into
+ * that order (mh_gather_columns) in front of the product. */
 typedef struct {
     const int32_t* qweight;
     const int32_t* qzeros;
     const void* scales;
+    const void* bias;
+    const int32_t* perm;
 } mh_qlinear;
 typedef struct {
     mh_qlinear qkv, o, gate_up, down;

@@ -475,6 +475,7 @@ struct Llama {
 
 struct Scratch {
     half_t *h, *xn, *qkv, *q, *attn, *delta, *gu, *act, *logits;
+    half_t* gathered;  // activations in the row order of an act-order weight (mh_qlinear::perm)
     float* attn_partial;
     float *ssq_a, *ssq_b;  // per-piece sums of squares of the residual stream, [batch, at most hidden / 32]
     int32_t* pos_base;     // positions at the start of a call that replays a recorded step
@@ -554,6 +555,12 @@ static Scratch carve(const Llama& m, int batch, char* base) {
     s.gu = (half_t*)take((size_t)batch * 2 * c.ffn * 2);
     s.act = (half_t*)take((size_t)batch * c.ffn * 2);
     s.logits = (half_t*)take((size_t)batch * c.vocab * 2);
+    {
+        size_t widest = (size_t)c.hidden;
+        if ((size_t)c.n_q_heads * c.head_dim > widest) widest = (size_t)c.n_q_heads * c.head_dim;
+        if ((size_t)c.ffn > widest) widest = (size_t)c.ffn;
+        s.gathered = (half_t*)take((size_t)batch * widest * 2);
+    }
     s.attn_partial = (float*)take((size_t)batch * c.n_q_heads * attn_splits(m, batch) * (c.head_dim + 4) * 4);
     s.ssq_a = (float*)take((size_t)batch * ((c.hidden + 31) / 32) * 4);
     s.ssq_b = (float*)take((size_t)batch * ((c.hidden + 31) / 32) * 4);
@@ -746,7 +753,17 @@ static int decode_impl(void* handle, mh_stream_t stream, int batch, int32_t* tok
     const unsigned ew_grid = (unsigned)compute_units() * 4;
     const bool fused_silu = gemm_silu_pairs_supported(batch, 2 * c.ffn, c.hidden, c.group_size, c.bits);
 
+    // activations of a linear whose rows were sorted by group at load time: gathered into that order
+    auto ordered = [&](const half_t* x, const mh_qlinear& w, int k) -> const half_t* {
+        if (w.perm == nullptr) return x;
+        (void)mh_gather_columns(stream, x, w.perm, s.gathered, (size_t)batch, (size_t)k, MH_F16);
+        return s.gathered;
+    };
     auto linear = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k) -> int {
+        x = ordered(x, w, k);
+        if (w.bias != nullptr)
+            return mh_gptq_linear(stream, x, w.qweight, w.qzeros, w.scales, nullptr, w.bias, y, batch, n, k,
+                                  c.group_size, c.bits, s.gptq_ws, s.gptq_ws_bytes);
         return gptq_matmul_dispatch(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
                                     s.gptq_ws, s.gptq_ws_bytes);
     };
@@ -763,9 +780,10 @@ static int decode_impl(void* handle, mh_stream_t stream, int batch, int32_t* tok
     const int o_pieces = gemm_residual_ssq_pieces(batch, c.hidden, c.n_q_heads * c.head_dim, c.group_size, c.bits);
     const int down_pieces = gemm_residual_ssq_pieces(batch, c.hidden, c.ffn, c.group_size, c.bits);
     auto fused = [&](const half_t* x, const mh_qlinear& w, half_t* y, int n, int k, int epilogue,
-                     const SmallFuse& fuse) -> int {
-        return gptq_matmul_fused(st, x, w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size, c.bits,
-                                 s.gptq_ws, s.gptq_ws_bytes, epilogue, fuse);
+                     SmallFuse fuse) -> int {
+        fuse.bias = (const half_t*)w.bias;
+        return gptq_matmul_fused(st, ordered(x, w, k), w.qweight, w.qzeros, w.scales, y, batch, n, k, c.group_size,
+                                 c.bits, s.gptq_ws, s.gptq_ws_bytes, epilogue, fuse);
     };
 
     // every launch of one step; out_row / pos_base as for argmax_advance_kernel
@@ -834,9 +852,7 @@ static int decode_impl(void* handle, mh_stream_t stream, int batch, int32_t* tok
             hipLaunchKernelGGL(add_rms_norm_kernel, dim3(batch), dim3(256), 0, st, s.h, s.delta,
                                (const half_t*)L.post_norm, s.xn, c.hidden, c.rms_eps);
             if (fused_silu) {
-                rc = gptq_matmul_silu_pairs(st, s.xn, L.gate_up.qweight, L.gate_up.qzeros, L.gate_up.scales, s.act,
-                                            batch, 2 * c.ffn, c.hidden, c.group_size, c.bits, s.gptq_ws,
-                                            s.gptq_ws_bytes);
+                rc = fused(s.xn, L.gate_up, s.act, 2 * c.ffn, c.hidden, kEpilogueSiluPairs, SmallFuse{});
                 if (rc) return rc;
             } else {
                 rc = linear(s.xn, L.gate_up, s.gu, 2 * c.ffn, c.hidden);

@@ -164,8 +164,9 @@ struct SmallFuse {
     float* ssq_out = nullptr;             // [M, pieces]: kEpilogueResidual
     const half_t* next_norm_w = nullptr;  // [N]
     half_t* xw_out = nullptr;             // [M, N]
-    // plain products only: out[m, n] = fp16(fp16(y[m, n]) + bias[n]), the two roundings of the
-    // reference's product followed by `output += bias` (examples/qwen1_5_int8.py:311-317)
+    // y[m, n] = fp16(fp16(y[m, n]) + bias[n]), the two roundings of the reference's product followed by
+    // `output += bias` (examples/qwen1_5_int8.py:311-317), before any epilogue (the activation of
+    // kEpilogueSiluPairs, the rotation, the residual add) sees y
     const half_t* bias = nullptr;         // [N]
     // kEpilogueRopeAppend
     const float* rope_cos = nullptr;  // [T, 64]

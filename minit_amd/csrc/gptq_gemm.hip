@@ -641,9 +641,15 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 const float* p = partial + (size_t)m * N + tile * kGemmCols + c4;
                 float4_t g, u;
                 sum_splits2(p, p + kGemmCols / 2, g, u);
+                half4_t gh = {(half_t)g[0], (half_t)g[1], (half_t)g[2], (half_t)g[3]};
+                half4_t uh = {(half_t)u[0], (half_t)u[1], (half_t)u[2], (half_t)u[3]};
+                if (fuse.bias) {  // the bias of the gate and of the up projection, before the activation
+                    gh = gh + *reinterpret_cast<const half4_t*>(fuse.bias + tile * kGemmCols + c4);
+                    uh = uh + *reinterpret_cast<const half4_t*>(fuse.bias + tile * kGemmCols + kGemmCols / 2 + c4);
+                }
                 half4_t h;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
+                for (int e = 0; e < 4; ++e) h[e] = silu_pair(gh[e], uh[e]);
                 *reinterpret_cast<half4_t*>(out + (size_t)m * (N / 2) + tile * (kGemmCols / 2) + c4) = h;
             }
             return;
@@ -666,7 +672,8 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                     }
                 }
                 const float4_t sum = sum_splits(partial + (size_t)m * N + c);
-                const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + c);
                 if (!rotated) {  // value head: copied, cache is tiled
                     half_t* dst = fuse.vt_cache + ((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 * fuse.max_seq +
                                   vt_offset(d, pos);
@@ -702,7 +709,8 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                     half4_t nw = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
                     if (fuse.xw_out) nw = *reinterpret_cast<const half4_t*>(fuse.next_norm_w + c);
                     const float4_t s = sum_splits(partial + (size_t)m * N + c);
-                    const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+                    half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+                    if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + c);
                     const half4_t h = h_old + y;  // fp16 add, one rounding
                     *reinterpret_cast<half4_t*>(hp) = h;
                     if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) = norm_weighted(h, nw);

@@ -336,7 +336,8 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         sum.x *= inv;
         sum.y *= inv;
     }
-    const half2_t y = {(half_t)sum.x, (half_t)sum.y};
+    half2_t y = {(half_t)sum.x, (half_t)sum.y};
+    if (fuse.bias) y = y + *reinterpret_cast<const half2_t*>(fuse.bias + col);  // before any epilogue
     half2_t* op = reinterpret_cast<half2_t*>(out + (size_t)m * N + col);
     if (epilogue == kEpilogueResidual) {
         // out is the residual stream: h += y in fp16, h * next_norm_w for the consumer,
@@ -371,7 +372,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         *reinterpret_cast<half2_t*>(dst) = o;
         return;
     }
-    *op = fuse.bias ? y + *reinterpret_cast<const half2_t*>(fuse.bias + col) : y;
+    *op = y;
 }
 
 bool gemm_cols_supported(int M, int N, int K, int group_size, int bits, int epilogue) {

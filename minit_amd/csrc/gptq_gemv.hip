@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __res
 // The same with the SiLU-pair epilogue: out is [M, N / 2].
 __global__ __launch_bounds__(256) void splitk_finalize_silu_kernel(const float* __restrict__ partial,
                                                                    half_t* __restrict__ out, int M, int N,
-                                                                   int split_k) {
+                                                                   int split_k, const half_t* __restrict__ bias) {
     const size_t half_n = (size_t)N / 2;
     const size_t o = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (o >= (size_t)M * half_n) return;
@@ -191,9 +191,15 @@ __global__ __launch_bounds__(256) void splitk_finalize_silu_kernel(const float* 
         g += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + gate);
         u += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + gate + 128);
     }
+    half4_t gh = {(half_t)g[0], (half_t)g[1], (half_t)g[2], (half_t)g[3]};
+    half4_t uh = {(half_t)u[0], (half_t)u[1], (half_t)u[2], (half_t)u[3]};
+    if (bias) {  // column of the gate sum within its row: gate - m * N
+        gh = gh + *reinterpret_cast<const half4_t*>(bias + (gate - m * N));
+        uh = uh + *reinterpret_cast<const half4_t*>(bias + (gate - m * N) + 128);
+    }
     half4_t h;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) h[e] = silu_pair((half_t)g[e], (half_t)u[e]);
+    for (int e = 0; e < 4; ++e) h[e] = silu_pair(gh[e], uh[e]);
     *reinterpret_cast<half4_t*>(out + o) = h;
 }
 
@@ -207,7 +213,8 @@ __global__ __launch_bounds__(256) void splitk_finalize_residual_kernel(const flo
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;  // within one row: N % 1024 == 0
     float4_t s = {0.f, 0.f, 0.f, 0.f};
     for (int sp = 0; sp < split_k; ++sp) s += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
-    const half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+    half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
+    if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + i % N);
     const half4_t r = *reinterpret_cast<const half4_t*>(h + i) + y;  // fp16 add, one rounding
     *reinterpret_cast<half4_t*>(h + i) = r;
     if (fuse.xw_out)
@@ -228,8 +235,9 @@ __global__ __launch_bounds__(256) void splitk_finalize_rope_kernel(const float* 
     if (i >= mn) return;
     float4_t sum = {0.f, 0.f, 0.f, 0.f};
     for (int sp = 0; sp < split_k; ++sp) sum += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
-    const half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+    half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
     const int m = (int)(i / N), c = (int)(i % N);
+    if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + c);
     const int head = c / 128, d = c % 128;
     const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
     if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is tiled
@@ -270,7 +278,7 @@ void launch_splitk_finalize(hipStream_t stream, const float* partial, void* out,
     if (epilogue == kEpilogueSiluPairs) {
         const size_t threads = ((size_t)M * (N / 2) + 3) / 4;
         hipLaunchKernelGGL(splitk_finalize_silu_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
-                           stream, partial, (half_t*)out, M, N, split_k);
+                           stream, partial, (half_t*)out, M, N, split_k, fuse.bias);
         return;
     }
     const size_t mn = (size_t)M * N;

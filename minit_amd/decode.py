@@ -22,7 +22,8 @@ class LlamaConfig(ctypes.Structure):
 
 
 class QLinear(ctypes.Structure):
-    _fields_ = [("qweight", c_void_p), ("qzeros", c_void_p), ("scales", c_void_p)]
+    _fields_ = [("qweight", c_void_p), ("qzeros", c_void_p), ("scales", c_void_p), ("bias", c_void_p),
+                ("perm", c_void_p)]
 
 
 class LlamaLayer(ctypes.Structure):
@@ -146,8 +147,9 @@ class LlamaDecoder:
         return kc, vc
 
     def _set_layer(self, index, linears, input_norm, post_norm, k_cache, v_cache):
-        def ql(t):
-            return QLinear(t[0].data_ptr, t[1].data_ptr, t[2].data_ptr)
+        def ql(t):   # (qweight, qzeros, scales[, bias[, perm]]); None where absent
+            extra = [e.data_ptr if e is not None else None for e in t[3:5]] + [None, None]
+            return QLinear(t[0].data_ptr, t[1].data_ptr, t[2].data_ptr, extra[0], extra[1])
         layer = LlamaLayer(ql(linears["qkv"]), ql(linears["o"]), ql(linears["gate_up"]), ql(linears["down"]),
                            input_norm.data_ptr, post_norm.data_ptr, k_cache.data_ptr, v_cache.data_ptr)
         lib.call("mh_llama_set_layer", self._handle, index, ctypes.byref(layer))
@@ -208,11 +210,33 @@ class LlamaDecoder:
 
     def load_host(self, model: dict, k_cache=None, v_cache=None):
         """Uploads a model given as numpy arrays (the layout of ``oracle.decode``)."""
+        from .quantize import gptq as host_gptq
+        bits, group = self.config["bits"], self.config["group_size"]
         for l, layer in enumerate(model["layers"]):
-            host = {name: layer[name][:3] for name in ("qkv", "o", "gate_up", "down")}
-            host["gate_up"] = interleave_gate_up(*host["gate_up"], bits=self.config["bits"])
-            linears = {name: tuple(HIPTensor.from_numpy(np.ascontiguousarray(a)) for a in host[name])
-                       for name in ("qkv", "o", "gate_up", "down")}
+            linears = {}
+            for name in ("qkv", "o", "gate_up", "down"):
+                # (qweight, qzeros, scales, group_size[, bias[, g_idx]]): the buffers of the reference's
+                # QLinear / QLinearWithBias (examples/qwen1_5_int8.py:276-305)
+                w = layer[name]
+                qweight, qzeros, scales = w[:3]
+                bias = w[4] if len(w) > 4 else None
+                g_idx = w[5] if len(w) > 5 else None
+                perm = None
+                if g_idx is not None and not np.array_equal(np.asarray(g_idx), np.arange(len(g_idx)) // group):
+                    # act-order: rows sorted by group once, here on the host; the loop gathers the activations
+                    res = host_gptq.sort_rows_by_group(qweight, np.asarray(g_idx), bits, group)
+                    assert res is not None, f"{name}: groups of uneven size are not served by the decode loop"
+                    qweight, perm = res
+                if name == "gate_up":
+                    cols_before = qweight.shape[1]
+                    qweight, qzeros, scales = interleave_gate_up(qweight, qzeros, scales, bits=bits)
+                    if bias is not None:   # the same column order
+                        ffn = cols_before // 2
+                        bias = np.stack([bias[:ffn].reshape(-1, 128), bias[ffn:].reshape(-1, 128)], axis=1).reshape(-1)
+                dev = [HIPTensor.from_numpy(np.ascontiguousarray(a)) for a in (qweight, qzeros, scales)]
+                dev.append(None if bias is None else HIPTensor.from_numpy(np.ascontiguousarray(bias, np.float16)))
+                dev.append(None if perm is None else HIPTensor.from_numpy(np.ascontiguousarray(perm, np.int32)))
+                linears[name] = tuple(dev)
             kc, vc = self._alloc_cache()
             if k_cache is not None:   # host caches are [B, KVH, T, D] with T <= max_seq
                 t = k_cache[l].shape[2]

@@ -9,6 +9,9 @@ single new token), softmax, P.V, output projection, residual adds in fp16,
 ``silu(gate) * up`` with its three roundings, and the lm_head product against
 ``[vocab, hidden]``; sampling is ``argmax`` (minit/chat/sample.py:11-14).
 
+Every linear may carry a bias and an act-order ``g_idx`` (the reference's own GPTQ model,
+examples/qwen1_5_int8.py:311-385, where gate is ``w2`` and up is ``w1``).
+
 Grouped-query attention: query head j uses KV head ``j // (QH / KVH)``
 (the reference repeats each KV head, llama3_70b.py:85-93).
 
@@ -21,10 +24,25 @@ import numpy as np
 from . import gptq, special
 
 
+def split_linear(w):
+    """``w`` is ``(qweight, qzeros, scales, group_size[, bias[, g_idx]])``: the buffers of the reference's
+    QLinear / QLinearWithBias (examples/qwen1_5_int8.py:276-305); ``bias`` and ``g_idx`` may be None."""
+    qweight, qzeros, scales, group_size = w[:4]
+    bias = w[4] if len(w) > 4 else None
+    g_idx = w[5] if len(w) > 5 else None
+    return qweight, qzeros, scales, group_size, bias, g_idx
+
+
+def add_bias(y, bias):
+    """``output += bias`` of QLinearWithBias.forward (examples/qwen1_5_int8.py:311-317): an fp16 add of the
+    fp16 product and the bias broadcast over the rows, one more rounding."""
+    return y if bias is None else (y + bias[None, :].astype(y.dtype))
+
+
 def _linear(x, w, bits=4):
-    """``w`` is ``(qweight, qzeros, scales, group_size)``."""
-    qweight, qzeros, scales, group_size = w
-    return gptq.matmul(x, qweight, qzeros, scales, None, bits, group_size)
+    """The quantized linear of the model code: the product (act-order ``g_idx`` included), then the bias."""
+    qweight, qzeros, scales, group_size, bias, g_idx = split_linear(w)
+    return add_bias(gptq.matmul(x, qweight, qzeros, scales, g_idx, bits, group_size), bias)
 
 
 def attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, positions: np.ndarray) -> np.ndarray:

@@ -330,3 +330,68 @@ def test_greedy_feeds_tokens_and_positions_back():
             assert out[step, b] == t
         written = np.abs(k[0][b].astype(np.float32)).sum(axis=(0, 2)) > 0
         assert written.tolist() == [pos[b] <= s < pos[b] + 4 for s in range(32)]
+
+
+# ------------------------------------------------------------------ biases and act-order (examples/qwen1_5_int8.py:276-385)
+
+def test_biases_are_added_to_the_rounded_product_in_fp16():
+    """o and down exactly zero but biased: the residual stream is embed + b_o + b_down, two fp16 adds; a
+    biased q|k|v that selects nothing appends k = RoPE(b_k) and v = b_v."""
+    rng = np.random.default_rng(21)
+    b_qkv = rng.normal(0, 1, (QH + 2 * KVH) * D).astype(np.float16)
+    b_o = rng.normal(0, 1, H).astype(np.float16)
+    b_down = rng.normal(0, 1, H).astype(np.float16)
+    model = _model(rng, qkv=_zeros(H, (QH + 2 * KVH) * D) + (b_qkv,), o=_zeros(QH * D, H) + (b_o,),
+                   down=_zeros(FFN, H) + (b_down,))
+    tokens, positions = np.array([5, 9]), np.array([0, 3])
+    k, v = _caches(rng, 2)
+    logits = OD.decode_step(model, tokens, positions, k, v)
+    for b, t in enumerate(tokens):
+        h = _add16(_add16(model["embed"][t], b_o), b_down)
+        np.testing.assert_array_equal(logits[b], _logits_from_hidden(h))
+        p = int(positions[b])
+        np.testing.assert_array_equal(v[0][b, :, p].reshape(-1), b_qkv[(QH + KVH) * D:])
+        want_k = OS.rope(b_qkv[QH * D:(QH + KVH) * D].reshape(1, 1, KVH, D), model["cos"], model["sin"],
+                         np.array([[p]]))[0, 0]
+        np.testing.assert_array_equal(k[0][b, :, p], want_k)
+
+
+def test_gate_and_up_biases_enter_before_the_activation():
+    """gate|up exactly zero with biases (b_gate, b_up), down the identity: h = embed + silu(b_gate) * b_up
+    with the three fp16 roundings of the models' silu (sigmoid, times the gate, times up)."""
+    rng = np.random.default_rng(22)
+    b_gate, b_up = rng.normal(0, 1, FFN).astype(np.float16), rng.normal(0, 1, FFN).astype(np.float16)
+    model = _model(rng, o=_zeros(QH * D, H), gate_up=_zeros(H, 2 * FFN) + (np.concatenate([b_gate, b_up]),),
+                   down=_eye(H))
+    tokens, positions = np.array([2, 30]), np.array([1, 6])
+    k, v = _caches(rng, 2)
+    logits = OD.decode_step(model, tokens, positions, k, v)
+    act = OG.silu_mul(b_gate, b_up)
+    for b, t in enumerate(tokens):
+        np.testing.assert_array_equal(logits[b], _logits_from_hidden(_add16(model["embed"][t], act)))
+
+
+def test_act_order_rows_take_the_scale_and_zero_point_of_their_own_group():
+    """A linear with a permuted g_idx (row k belongs to group g_idx[k]) against the dense product written
+    out from the unpacked tensors, and invariance: the same rows listed group by group with a sequential
+    g_idx, fed the activations in that order, give the same numbers."""
+    rng = np.random.default_rng(23)
+    k_dim, n = 2 * G, 24
+    q = rng.integers(0, 16, (k_dim, n)).astype(np.uint8)
+    z = rng.integers(0, 16, (k_dim // G, n)).astype(np.uint8)
+    s = (rng.uniform(0.01, 0.05, (k_dim // G, n))).astype(np.float16)
+    g_idx = rng.permutation(np.arange(k_dim) // G).astype(np.int32)
+    bias = rng.normal(0, 1, n).astype(np.float16)
+    x = rng.normal(0, 1, (3, k_dim)).astype(np.float16)
+    w = (OG.pack(q, 0, 4), OG.pack(z, 1, 4), s, G, bias, g_idx)
+    got = OD._linear(x, w)
+    dense = np.empty((k_dim, n), np.float64)
+    for r in range(k_dim):
+        g = g_idx[r]
+        dense[r] = ((q[r].astype(np.float64) - (z[g].astype(np.float64) + 1)) * s[g].astype(np.float64)).astype(np.float16)
+    want = _add16((x.astype(np.float64) @ dense).astype(np.float16), np.broadcast_to(bias, (3, n)))
+    np.testing.assert_array_equal(got, want)
+    perm = np.argsort(g_idx, kind="stable")
+    sorted_w = (OG.pack(q[perm], 0, 4), w[1], s, G, bias, None)
+    same = OD._linear(np.ascontiguousarray(x[:, perm]), sorted_w)
+    assert np.abs(same.astype(np.float64) - got.astype(np.float64)).max() <= 2 * np.spacing(np.abs(got).max())
