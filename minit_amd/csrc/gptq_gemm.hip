@@ -244,8 +244,13 @@ constexpr int kSmallDepth = 8;  // steps per stage = ring depth
 // of its own.
 // STREAM: the balanced plan described below (it costs registers: a second set of
 // accumulators), otherwise only the regular one.
-template <int BITS, int MT, int SPG, bool NORM, bool STREAM>
-__global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
+// KW: K shares inside the workgroup.  With KW = 2 the workgroup has eight waves, two sets of four that
+// walk consecutive K ranges of the same column tile, each with its own staged activations and constants,
+// and add their sums through LDS at the end: where the column tiles alone nearly fill the GPU (one
+// workgroup per CU, two waves per SIMD) a tile then needs no partial sums from another workgroup, so up
+// to 32 rows finish -- epilogue included -- inside the launch, without a second stage.
+template <int BITS, int MT, int SPG, bool NORM, bool STREAM, int KW = 1>
+__global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
     const half_t* __restrict__ x_all, const uint32_t* __restrict__ qweight,
     const uint32_t* __restrict__ qzeros, const half_t* __restrict__ scales,
     half_t* out_all, float* partial_all, unsigned* counters,
@@ -274,11 +279,15 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     constexpr int XL = BM * XCH / 256;      // chunks each thread stages: 2 (MT=1) or 4 (MT=2)
     static_assert(D % SPG == 0, "a stage must hold whole groups");
 
-    __shared__ uint4 xs[2][BM * RS];
-    __shared__ uint32_t cs[2][GPS][3][kGemmCols];  // scale pair, zero_lo pair, zero_hi pair
+    static_assert(KW == 1 || (KW == 2 && !STREAM), "one or two K shares; the balanced plan has one");
+    constexpr int NT = 256 * KW;  // threads of the workgroup
+    __shared__ uint4 xs_all[2][KW][BM * RS];
+    __shared__ uint32_t cs_all[2][KW][GPS][3][kGemmCols];  // scale pair, zero_lo pair, zero_hi pair
     __shared__ float inv_rms_s[NORM ? BM : 1];
 
-    const int tid = threadIdx.x;
+    const int wg_tid = threadIdx.x;                                            // 0 .. NT - 1: results and epilogues
+    const int kh = KW == 1 ? 0 : __builtin_amdgcn_readfirstlane(wg_tid >> 8);  // this thread's K share
+    const int tid = wg_tid & 255;                                              // within the share: loop and staging
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 15, kq = lane >> 4;
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     int t0, s0, n0, n1, slot0, nseg0, nseg1;
     if (!STREAM || stream_units == 0) {
         t0 = blockIdx.x;
-        s0 = blockIdx.y * stages_per_block;
+        s0 = (blockIdx.y * KW + kh) * stages_per_block;  // the shares of a workgroup walk consecutive ranges
         n0 = stages_per_block;
         n1 = 0;
         slot0 = blockIdx.y;
@@ -419,7 +428,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             }
             // steps past the end of K contribute nothing
             const bool live = stage_step + x_chunk[u] / 4 <= last_step;
-            xs[buf][(u * 256 + tid) / XCH * RS + x_chunk[u]] =
+            xs_all[buf][kh][(u * 256 + tid) / XCH * RS + x_chunk[u]] =
                 live ? make_uint4(o[0], o[1], o[2], o[3]) : make_uint4(0, 0, 0, 0);
         }
         {
@@ -441,7 +450,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
                 ConstWords v;
 #pragma unroll
                 for (int j = 0; j < CE; ++j) v.w[j] = src[j];
-                *reinterpret_cast<ConstWords*>(&cs[buf][c_group][r][c_col0]) = v;
+                *reinterpret_cast<ConstWords*>(&cs_all[buf][kh][c_group][r][c_col0]) = v;
             }
         }
     };
@@ -462,7 +471,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             }
 #pragma unroll
             for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
-            if (p0 == 0 && row < BM) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
+            if (p0 == 0 && row < BM && kh == 0) inv_rms_s[row] = 1.f / sqrtf(ss / (float)K + fuse.eps);
         }
     }
     store_stage(0, 0);
@@ -490,9 +499,9 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             if (d % SPG == 0) {  // compile-time: a new group starts here
-                const uint4 sc4 = *reinterpret_cast<const uint4*>(&cs[buf][d / SPG][0][lcol]);
-                const uint4 lo4 = *reinterpret_cast<const uint4*>(&cs[buf][d / SPG][1][lcol]);
-                const uint4 hi4 = *reinterpret_cast<const uint4*>(&cs[buf][d / SPG][2][lcol]);
+                const uint4 sc4 = *reinterpret_cast<const uint4*>(&cs_all[buf][kh][d / SPG][0][lcol]);
+                const uint4 lo4 = *reinterpret_cast<const uint4*>(&cs_all[buf][kh][d / SPG][1][lcol]);
+                const uint4 hi4 = *reinterpret_cast<const uint4*>(&cs_all[buf][kh][d / SPG][2][lcol]);
                 cc[0] = ColumnConst{as_half2(sc4.x), as_half2(lo4.x), as_half2(hi4.x)};
                 cc[1] = ColumnConst{as_half2(sc4.y), as_half2(lo4.y), as_half2(hi4.y)};
                 cc[2] = ColumnConst{as_half2(sc4.z), as_half2(lo4.z), as_half2(hi4.z)};
@@ -514,7 +523,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             __builtin_amdgcn_sched_barrier(0);  // keep the reload here (see above)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                const half8_t a = __builtin_bit_cast(half8_t, xs[buf][(mt * 16 + nl) * RS + d * 4 + kq]);
+                const half8_t a = __builtin_bit_cast(half8_t, xs_all[buf][kh][(mt * 16 + nl) * RS + d * 4 + kq]);
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[mt][t], 0, 0, 0);
@@ -535,6 +544,27 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         }
     }
 
+    if constexpr (KW == 2) {
+        // the second share's sums go through LDS (the staging area, no longer read) to the first one, which
+        // from here on is the workgroup: accumulator (mt, t) of lane `tid` at [(mt * 4 + t) * 256 + tid]
+        static_assert(sizeof(xs_all) >= (size_t)MT * 4 * 256 * sizeof(float4_t), "staging area too small for the sums");
+        float4_t* red = reinterpret_cast<float4_t*>(&xs_all[0][0][0]);
+        __syncthreads();
+        if (kh == 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) red[(mt * 4 + t) * 256 + tid] = acc[mt][t];
+        }
+        __syncthreads();
+        if (kh == 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[mt][t] += red[(mt * 4 + t) * 256 + tid];
+        }
+    }
+
     // ---- results.  A tile with several contributors: every one publishes its
     // fp32 partial tile with agent-scope stores (they go through to memory, which
     // is what workgroups on other XCDs see) and counts itself in; the one that
@@ -552,7 +582,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         const bool first_of_two = STREAM && sg == 0 && n1 > 0;
         const bool direct = nseg == 1 && epilogue == kEpilogueNone;
         need_reduce = need_reduce || !direct;
-        if (col >= N) continue;
+        if (col >= N || kh != 0) continue;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -581,7 +611,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
     // every thread's stores acknowledged, then one arrival per tile
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (tid == 0) {
+    if (wg_tid == 0) {
         for (int sg = 0; sg < n_seg; ++sg) {
             const unsigned expected = sg == 0 ? nseg0 : nseg1;
             int last = 0;
@@ -636,7 +666,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         };
         if (epilogue == kEpilogueSiluPairs) {
             // columns [0, 128) of the tile are gate, [128, 256) the matching up columns
-            for (int item = tid; item < M * (kGemmCols / 8); item += 256) {
+            for (int item = wg_tid; item < M * (kGemmCols / 8); item += NT) {
                 const int m = item / (kGemmCols / 8), c4 = item % (kGemmCols / 8) * 4;
                 const float* p = partial + (size_t)m * N + tile * kGemmCols + c4;
                 float4_t g, u;
@@ -656,7 +686,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         }
         if (epilogue == kEpilogueRopeAppend) {
             // four consecutive columns = two interleaved pairs of one head
-            for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
+            for (int item = wg_tid; item < M * (kGemmCols / 4); item += NT) {
                 const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
                 // the row's position and its cos/sin are requested before the partials,
                 // whose wait then covers them
@@ -698,8 +728,8 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
         if (epilogue == kEpilogueResidual) {
             // a wave owns one row of the tile per pass (64 lanes x 4 columns), so the
             // row's sum of squares is one wave reduction; N is a multiple of 256
-            for (int base = 0; base < M * (kGemmCols / 4); base += 256) {
-                const int m = base / (kGemmCols / 4) + wave, c = tile * kGemmCols + lane * 4;
+            for (int base = 0; base < M * (kGemmCols / 4); base += NT) {
+                const int m = base / (kGemmCols / 4) + (wg_tid >> 6), c = tile * kGemmCols + lane * 4;
                 float ss = 0.f;
                 if (m < M) {
                     // the old value of the stream and the next norm's weight are requested
@@ -722,7 +752,7 @@ __global__ __launch_bounds__(256) void gptq_gemm_small_kernel(
             }
             return;
         }
-        for (int item = tid; item < M * (kGemmCols / 4); item += 256) {
+        for (int item = wg_tid; item < M * (kGemmCols / 4); item += NT) {
             const int m = item / (kGemmCols / 4), c = tile * kGemmCols + item % (kGemmCols / 4) * 4;
             if (c >= N) continue;
             const float4_t s = sum_splits(partial + (size_t)m * N + c);
@@ -766,6 +796,7 @@ struct GemmPlan {
     int steps_per_block;
     int stream_units = 0;  // small-M kernel, balanced plan: stages per tile of the walk (0: regular plan)
     int blocks = 0;        // balanced plan: workgroups
+    int k_ways = 1;        // small-M kernel: K shares inside a workgroup (2: eight waves, sums meet in LDS)
 };
 
 static int env_int_gemm(const char* name, int fallback) {
@@ -785,13 +816,36 @@ static const int kFusedReduceMaxM = [] {
 // Plan of the small-M kernel: column tiles x K splits sized so the GPU holds
 // about MH_GEMM_SMALL_WAVES_PER_CU waves per CU; a block walks whole stages.
 // GemmPlan::steps_per_block carries stages_per_block * kSmallDepth.
-GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_blocks = 1) {
+// Two K shares inside a workgroup of eight waves (KW = 2 of the kernel), K not split over workgroups: taken
+// where the column tiles alone fill three quarters of the CUs or more (gate|up of the 70B shape: 224 tiles
+// on 256 CUs) above the rows whose split-K sums the last workgroup of a tile adds cheaply -- from there on
+// the fp32 partial sums of a split plan and their second stage cost more than the CUs left idle
+// (8192 x 57344 at 32 rows: 14.7 MB of partial sums each way and a launch).  MH_GEMM_SMALL_KW (read at every
+// call): 2 takes it for every row count it serves, 1 never.
+static bool small_two_shares(int M, int N, int K, int group_size, int row_blocks) {
+    // (groups of 32 would need 98 KiB of staged constants for the two shares)
+    if (row_blocks != 1 || M > kSmallMaxM || group_size < 64) return false;
+    const int tiles = (N + kGemmCols - 1) / kGemmCols, cus = compute_units();
+    const long stages_total = (K / 32 + kSmallDepth - 1) / kSmallDepth;
+    if (tiles > cus || 4 * tiles < 3 * cus || stages_total < 2 || tiles > kMaxTileCounters) return false;
+    const char* v = getenv("MH_GEMM_SMALL_KW");
+    if (v && *v) return atoi(v) == 2;
+    return M > kFusedReduceMaxM;
+}
+
+GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_blocks = 1, int group_size = 128) {
     GemmPlan p;
     p.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     p.col_tiles = (N + kGemmCols - 1) / kGemmCols;
     p.m_blocks = row_blocks;
     p.steps_total = K / 32;
     const long stages_total = (p.steps_total + kSmallDepth - 1) / kSmallDepth;
+    if (small_two_shares(M, N, K, group_size, row_blocks)) {
+        p.k_ways = 2;
+        p.split_k = 1;
+        p.steps_per_block = (int)((stages_total + 1) / 2 * kSmallDepth);  // stages of one share
+        return p;
+    }
     static const int waves_per_cu = env_int_gemm("MH_GEMM_SMALL_WAVES_PER_CU", 8);
     const long target_blocks = (long)compute_units() * waves_per_cu / 4;
     long split = target_blocks / ((long)p.col_tiles * row_blocks);
@@ -842,7 +896,7 @@ static bool use_small(int M, int group_size) {
 }
 
 GemmPlan plan_gemm(int M, int N, int K, int group_size, bool allow_balanced) {
-    if (use_small(M, group_size)) return plan_gemm_small(M, N, K, allow_balanced);
+    if (use_small(M, group_size)) return plan_gemm_small(M, N, K, allow_balanced, 1, group_size);
     GemmPlan p;
     p.mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
     const int bm = 16 * p.mt;
@@ -891,7 +945,8 @@ bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, i
     if ((epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
         gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
         return true;
-    if (M <= kFusedReduceMaxM) return N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
+    if (M <= kFusedReduceMaxM || small_two_shares(M, N, K, group_size, 1))
+        return N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
     return N % (epilogue == kEpilogueResidual ? 1024 : kGemmCols) == 0;
 }
 
@@ -908,7 +963,7 @@ bool gemm_bias_supported(int M, int N, int K, int group_size, int bits) {
 // Per-row pieces a kEpilogueResidual producer leaves in ssq_out for this shape.
 int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
     if (gemm_cols_preferred(M, N, K, group_size, bits, kEpilogueResidual)) return N / 32;
-    return M <= kFusedReduceMaxM ? N / kGemmCols : N / 1024;
+    return M <= kFusedReduceMaxM || small_two_shares(M, N, K, group_size, 1) ? N / kGemmCols : N / 1024;
 }
 
 static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_small(kSmallMaxM, group_size); }
@@ -952,16 +1007,28 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
                               int N, int K, int group_size, int epilogue, const SmallFuse& fuse) {
     // workspace: [tile counters, zero between launches][fp32 partials]
     // in-kernel reduction by the last workgroup of a tile pays for few rows only
-    unsigned* counters =
-        (M <= kFusedReduceMaxM && p.col_tiles <= kMaxTileCounters) ? reinterpret_cast<unsigned*>(workspace) : nullptr;
+    // (with two K shares per workgroup a tile has one contributor: its epilogue runs in the launch at any row count)
+    unsigned* counters = ((M <= kFusedReduceMaxM || p.k_ways == 2) && p.col_tiles <= kMaxTileCounters)
+                             ? reinterpret_cast<unsigned*>(workspace)
+                             : nullptr;
     float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
     const dim3 grid = p.stream_units ? dim3(p.blocks) : dim3(p.col_tiles, p.split_k, p.m_blocks);
     const bool norm = fuse.ssq_in != nullptr;
-#define MH_LAUNCH_SMALL_N(SPG, NORM, STREAM)                                                                  \
-    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG, NORM, STREAM>), grid, dim3(256), 0, stream,         \
+#define MH_LAUNCH_SMALL_K(SPG, NORM, STREAM, KW)                                                                  \
+    hipLaunchKernelGGL((gptq_gemm_small_kernel<BITS, MT, SPG, NORM, STREAM, KW>), grid, dim3(256 * KW), 0, stream, \
                        (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros, (const half_t*)scales, \
                        (half_t*)out, partial, counters, M, N, K, p.steps_total, p.steps_per_block / kSmallDepth,  \
                        p.split_k, p.stream_units, epilogue, fuse)
+#define MH_LAUNCH_SMALL_N(SPG, NORM, STREAM)                     \
+    do {                                                         \
+        if constexpr (MT <= 2 && !(STREAM) && SPG >= 2) {        \
+            if (p.k_ways == 2) {                                 \
+                MH_LAUNCH_SMALL_K(SPG, NORM, false, 2);          \
+                break;                                           \
+            }                                                    \
+        }                                                        \
+        MH_LAUNCH_SMALL_K(SPG, NORM, STREAM, 1);                 \
+    } while (0)
 #define MH_LAUNCH_SMALL(SPG)                                     \
     do {                                                         \
         if constexpr (MT <= 2) {                                 \
@@ -984,6 +1051,7 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
     }
 #undef MH_LAUNCH_SMALL
 #undef MH_LAUNCH_SMALL_N
+#undef MH_LAUNCH_SMALL_K
     if (counters == nullptr && (p.split_k > 1 || epilogue != kEpilogueNone))
         launch_splitk_finalize(stream, partial, out, M, N, p.split_k, epilogue, fuse);
 }

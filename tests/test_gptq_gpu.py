@@ -502,3 +502,46 @@ def test_quantized_tensor_from_the_reference_s_unpacked_form(hip, bits):
                                   F.matrix_multiply(x, b).numpy().view(np.uint16))
     np.testing.assert_array_equal(a.dequantize().numpy().view(np.uint16),
                                   O.dequantize_packed(qweight, qzeros, scales, None, bits, g).view(np.uint16))
+
+
+@pytest.mark.parametrize("m,k,bits,forced", [(9, 512, 4, False), (17, 768, 4, False), (32, 1024, 4, False), (20, 512, 8, False),
+                                             (1, 1024, 4, True), (8, 768, 4, True)])
+def test_two_k_shares_inside_a_workgroup(hip, m, k, bits, forced):
+    """A wide output (224 column tiles, as many as the 70B gate|up projection has) above 8 rows: workgroups of
+    eight waves whose two K shares meet in LDS (K of three stages leaves the second share a dead stage), the
+    plain product against the oracle and the SiLU*up epilogue, which then runs inside the launch, against the
+    plain product; with MH_GEMM_SMALL_KW=2 also at 1 and 8 rows, where the balanced plan is the default."""
+    import os
+    from minit_amd import synthetic
+    from minit_amd.decode import interleave_gate_up
+    from minit_amd.hip import memory
+    from minit_amd.hip.tensor import HIPTensor
+    n, g = 57344, 128
+    prev = os.environ.get("MH_GEMM_SMALL_KW")
+    if forced:
+        os.environ["MH_GEMM_SMALL_KW"] = "2"
+    try:
+        if bits == 8:  # zero points in the middle of the range and finer steps: the same spread as 4 bit
+            qweight, qzeros, scales = _weights(k, n, g, bits, seed=61, zero_range=(120, 135))
+            scales = (scales.astype(np.float32) / 16).astype(np.float16)
+        else:
+            qweight, qzeros, scales = _weights(k, n, g, bits, seed=61)
+        qweight, qzeros, scales = interleave_gate_up(qweight, qzeros, scales, bits=bits)
+        x = synthetic.activations("test61", f"x{m}", (m, k))
+        y = _run_linear(hip, "mh_gptq_matmul", x, qweight, qzeros, scales, g, bits)
+        assert_fp16_close(y, O.matmul_f64(x, qweight, qzeros, scales, None, bits, g), what=f"two shares M={m} K={k}")
+        dx, dq, dz, ds = _dev(hip, x), _dev(hip, qweight), _dev(hip, qzeros), _dev(hip, scales)
+        out = HIPTensor.allocate((m, n // 2), "float16")
+        ws = memory.workspace(max(hip.call("mh_gptq_silu_pairs_workspace_bytes", m, n, k, g, bits), 256))
+        hip.call("mh_gptq_matmul_silu_pairs", None, dx.data_ptr, dq.data_ptr, dz.data_ptr, ds.data_ptr, out.data_ptr,
+                 m, n, k, g, bits, ws._pointer, ws._size)
+        pairs = y.reshape(m, n // 256, 2, 128)
+        ref = O.silu_mul_f64(pairs[:, :, 0], pairs[:, :, 1]).reshape(m, n // 2)
+        got = out.numpy().astype(np.float64)
+        # same kernel, same sums: the epilogue sees exactly the fp16 values of the plain product
+        assert (np.abs(got - ref) <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) + 1e-7).all()
+    finally:
+        if prev is None:
+            os.environ.pop("MH_GEMM_SMALL_KW", None)
+        else:
+            os.environ["MH_GEMM_SMALL_KW"] = prev
