@@ -862,6 +862,21 @@ GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_block
     const long spb = (stages_total + split - 1) / split;
     p.steps_per_block = (int)(spb * kSmallDepth);
     p.split_k = (int)((stages_total + spb - 1) / spb);
+    // Above the rows of the in-kernel reduction every split costs 8 M N bytes of partial sums through HBM
+    // and the second stage reads them all: pairs of consecutive K ranges go to one workgroup of eight
+    // waves (KW = 2), whose two sums meet in LDS, which halves both (8192x10240 at 32 rows: 8 -> 4 slots).
+    // Measured (us, paired / not): 8192x10240 at 24 / 32 rows 21.0 / 22.5, 21.8 / 24.2 (equal below);
+    // 28672x8192 at 9 / 16 / 17 rows 28.5 / 28.9, 29.4 / 30.9, 34.1 / 35.2 but 38.8 / 36.7 at 32 rows, where
+    // two row tiles meet long K ranges and the eight waves' common barrier per stage costs more than the
+    // partial sums saved: with two row tiles it is taken up to K = 16384.
+    if (M > kFusedReduceMaxM && M <= kSmallMaxM && row_blocks == 1 && group_size >= 64 && p.split_k >= 2 &&
+        p.split_k % 2 == 0 && (M <= 16 || K <= 16384)) {
+        const char* v = getenv("MH_GEMM_SMALL_KW");
+        if (!(v && *v && atoi(v) == 1)) {
+            p.k_ways = 2;
+            p.split_k /= 2;
+        }
+    }
     // Balanced plan (in-kernel reduction only): the tiles' stages form one walk that
     // is cut into target_blocks equal ranges, so every CU gets the same number of
     // stages even where tiles x splits does not divide by the CUs (224 tiles x 2
@@ -1007,8 +1022,9 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
                               int N, int K, int group_size, int epilogue, const SmallFuse& fuse) {
     // workspace: [tile counters, zero between launches][fp32 partials]
     // in-kernel reduction by the last workgroup of a tile pays for few rows only
-    // (with two K shares per workgroup a tile has one contributor: its epilogue runs in the launch at any row count)
-    unsigned* counters = ((M <= kFusedReduceMaxM || p.k_ways == 2) && p.col_tiles <= kMaxTileCounters)
+    // (a tile whose two K shares sit in one workgroup and that is not split further has one contributor: its
+    // epilogue runs in the launch at any row count, small_two_shares)
+    unsigned* counters = ((M <= kFusedReduceMaxM || (p.k_ways == 2 && p.split_k == 1)) && p.col_tiles <= kMaxTileCounters)
                              ? reinterpret_cast<unsigned*>(workspace)
                              : nullptr;
     float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes);
