@@ -565,70 +565,16 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
         }
     }
 
-    // ---- results.  A tile with several contributors: every one publishes its
-    // fp32 partial tile with agent-scope stores (they go through to memory, which
-    // is what workgroups on other XCDs see) and counts itself in; the one that
-    // arrives last adds the partials in slot order -- a fixed order, so the result
-    // does not depend on which workgroup that is -- and puts the counter back to
-    // zero for the next launch.  The SiLU-pair, residual and RoPE epilogues always
-    // take this route (they need the whole tile).  A workgroup that worked on two
-    // tiles publishes both, waits once, and may be the last one of either.
-    const int n_seg = STREAM && n1 > 0 ? 2 : 1;
-    __shared__ int is_last[2];
-    bool need_reduce = false;
-    for (int sg = 0; sg < n_seg; ++sg) {
-        const int tile = t0 + sg, slot = sg == 0 ? slot0 : 0, nseg = sg == 0 ? nseg0 : nseg1;
-        const int col = tile * kGemmCols + lcol;
-        const bool first_of_two = STREAM && sg == 0 && n1 > 0;
-        const bool direct = nseg == 1 && epilogue == kEpilogueNone;
-        need_reduce = need_reduce || !direct;
-        if (col >= N || kh != 0) continue;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int m = mt * 16 + kq * 4 + r;
-                if (m >= M) continue;
-                float4_t v;
-#pragma unroll
-                for (int t = 0; t < 4; ++t) v[t] = first_of_two ? acc_first[STREAM ? mt : 0][t][r] : acc[mt][t][r];
-                if constexpr (NORM) v *= inv_rms_s[m];
-                if (direct) {
-                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                    if (fuse.bias) h = h + *reinterpret_cast<const half4_t*>(fuse.bias + col);
-                    *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
-                } else {
-                    float* dst = partial + (size_t)slot * plane + (size_t)m * N + col;
-                    if (counters)
-                        store_agent4(dst, v);
-                    else
-                        *reinterpret_cast<float4_t*>(dst) = v;
-                }
-            }
-    }
-    if (!need_reduce || counters == nullptr) return;  // without counters a second kernel adds the partials
-
-    // every thread's stores acknowledged, then one arrival per tile
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (wg_tid == 0) {
-        for (int sg = 0; sg < n_seg; ++sg) {
-            const unsigned expected = sg == 0 ? nseg0 : nseg1;
-            int last = 0;
-            if (!(expected == 1 && epilogue == kEpilogueNone)) {
-                const unsigned prev =
-                    __hip_atomic_fetch_add(&counters[t0 + sg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                last = prev == expected - 1;
-                if (last) __hip_atomic_store(&counters[t0 + sg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            is_last[sg] = last;
-        }
-    }
-    __syncthreads();
-
-    auto reduce_tile = [&](int tile, int nseg) {
+    // Sums of a finished tile -> results, with the epilogue.  The sums are the splits' partial sums in
+    // the workspace, added here in slot order, or (lds_tile != nullptr: a tile with a single contributor
+    // whose sums never left the workgroup) one fp32 tile [BM][kGemmCols] in LDS.
+    auto reduce_tile = [&](int tile, int nseg, const float* lds_tile) {
         constexpr int BATCH = 16;  // partial loads in flight per thread
         auto sum_splits = [&](const float* p) {
+            if (lds_tile != nullptr) {  // p - partial = m * N + column: the tile's own column from LDS
+                const size_t off = (size_t)(p - partial);
+                return *reinterpret_cast<const float4_t*>(lds_tile + (off / N) * kGemmCols + (off % N - (size_t)tile * kGemmCols));
+            }
             float4_t s = {0.f, 0.f, 0.f, 0.f};
             for (int sp = 0; sp < nseg; sp += BATCH) {
                 float4_t v[BATCH];
@@ -644,6 +590,11 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
         };
         // two runs of partials (same slots), requested together: one wait instead of two
         auto sum_splits2 = [&](const float* p, const float* q, float4_t& a, float4_t& b) {
+            if (lds_tile != nullptr) {
+                a = sum_splits(p);
+                b = sum_splits(q);
+                return;
+            }
             constexpr int HALF = BATCH / 2;
             a = float4_t{0.f, 0.f, 0.f, 0.f};
             b = a;
@@ -761,8 +712,94 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
             *reinterpret_cast<half4_t*>(out + (size_t)m * N + c) = h;
         }
     };
+    if constexpr (KW == 2) {
+        if (counters != nullptr && epilogue != kEpilogueNone) {
+            // two shares, K not split over workgroups: this workgroup holds the tile's finished sums, and the
+            // epilogue reads them from LDS instead of from partial sums published to memory
+            float* tile_s = reinterpret_cast<float*>(&xs_all[0][0][0]);
+            static_assert(sizeof(xs_all) >= (size_t)BM * kGemmCols * sizeof(float), "staging area too small for the tile");
+            __syncthreads();  // the sums of the second share have been read
+            if (kh == 0) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int m = mt * 16 + kq * 4 + r;
+                        if (m >= M) continue;
+                        float4_t v = {acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
+                        if constexpr (NORM) v *= inv_rms_s[m];
+                        *reinterpret_cast<float4_t*>(tile_s + m * kGemmCols + lcol) = v;
+                    }
+            }
+            __syncthreads();
+            reduce_tile(t0, 1, tile_s);
+            return;
+        }
+    }
+
+    // ---- results.  A tile with several contributors: every one publishes its
+    // fp32 partial tile with agent-scope stores (they go through to memory, which
+    // is what workgroups on other XCDs see) and counts itself in; the one that
+    // arrives last adds the partials in slot order -- a fixed order, so the result
+    // does not depend on which workgroup that is -- and puts the counter back to
+    // zero for the next launch.  The SiLU-pair, residual and RoPE epilogues always
+    // take this route (they need the whole tile).  A workgroup that worked on two
+    // tiles publishes both, waits once, and may be the last one of either.
+    const int n_seg = STREAM && n1 > 0 ? 2 : 1;
+    __shared__ int is_last[2];
+    bool need_reduce = false;
+    for (int sg = 0; sg < n_seg; ++sg) {
+        const int tile = t0 + sg, slot = sg == 0 ? slot0 : 0, nseg = sg == 0 ? nseg0 : nseg1;
+        const int col = tile * kGemmCols + lcol;
+        const bool first_of_two = STREAM && sg == 0 && n1 > 0;
+        const bool direct = nseg == 1 && epilogue == kEpilogueNone;
+        need_reduce = need_reduce || !direct;
+        if (col >= N || kh != 0) continue;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = mt * 16 + kq * 4 + r;
+                if (m >= M) continue;
+                float4_t v;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = first_of_two ? acc_first[STREAM ? mt : 0][t][r] : acc[mt][t][r];
+                if constexpr (NORM) v *= inv_rms_s[m];
+                if (direct) {
+                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    if (fuse.bias) h = h + *reinterpret_cast<const half4_t*>(fuse.bias + col);
+                    *reinterpret_cast<half4_t*>(out + (size_t)m * N + col) = h;
+                } else {
+                    float* dst = partial + (size_t)slot * plane + (size_t)m * N + col;
+                    if (counters)
+                        store_agent4(dst, v);
+                    else
+                        *reinterpret_cast<float4_t*>(dst) = v;
+                }
+            }
+    }
+    if (!need_reduce || counters == nullptr) return;  // without counters a second kernel adds the partials
+
+    // every thread's stores acknowledged, then one arrival per tile
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (wg_tid == 0) {
+        for (int sg = 0; sg < n_seg; ++sg) {
+            const unsigned expected = sg == 0 ? nseg0 : nseg1;
+            int last = 0;
+            if (!(expected == 1 && epilogue == kEpilogueNone)) {
+                const unsigned prev =
+                    __hip_atomic_fetch_add(&counters[t0 + sg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = prev == expected - 1;
+                if (last) __hip_atomic_store(&counters[t0 + sg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            is_last[sg] = last;
+        }
+    }
+    __syncthreads();
+
     for (int sg = 0; sg < n_seg; ++sg)
-        if (is_last[sg]) reduce_tile(t0 + sg, sg == 0 ? nseg0 : nseg1);
+        if (is_last[sg]) reduce_tile(t0 + sg, sg == 0 ? nseg0 : nseg1, nullptr);
 }
 
 // gptq_gemm_cols.hip
