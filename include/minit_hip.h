@@ -371,6 +371,14 @@ int mh_llama_set_globals(void* handle, const void* embed, const void* lm_head, c
                          const float* freqs_cos, const float* freqs_sin);
 /* Scratch for activations, split-K partials and counters; zero-fill it once. */
 size_t mh_llama_scratch_bytes(void* handle, int batch);
+/* Whether a fused residual + RMSNorm launch of the loop has saturated since `scratch` was zero-filled:
+ * those launches keep fp16(h * norm_weight) and apply the row's 1 / rms in the consuming product
+ * (the reference rounds x / rms * w once, rms_norm.py:69-89), and a residual channel with
+ * |h * w| > 65504 is held at the largest finite fp16 value there, which makes that channel of the
+ * normalised row smaller than the reference's.  *clamped is 1 after such a step (the decoded tokens
+ * then carry no parity claim), 0 otherwise; waits for `stream`.  Same batch and scratch as the decode
+ * calls. */
+int mh_llama_norm_clamped(void* handle, mh_stream_t stream, int batch, const void* scratch, int32_t* clamped);
 /* Runs n_steps greedy steps.  tokens [batch] int32 holds the input token of the
  * first step and the last sampled token on return; positions [batch] int32 is
  * where each row's next K/V entry goes and is advanced by one per step;

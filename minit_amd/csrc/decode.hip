@@ -480,6 +480,7 @@ struct Scratch {
     float *ssq_a, *ssq_b;  // per-piece sums of squares of the residual stream, [batch, at most hidden / 32]
     int32_t* pos_base;     // positions at the start of a call that replays a recorded step
     unsigned* attn_counters;
+    unsigned* norm_clamped;  // one word, set when a fused norm's h * w left the fp16 range (never cleared by the loop)
     void* gptq_ws;
     size_t gptq_ws_bytes;
     size_t total;
@@ -537,6 +538,7 @@ static Scratch carve(const Llama& m, int batch, char* base) {
     Scratch s;
     // counters first: they must start (and are left) zero
     s.attn_counters = (unsigned*)take((size_t)batch * c.n_kv_heads * sizeof(unsigned));
+    s.norm_clamped = (unsigned*)take(sizeof(unsigned));
     size_t ws = 0;
     const int shapes[4][2] = {{c.hidden, (int)qkv_n}, {c.n_q_heads * c.head_dim, c.hidden},
                               {c.hidden, 2 * c.ffn}, {c.ffn, c.hidden}};
@@ -726,6 +728,17 @@ size_t mh_llama_scratch_bytes(void* handle, int batch) {
     return carve(*m, batch, nullptr).total;
 }
 
+int mh_llama_norm_clamped(void* handle, mh_stream_t stream, int batch, const void* scratch, int32_t* clamped) {
+    Llama* m = reinterpret_cast<Llama*>(handle);
+    MH_REQUIRE(m != nullptr && batch > 0 && scratch && clamped, "mh_llama_norm_clamped: bad argument");
+    const Scratch s = carve(*m, batch, reinterpret_cast<char*>(const_cast<void*>(scratch)));
+    unsigned word = 0;
+    MH_CHECK_HIP(hipMemcpyAsync(&word, s.norm_clamped, sizeof(word), hipMemcpyDeviceToHost, as_stream(stream)));
+    MH_CHECK_HIP(hipStreamSynchronize(as_stream(stream)));
+    *clamped = word != 0;
+    return MH_OK;
+}
+
 }  // extern "C"
 
 // One decode step is the same sequence of launches on the same buffers for every
@@ -833,6 +846,7 @@ static int decode_impl(void* handle, mh_stream_t stream, int batch, int32_t* tok
                 res.ssq_out = s.ssq_b;
                 res.next_norm_w = (const half_t*)L.post_norm;
                 res.xw_out = s.xn;
+                res.xw_clamped = s.norm_clamped;
                 rc = fused(s.attn, L.o, s.h, c.hidden, c.n_q_heads * c.head_dim, kEpilogueResidual, res);
                 if (rc) return rc;
                 SmallFuse f;

@@ -164,6 +164,7 @@ struct SmallFuse {
     float* ssq_out = nullptr;             // [M, pieces]: kEpilogueResidual
     const half_t* next_norm_w = nullptr;  // [N]
     half_t* xw_out = nullptr;             // [M, N]
+    unsigned* xw_clamped = nullptr;       // optional: set to 1 when an element of xw left the fp16 range
     // y[m, n] = fp16(fp16(y[m, n]) + bias[n]), the two roundings of the reference's product followed by
     // `output += bias` (examples/qwen1_5_int8.py:311-317), before any epilogue (the activation of
     // kEpilogueSiluPairs, the rotation, the residual add) sees y
@@ -181,11 +182,22 @@ struct SmallFuse {
 // xw = fp16(h * w) of the split norm, kept finite: where the reference's x / rms * w is of
 // order w, h * w can leave the fp16 range for a very large residual channel (|h| above
 // 65504 / w); the product then saturates at the largest finite value instead of becoming
-// an infinity that would turn the whole row of the next product into NaN.
+// an infinity that would turn the whole row of the next product into NaN.  A saturated
+// element makes that channel of the normalised row smaller in magnitude than the
+// reference's (which stays exact): `clamped`, when given, is set to 1 so that the caller
+// can tell such a step from an exact one.
 template <typename V>
-__device__ __forceinline__ V norm_weighted(V h, V w) {
+__device__ __forceinline__ V norm_weighted(V h, V w, unsigned* clamped) {
     const V hi = (half_t)65504.f - V{}, lo = -hi;
-    return __builtin_elementwise_max(__builtin_elementwise_min(h * w, hi), lo);
+    const V p = h * w;
+    const V c = __builtin_elementwise_max(__builtin_elementwise_min(p, hi), lo);
+    if (clamped != nullptr) {
+        bool any = false;
+#pragma unroll
+        for (unsigned e = 0; e < sizeof(V) / sizeof(half_t); ++e) any |= !(p[e] == c[e]);
+        if (any) atomicOr(clamped, 1u);
+    }
+    return c;
 }
 
 __device__ __forceinline__ half_t silu_pair(half_t gate, half_t up) {

@@ -694,7 +694,7 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
                     if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + c);
                     const half4_t h = h_old + y;  // fp16 add, one rounding
                     *reinterpret_cast<half4_t*>(hp) = h;
-                    if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) = norm_weighted(h, nw);
+                    if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + (size_t)m * N + c) = norm_weighted(h, nw, fuse.xw_clamped);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) ss += (float)h[e] * (float)h[e];
                 }

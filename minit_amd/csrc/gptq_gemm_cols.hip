@@ -345,7 +345,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         // are adjacent lanes of one wave)
         const half2_t h = ep_h + y;  // ep_h: this thread's two elements of the stream, read at the start
         *op = h;
-        if (fuse.xw_out) *reinterpret_cast<half2_t*>(fuse.xw_out + (size_t)m * N + col) = norm_weighted(h, ep_w);
+        if (fuse.xw_out) *reinterpret_cast<half2_t*>(fuse.xw_out + (size_t)m * N + col) = norm_weighted(h, ep_w, fuse.xw_clamped);
         float ss = (float)h[0] * (float)h[0] + (float)h[1] * (float)h[1];
 #pragma unroll
         for (int off = 1; off < kColsTile / 2; off <<= 1) ss += __shfl_xor(ss, off);

@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void splitk_finalize_residual_kernel(const flo
     const half4_t r = *reinterpret_cast<const half4_t*>(h + i) + y;  // fp16 add, one rounding
     *reinterpret_cast<half4_t*>(h + i) = r;
     if (fuse.xw_out)
-        *reinterpret_cast<half4_t*>(fuse.xw_out + i) = norm_weighted(r, *reinterpret_cast<const half4_t*>(fuse.next_norm_w + i % N));
+        *reinterpret_cast<half4_t*>(fuse.xw_out + i) = norm_weighted(r, *reinterpret_cast<const half4_t*>(fuse.next_norm_w + i % N), fuse.xw_clamped);
     float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) ss += (float)r[e] * (float)r[e];

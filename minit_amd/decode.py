@@ -302,6 +302,15 @@ class LlamaDecoder:
             result = out.numpy()
         return result, (logits.numpy() if logits else None)
 
+    def norm_clamped(self, batch: int) -> bool:
+        """True when a fused residual + norm launch at this batch size has held an ``h * norm_weight``
+        at the fp16 limit since the decoder was built (``mh_llama_norm_clamped``): the steps since
+        then differ from the reference's in that channel and carry no parity claim."""
+        flag = ctypes.c_int(0)
+        lib.call("mh_llama_norm_clamped", self._handle, None, batch, self._scratch_for(batch)._pointer,
+                 ctypes.byref(flag))
+        return bool(flag.value)
+
     def weight_bytes_per_token(self, batch: int, context: int) -> int:
         """Algorithmic HBM bytes one decode step has to move."""
         c = self.config

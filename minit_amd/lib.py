@@ -81,6 +81,7 @@ PROTOTYPES = {
     "mh_llama_set_layer": (c_int, [_P, c_int, _P]),
     "mh_llama_set_globals": (c_int, [_P, _P, _P, _P, _P, _P]),
     "mh_llama_scratch_bytes": (c_size_t, [_P, c_int]),
+    "mh_llama_norm_clamped": (c_int, [_P, _P, c_int, _P, POINTER(c_int)]),
     "mh_llama_decode": (c_int, [_P, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t]),
     "mh_llama_decode_graph": (c_int, [_P, _P, c_int, _P, _P, c_int, _P, _P, _P, c_size_t]),
     "mh_synth_u32": (c_int, [_P, _P, c_size_t, c_uint64]),

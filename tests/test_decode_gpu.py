@@ -343,6 +343,7 @@ def test_large_residual_channels(hip, batch):
     assert np.isfinite(g).all()
     assert np.linalg.norm(g - r) / np.linalg.norm(r) <= 1e-2
     assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
+    assert not dec.norm_clamped(batch)
 
     # beyond the fp16 range: 3e4 * 3 = 9e4
     model["embed"][:, big] = (3e4 * np.sign(model["embed"][:, big].astype(np.float32))).astype(np.float16)
@@ -350,6 +351,7 @@ def test_large_residual_channels(hip, batch):
     dec2.load_host(model, k_cache, v_cache)
     _, got2 = dec2.decode(tokens, positions, 1, want_logits=True)
     assert np.isfinite(got2.astype(np.float64)).all(), "a saturated h * w must not turn the step into NaN"
+    assert dec2.norm_clamped(batch), "the saturated step must be reported"
 
 
 @pytest.mark.parametrize("batch", [2, 9])
