@@ -1,15 +1,17 @@
 // W8A8 int8 GEMM, operand tiles fetched straight from global memory into LDS.
 //
-// Same tiling and fragment schedule as i8_gemm_k128_kernel (i8_gemm.hip): block
-// tile 128 x 256, 128-k stages, eight waves 2 x 4, each 64 x 64 as 2 x 2 tiles of
-// v_mfma_i32_32x32x32_i8, a k-step split into four quarters with double-buffered
-// fragments.  What differs is how a stage reaches LDS: gfx950's 128-bit
-// LDS-destination buffer loads write 16 bytes per lane to consecutive LDS
-// addresses (wave base in M0), so there is no register ring, no ds_write and no
+// Block tile 128 x 256, 128-k stages, eight waves 2 x 4, each 64 x 64 as 4 x 4 tiles
+// of v_mfma_i32_16x16x64_i8; a k-step is two 64-k halves with double-buffered
+// fragments (lane l: 16 bytes of row l % 16, k chunk l / 16).  The 16 x 16 x 64 form
+// is chosen for what the part sustains under its power limit: a register-resident
+// stream of it on random int8 operands runs at 4.1 POP/s (2.06 GHz) where the
+// 32 x 32 x 32 form runs at 3.3 POP/s (1.68 GHz), at the same fragment bytes per MAC.
+// gfx950's 128-bit LDS-destination buffer loads write 16 bytes per lane to consecutive
+// LDS addresses (wave base in M0), so there is no register ring, no ds_write and no
 // wait for loaded registers on the issue path.  The LDS swizzle that keeps the
 // fragment reads conflict-free is applied on the global side instead: a wave load
 // covers eight 128-byte LDS rows, and the lane that fills chunk position c' of row r
-// fetches chunk c' ^ ((r >> 1) & 7) of that row's line.  Without the ring's
+// fetches chunk c' ^ ((r >> 1) & 7) of that row's line.  Without a ring's
 // registers three stages fit into LDS (144 KiB), which lets a stage be requested
 // almost three k-steps before its first use.
 //
@@ -71,20 +73,18 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 2, wx = wave & 3;
-    const int l32 = lane & 31, lh = lane >> 5;
+    const int l16 = lane & 15, lg = lane >> 4;
 
     if (out) {  // visible to the epilogue through the barriers of the main loop
         if (tid < kDmaBN) s_w[tid] = w_scale[min(n0 + tid, N - 1)];
         if (tid < kDmaBM) s_a[tid] = a_scale[min(m0 + tid, M - 1)];
     }
 
-    int16_t_v acc[2][2];
+    int4_t acc[4][4];  // [m tile][n tile] of 16 x 16
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+        for (int j = 0; j < 4; ++j) acc[i][j] = int4_t{0, 0, 0, 0};
 
     // Wave load L = j * 8 + wave (j = 0..5) fills LDS rows L * 8 .. L * 8 + 7 of a stage:
     // rows 0..127 are the A tile (L < 16, j < 2), rows 128..383 the W tile.
@@ -112,30 +112,29 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     };
 
     auto swz128 = [](int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); };
-    int4_t fa[2][2], fb[2][2];
-    auto read_frag = [&](int set, int buf, int ks) {
-        const int chunk = ks * 2 + lh;
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-            fa[set][i] = *reinterpret_cast<const int4_t*>(As(buf) + swz128(wy * 64 + i * 32 + l32, chunk));
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            fb[set][j] = *reinterpret_cast<const int4_t*>(Bs(buf) + swz128(wx * 64 + j * 32 + l32, chunk));
+    // Fragments of one 64-k half of a stage: lane l holds 16 bytes of row l % 16, k chunk l / 16
+    // (the same mapping for both operands, which is all a dot product needs).
+    int4_t fa[2][4], fb[2][4];
+    auto read_a = [&](int set, int buf, int half, int i) {
+        fa[set][i] = *reinterpret_cast<const int4_t*>(As(buf) + swz128(wy * 64 + i * 16 + l16, half * 4 + lg));
     };
-    auto mfma_one = [&](int set, int t) {
-        const int i = t >> 1, j = t & 1;
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+    auto read_b = [&](int set, int buf, int half, int j) {
+        fb[set][j] = *reinterpret_cast<const int4_t*>(Bs(buf) + swz128(wx * 64 + j * 16 + l16, half * 4 + lg));
     };
-    auto mfma_rest = [&](int set) {
-        mfma_one(set, 1);
-        mfma_one(set, 2);
-        mfma_one(set, 3);
+    auto mfma_row = [&](int set, int i) {  // the four column tiles of row tile i
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+    };
+    auto mfma_pair = [&](int set, int i, int j) {
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+        acc[i][j + 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[set][j + 1], fa[set][i], acc[i][j + 1], 0, 0, 0);
     };
 
     // Stage s lives in LDS buffer s % 3.  It is requested after the barrier of k-step
     // s - 3 (every wave has then read the last fragments of that buffer) and in the
-    // first quarter of k-step s - 2, and must have landed at the barrier of k-step
-    // s - 1, whose last quarter reads its first fragments.
+    // first half of k-step s - 2, and must have landed at the barrier of k-step
+    // s - 1, whose second half reads its first fragments.
 #pragma unroll
     for (int s = 0; s < kDmaStages; ++s) {
         load_stage_part(0, s);
@@ -143,92 +142,77 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     }
     asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // stage 0 of this wave
     __syncthreads();
-    read_frag(0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        read_a(0, 0, 0, t);
+        read_b(0, 0, 0, t);
+    }
     int buf = 0;
     for (int kt = 0; kt < KT; ++kt) {
         const int nbuf = buf == kDmaStages - 1 ? 0 : buf + 1;
-        // quarter 0 (second half of the loads of stage kt + 2)
-        // (one load between two MFMAs: issued back to back by all eight waves the loads fill the vector
-        // memory queue and the waves stall in issue with the matrix pipes idle)
-        mfma_one(0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt > 0) load_stage_piece(3, kt + 2);
-        read_frag(1, buf, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt > 0) load_stage_piece(4, kt + 2);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(0, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt > 0) load_stage_piece(5, kt + 2);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(0, 3);
-        __builtin_amdgcn_sched_barrier(0);
-        // quarter 1
-        mfma_one(1, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frag(0, buf, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_rest(1);
-        __builtin_amdgcn_sched_barrier(0);
-        // quarter 2
-        mfma_one(0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frag(1, buf, 3);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_rest(0);
+        // first half: 16 MFMAs on set 0; the fragments of the second half and the second half of the
+        // loads of stage kt + 2 go between them (one load between two pairs of MFMAs: issued back to
+        // back by all eight waves the loads fill the vector memory queue and the waves stall in issue
+        // with the matrix pipes idle)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            mfma_pair(0, t >> 1, (t & 1) * 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t < 4) {
+                read_a(1, buf, 1, t);
+                read_b(1, buf, 1, t);
+            } else if (t < 7) {
+                if (kt > 0) load_stage_piece(t - 1, kt + 2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // second half, first quarter of its MFMAs
+        mfma_row(1, 0);
         __builtin_amdgcn_sched_barrier(0);
         // stage kt + 1 of this wave has landed (the six loads of stage kt + 2 may still be
         // in flight) and this wave's reads of `buf` are complete: publish / release
         asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
         __syncthreads();
-        // quarter 3 (first half of the loads of stage kt + 3 into the buffer just released)
-        mfma_one(1, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_stage_piece(0, kt + 3);
-        read_frag(0, nbuf, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        load_stage_piece(1, kt + 3);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(1, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        load_stage_piece(2, kt + 3);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(1, 3);
-        __builtin_amdgcn_sched_barrier(0);
+        // the rest: first fragments of stage kt + 1 and the first half of the loads of stage kt + 3
+        // into the buffer just released
+#pragma unroll
+        for (int t = 2; t < 8; ++t) {
+            mfma_pair(1, t >> 1, (t & 1) * 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t < 6) {
+                read_a(0, nbuf, 0, t - 2);
+                read_b(0, nbuf, 0, t - 2);
+            }
+            if (t >= 3 && t < 6) load_stage_piece(t - 3, kt + 3);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         buf = nbuf;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the (empty) loads past the end write LDS too
     __syncthreads();  // every wave is done with the operand buffers
 
-    // Epilogue.  acc[i][j][q * 4 + e] belongs to row m = l32 and column
-    // n = q * 8 + lh * 4 + e of its tile: four consecutive n per (lane, q).
+    // Epilogue.  acc[i][j][e] belongs to row m = i * 16 + l16 and column
+    // n = j * 16 + lg * 4 + e of the wave tile: four consecutive n per lane.
     const int wm = wy * 64, wn = wx * 64;  // wave tile origin inside the block tile
     if (acc_out) {
         const bool n_vec = (N % 4 == 0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int m = m0 + wm + i * 32 + l32;
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + wm + i * 16 + l16;
             if (m >= M) continue;
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + wn + j * 16 + lg * 4;
+                if (n >= N) continue;
+                int32_t* dst = acc_out + (size_t)m * N + n;
+                if (n_vec && n + 4 <= N) {
+                    *reinterpret_cast<int4_t*>(dst) = acc[i][j];
+                } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int n = n0 + wn + j * 32 + q * 8 + lh * 4;
-                    if (n >= N) continue;
-                    int32_t* dst = acc_out + (size_t)m * N + n;
-                    if (n_vec && n + 4 <= N) {
-                        int4_t v = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
-                        *reinterpret_cast<int4_t*>(dst) = v;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (n + e < N) dst[e] = acc[i][j][q * 4 + e];
-                    }
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) dst[e] = acc[i][j][e];
                 }
+            }
         }
     }
     if (out) {
@@ -237,13 +221,14 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
         int8_t* stage = smem + wave * (32 * kDmaStagePitch);
         const bool n_vec = (N % 8 == 0);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const float sa = s_a[wm + i * 32 + l32];
+        for (int ip = 0; ip < 2; ++ip) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int ii = 0; ii < 2; ++ii) {
+                const int i = ip * 2 + ii;
+                const float sa = s_a[wm + i * 16 + l16];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int nl = j * 32 + q * 8 + lh * 4;
+                for (int j = 0; j < 4; ++j) {
+                    const int nl = j * 16 + lg * 4;
                     const float4_t sw = *reinterpret_cast<const float4_t*>(s_w + wn + nl);
                     half4_t h;
 #pragma unroll
@@ -251,12 +236,13 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
                         // The scale product and its product with the sum are each rounded to
                         // fp32 and only then to fp16; the empty asm keeps the compiler from
                         // fusing the last two steps into one instruction that rounds once.
-                        float prod = (float)acc[i][j][q * 4 + e] * (sa * sw[e]);
+                        float prod = (float)acc[i][j][e] * (sa * sw[e]);
                         asm volatile("" : "+v"(prod));
                         h[e] = (half_t)prod;
                     }
-                    *reinterpret_cast<half4_t*>(stage + l32 * kDmaStagePitch + nl * 2) = h;
+                    *reinterpret_cast<half4_t*>(stage + (ii * 16 + l16) * kDmaStagePitch + nl * 2) = h;
                 }
+            }
             // wave-private region: only this wave's own LDS traffic has to land
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -264,7 +250,7 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const int row = rr * 8 + (lane >> 3), c8 = (lane & 7) * 8;
-                const int m = m0 + wm + i * 32 + row, n = n0 + wn + c8;
+                const int m = m0 + wm + ip * 32 + row, n = n0 + wn + c8;
                 const int4_t v = *reinterpret_cast<const int4_t*>(stage + row * kDmaStagePitch + c8 * 2);
                 if (m >= M || n >= N) continue;
                 half_t* dst = out + (size_t)m * N + n;
