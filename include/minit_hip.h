@@ -317,9 +317,12 @@ int mh_gather_columns(mh_stream_t stream, const void* x, const int32_t* index, v
  *                       position (clamped to the cache); max_seq a multiple of 64
  *   mh_attn_decode      out[b, h] = softmax(q[b, h] . K[b, h / (QH / KVH), 0..positions[b]] / sqrt(D)) . V,
  *                       fp32 inside, one rounding; D == 128, QH / KVH in {1, 2, 4, 8};
- *                       positions[b] is the index of the newest cache entry.  The
- *                       workspace is zero-filled once by the caller and left with its
- *                       counters at zero. */
+ *                       positions[b] is the index of the newest cache entry; cache
+ *                       entries past it are never part of the result, whatever they hold.
+ *                       The workspace is zero-filled once by the caller and left with its
+ *                       counters at zero; where the counters end depends on batch and
+ *                       KVH, so a workspace that moves to a call with other sizes is
+ *                       zero-filled again. */
 /* The residual add and the norm that follows it in one pass over the row
  * (examples/llama3_70b.py:159-162: `x = x + attn(...)`, then `norm(x)`): h[r, :] =
  * fp16(h + delta) in place (skipped when delta is NULL), out[r, :] = RMSNorm(h) *

@@ -240,10 +240,14 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
     const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i16 = lane & 15, kq = lane >> 4;
-    const int len = min(max(positions[b], 0), max_seq - 1) + 1;  // the new token has been appended
-    // chunk starts stay multiples of 64: a chunk is one tile of the V cache
-    const int span = ((len + splits - 1) / splits + 63) / 64 * 64;
-    const int t0 = split * span, t1 = min(len, t0 + span);
+    // Chunks of 64 positions (one tile of the V cache) are dealt round robin, first over the
+    // blocks of a (row, KV head) pair and then over their waves: chunk c belongs to block
+    // c % splits, wave (c / splits) % WAVES.  The deal does not depend on the length, so a
+    // wave requests its first chunk before the position has arrived, and no wave holds more
+    // than one chunk over the others.
+    const int stride = splits * WAVES * 64;
+    const int c_first = (split + wave * splits) * 64;
+    const int t1 = min(max(positions[b], 0), max_seq - 1) + 1;  // the new token has been appended
 
     __shared__ __attribute__((aligned(16))) half_t p_s[WAVES][16 * PP];
     __shared__ float m_s[WAVES][16], l_s[WAVES][16];
@@ -273,14 +277,15 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) acc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int c0 = t0 + wave * 64; c0 < t1; c0 += WAVES * 64) {
-        // all loads of the chunk are issued before the first use (refilling K after
-        // Q K^T and V after P V for the wave's next chunk, so that loads stay in flight
-        // under the arithmetic, measured no faster at batch 1 and 32 and slower at 8)
-        uint4 kf[4][4], vf[8][2];
+    // all loads of a chunk are issued before the first use (refilling K after Q K^T and V
+    // after P V for the wave's next chunk, so that loads stay in flight under the arithmetic,
+    // measured no faster at batch 1 and 32 and slower at 8).  Rows and tiles are clamped to
+    // the cache, not to the length: what lies past the end is masked below.
+    uint4 kf[4][4], vf[8][2];
+    auto load_chunk = [&](int c0) {
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt) {
-            const int row = min(c0 + pt * 16 + i16, t1 - 1);
+            const int row = min(c0 + pt * 16 + i16, max_seq - 1);
             const half_t* kp = kbase + (size_t)row * D + kq * 8;
 #pragma unroll
             for (int s = 0; s < 4; ++s) kf[pt][s] = *reinterpret_cast<const uint4*>(kp + s * 32);
@@ -292,7 +297,9 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
             for (int dt = 0; dt < 8; ++dt)
                 vf[dt][ks] = *reinterpret_cast<const uint4*>(vbase + vt_offset(dt * 16 + i16, p0));
         }
-
+    };
+    load_chunk(c_first);
+    for (int c0 = c_first; c0 < t1;) {
         // S tile pt: rows = heads kq*4 + r, column = position c0 + pt*16 + i16
         float4_t sc[4];
 #pragma unroll
@@ -365,6 +372,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();  // p_s is rewritten by the next chunk
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        c0 += stride;
+        if (c0 < t1) load_chunk(c0);
     }
 
     // acc[dt][r] is head kq*4 + r, dim dt*16 + i16
@@ -488,19 +497,21 @@ struct Scratch {
 
 static size_t align_up(size_t v) { return (v + 255) / 256 * 256; }
 
-// With a (row, KV head) pair per CU or more, a pair is one block of eight waves and nothing is merged
-// across blocks (the merge of two splits costs 3.5 us of a 56 us launch at 32 rows).
-static bool attn_unsplit(int n_kv_heads, int batch) { return batch * n_kv_heads >= compute_units(); }
-
+// Blocks of a (row, KV head) pair.  A CU sustains about 90 KB of cache reads in flight whatever
+// the number of waves asking, so a second block on a CU doubles that CU's time: the launch
+// takes as many blocks as there are CUs and no more (measured at context 2048, batch 2 to 24:
+// 192 to 256 blocks are the fastest launch at every batch size, 288 and more are 15 to 40 %
+// slower), and not more than one 64-position chunk per wave needs.  A pair that is left with
+// one block runs eight waves instead of four and merges nothing across blocks.
 static int attn_splits(int n_kv_heads, int max_seq, int batch) {
     const int pairs = batch * n_kv_heads;
-    if (attn_unsplit(n_kv_heads, batch)) return 1;
-    // two blocks per CU: 0.5, 1, 1.5, 4 and 8 measured no faster at any batch size (context 2048)
-    int splits = (2 * compute_units() + pairs - 1) / pairs;
-    // a block walks 256 positions per pass of its four waves
-    const int max_splits = (max_seq + 255) / 256;
-    if (splits > max_splits) splits = max_splits;
+    const int chunks = (max_seq + 63) / 64;
+    int splits = (chunks + 3) / 4;
+    const int cap = compute_units() / pairs;
+    if (splits > cap) splits = cap;
     if (splits > 64) splits = 64;
+    static const char* env = getenv("MH_ATTN_SPLITS");
+    if (env && *env && atoi(env) > 0) splits = atoi(env) > 64 ? 64 : atoi(env);
     return splits < 1 ? 1 : splits;
 }
 static int attn_splits(const Llama& m, int batch) { return attn_splits(m.cfg.n_kv_heads, m.cfg.max_seq, batch); }
@@ -517,7 +528,7 @@ template <int G>
 static void launch_attn_raw(hipStream_t st, const half_t* q, const half_t* k_cache, const half_t* vt_cache,
                             const int32_t* positions, half_t* out, float* partial, unsigned* counters, int batch,
                             int n_kv_heads, int max_seq, int splits) {
-    if (splits == 1 && attn_unsplit(n_kv_heads, batch))
+    if (splits == 1)
         hipLaunchKernelGGL((attn_decode_kernel<G, 128, 8>), dim3(1, n_kv_heads, batch), dim3(512), 0, st, q, k_cache,
                            vt_cache, positions, out, partial, counters, n_kv_heads, max_seq, 1.0f / sqrtf(128.f), 1);
     else

@@ -85,25 +85,26 @@ def decode_attention(q, k_cache, vt_cache, positions, max_seq: int):
     batch, qh, d = q._shape
     kvh = k_cache._shape[1]
     nbytes = lib.call("mh_attn_decode_workspace_bytes", batch, qh, kvh, d, max_seq)
-    ws = _attention_workspace(nbytes)
+    ws = _attention_workspace(nbytes, (batch, qh, kvh, d, max_seq))
     out = HIPTensor.allocate((batch, qh, d), q.dtype)
     lib.call("mh_attn_decode", None, q.data_ptr, k_cache.data_ptr, vt_cache.data_ptr, positions.data_ptr,
              out.data_ptr, batch, qh, kvh, d, max_seq, ws._pointer, ws._size)
     return out
 
 
-_ATTN_WS = None
+_ATTN_WS = {}
 
 
-def _attention_workspace(nbytes: int):
-    """Zero-filled once; the kernel leaves its counters at zero."""
-    global _ATTN_WS
-    if _ATTN_WS is None or _ATTN_WS._size < nbytes:
+def _attention_workspace(nbytes: int, key):
+    """One workspace per call geometry, zero-filled once: the kernel leaves its counters at zero,
+    but where the counters end and the records begin depends on the geometry, so a buffer shared
+    between geometries would hand one call's records to the next as counters."""
+    if key not in _ATTN_WS:
+        mem = memory.HIPMemory(max(nbytes, 256))
+        mem.reset()
         memory.synchronize()
-        _ATTN_WS = memory.HIPMemory(max(nbytes, 1 << 20))
-        _ATTN_WS.reset()
-        memory.synchronize()
-    return _ATTN_WS
+        _ATTN_WS[key] = mem
+    return _ATTN_WS[key]
 
 
 class LlamaDecoder:
