@@ -255,7 +255,9 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
                 if (m >= M || n >= N) continue;
                 half_t* dst = out + (size_t)m * N + n;
                 if (n_vec) {
-                    *reinterpret_cast<int4_t*>(dst) = v;
+                    // streamed out: with one tile per CU every workgroup stores at the same time, and the
+                    // 16.8 MB of a 2048 x 4096 result are 3 us of the launch
+                    __builtin_nontemporal_store(v, reinterpret_cast<int4_t*>(dst));
                 } else {
                     const half_t* hv = reinterpret_cast<const half_t*>(&v);
 #pragma unroll
