@@ -494,6 +494,18 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
 
     for (int stage = 0; stage < n_stages; ++stage) {
         const int buf = stage & 1;
+        // Two workgroups share a CU on most plans, and the older one wins every arbitration: it runs
+        // ahead and leaves the younger one to finish alone, with half the CU's loads in flight
+        // (8192 x 57344 at one row: the first 256 workgroups leave the loop 13 us before the other
+        // 256).  The priority of a wave falls with its progress through its range, in four steps, so
+        // whichever workgroup is behind is served first (46.4 -> 45.2 us for that launch).
+        if constexpr (KW == 1) {
+            const int level = 3 - min(3, stage * 4 / n_stages);
+            if (level == 3) __builtin_amdgcn_s_setprio(3);
+            else if (level == 2) __builtin_amdgcn_s_setprio(2);
+            else if (level == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
         const int next_tile = tile_of(stage + 1), next_step = step_of(stage + 1);
         const __amdgpu_buffer_rsrc_t next_rsrc = stage + 1 < n_stages ? q_rsrc : q_none;
 #pragma unroll
