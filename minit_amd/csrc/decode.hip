@@ -299,7 +299,20 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
         }
     };
     load_chunk(c_first);
+    // Two waves share a SIMD when a block has eight, and the older one wins every arbitration: the
+    // priority of a wave falls with the share of its chunks it has behind it, so that the four
+    // younger waves are not left to walk their last chunks alone.
+    const int n_chunks = t1 > c_first ? (t1 - c_first + stride - 1) / stride : 0;
+    int chunk_no = 0;
     for (int c0 = c_first; c0 < t1;) {
+        if constexpr (WAVES > 4) {
+            const int level = 3 - min(3, chunk_no * 4 / n_chunks);
+            if (level == 3) __builtin_amdgcn_s_setprio(3);
+            else if (level == 2) __builtin_amdgcn_s_setprio(2);
+            else if (level == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+            ++chunk_no;
+        }
         // S tile pt: rows = heads kq*4 + r, column = position c0 + pt*16 + i16
         float4_t sc[4];
 #pragma unroll
