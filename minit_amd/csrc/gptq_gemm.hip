@@ -799,18 +799,19 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
     // every thread's stores acknowledged, then one arrival per tile
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (wg_tid == 0) {
-        for (int sg = 0; sg < n_seg; ++sg) {
-            const unsigned expected = sg == 0 ? nseg0 : nseg1;
-            int last = 0;
-            if (!(expected == 1 && epilogue == kEpilogueNone)) {
-                const unsigned prev =
-                    __hip_atomic_fetch_add(&counters[t0 + sg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                last = prev == expected - 1;
-                if (last) __hip_atomic_store(&counters[t0 + sg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            is_last[sg] = last;
+    // (a workgroup that worked on two tiles counts in at both at once, from two waves: one after the
+    // other the two round trips are 1.5 us of the launch's tail)
+    if ((wg_tid & 63) == 0 && (wg_tid >> 6) < n_seg) {
+        const int sg = wg_tid >> 6;
+        const unsigned expected = sg == 0 ? nseg0 : nseg1;
+        int last = 0;
+        if (!(expected == 1 && epilogue == kEpilogueNone)) {
+            const unsigned prev =
+                __hip_atomic_fetch_add(&counters[t0 + sg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last = prev == expected - 1;
+            if (last) __hip_atomic_store(&counters[t0 + sg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        is_last[sg] = last;
     }
     __syncthreads();
 
