@@ -142,6 +142,19 @@ __device__ __forceinline__ bool arrive_and_check_last(unsigned* counter, unsigne
     return *flag != 0;
 }
 
+// Wave priority that falls as the wave's work gets done: `done` of `total` units behind it -> 3, 2, 1, 0
+// by quarters (delay8: eighths of a unit of grace before the first step down).  Waves that share a SIMD --
+// of one workgroup or of two on one CU -- are otherwise served oldest first, so the older one runs
+// ahead and the younger one finishes alone; with this the one behind is served first.
+// (s_setprio takes an immediate.)
+__device__ __forceinline__ void set_priority_by_progress(int done, int total, int delay8 = 0) {
+    const int level = 3 - min(3, max(done * 8 - delay8, 0) / (2 * total));
+    if (level == 3) __builtin_amdgcn_s_setprio(3);
+    else if (level == 2) __builtin_amdgcn_s_setprio(2);
+    else if (level == 1) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
+}
+
 // 16-bit storage <-> fp32.
 template <typename T> struct Cvt;
 template <> struct Cvt<half_t> {

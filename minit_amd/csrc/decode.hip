@@ -306,12 +306,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_decode_kernel(
     int chunk_no = 0;
     for (int c0 = c_first; c0 < t1;) {
         if constexpr (WAVES > 4) {
-            const int level = 3 - min(3, chunk_no * 4 / n_chunks);
-            if (level == 3) __builtin_amdgcn_s_setprio(3);
-            else if (level == 2) __builtin_amdgcn_s_setprio(2);
-            else if (level == 1) __builtin_amdgcn_s_setprio(1);
-            else __builtin_amdgcn_s_setprio(0);
-            ++chunk_no;
+            set_priority_by_progress(chunk_no++, n_chunks);
         }
         // S tile pt: rows = heads kq*4 + r, column = position c0 + pt*16 + i16
         float4_t sc[4];

@@ -503,12 +503,8 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
             // (balanced plan: the workgroups of the second half of the grid are the younger ones of their
             // CUs; they step down an eighth of the range later, which halves the lead the older one can
             // take: 46.3 -> 45.3 us more.  On the two-dimensional grids the same offset measured slower.)
-            const int late = (STREAM && stream_units != 0 && blockIdx.x * 2 >= gridDim.x) ? n_stages : 0;
-            const int level = 3 - min(3, max(stage * 8 - late, 0) / (2 * n_stages));
-            if (level == 3) __builtin_amdgcn_s_setprio(3);
-            else if (level == 2) __builtin_amdgcn_s_setprio(2);
-            else if (level == 1) __builtin_amdgcn_s_setprio(1);
-            else __builtin_amdgcn_s_setprio(0);
+            const int late = (STREAM && stream_units != 0 && blockIdx.x * 2 >= gridDim.x) ? n_stages : 0;  // in eighths of a stage
+            set_priority_by_progress(stage, n_stages, late);
         }
         const int next_tile = tile_of(stage + 1), next_step = step_of(stage + 1);
         const __amdgpu_buffer_rsrc_t next_rsrc = stage + 1 < n_stages ? q_rsrc : q_none;

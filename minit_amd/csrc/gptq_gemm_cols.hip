@@ -250,13 +250,7 @@ __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
         // four on 28672 x 8192 (1.6 us on 8192 x 8192), which then stream alone.  The priority of
         // a wave falls with its progress through its K range, so the one behind is served first.
         // (Not on the cut plan, where a CU holds two workgroups of unequal ranges: 0.4 us slower there.)
-        if (parts == 1) {
-            const int level = 3 - min(3, base * 4 / steps_per_wave);
-            if (level == 3) __builtin_amdgcn_s_setprio(3);
-            else if (level == 2) __builtin_amdgcn_s_setprio(2);
-            else if (level == 1) __builtin_amdgcn_s_setprio(1);
-            else __builtin_amdgcn_s_setprio(0);
-        }
+        if (parts == 1) set_priority_by_progress(base, steps_per_wave);
 #pragma unroll
         for (int d = 0; d < R; ++d) {
             const int step = begin + base + d;
