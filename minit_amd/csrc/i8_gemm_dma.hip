@@ -53,7 +53,6 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     constexpr int BK = kDmaBK;
     // [3][A tile | W tile]; reused by the epilogue as eight 32-row output stages
     __shared__ __attribute__((aligned(1024))) int8_t smem[kDmaStages * kDmaStageBytes];
-    __shared__ float s_a[kDmaBM], s_w[kDmaBN];
     auto As = [&](int buf) { return smem + buf * kDmaStageBytes; };
     auto Bs = [&](int buf) { return smem + buf * kDmaStageBytes + kDmaBM * BK; };
 
@@ -75,9 +74,25 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
     const int wy = wave >> 2, wx = wave & 3;
     const int l16 = lane & 15, lg = lane >> 4;
 
-    if (out) {  // visible to the epilogue through the barriers of the main loop
-        if (tid < kDmaBN) s_w[tid] = w_scale[min(n0 + tid, N - 1)];
-        if (tid < kDmaBM) s_a[tid] = a_scale[min(m0 + tid, M - 1)];
+    // The scales of this lane's results (rows i * 16 + l16, columns j * 16 + lg * 4 .. + 3 of the wave
+    // tile), requested here and used in the epilogue.  They stay in registers: staged through LDS at
+    // this point, two loads, each waited for and stored, stood in front of the first operand load of
+    // every launch (two memory round trips, 2 us of a 31 us launch).
+    // (No branch around the loads -- the values of a branch are waited for where it ends: without an
+    // fp16 output, when the scales may be absent, the loads read the first words of A instead.)
+    float sa_r[4];
+    float4_t sw_r[4];
+    {
+        const float* as = out ? a_scale : reinterpret_cast<const float*>(A);
+        const float* ws = out ? w_scale : reinterpret_cast<const float*>(A);
+        const int m_last = out ? M - 1 : 0, n_last = out ? N - 1 : 0;
+        const int wm0 = m0 + (wave >> 2) * 64, wn0 = n0 + (wave & 3) * 64;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sa_r[i] = as[min(wm0 + i * 16 + l16, m_last)];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sw_r[j][e] = ws[min(wn0 + j * 16 + lg * 4 + e, n_last)];
     }
 
     int4_t acc[4][4];  // [m tile][n tile] of 16 x 16
@@ -225,11 +240,11 @@ __global__ __launch_bounds__(kDmaThreads) void i8_gemm_dma_kernel(
 #pragma unroll
             for (int ii = 0; ii < 2; ++ii) {
                 const int i = ip * 2 + ii;
-                const float sa = s_a[wm + i * 16 + l16];
+                const float sa = sa_r[i];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int nl = j * 16 + lg * 4;
-                    const float4_t sw = *reinterpret_cast<const float4_t*>(s_w + wn + nl);
+                    const float4_t sw = sw_r[j];
                     half4_t h;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
