@@ -355,6 +355,24 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
             dst[j] = __builtin_bit_cast(
                 uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off[j], soff, kBufferStreamAgent));
     };
+    // NORM, two row tiles: the producer's sums of squares are requested ahead of the ring -- loads
+    // return in order, and behind the ring's 8 KiB per wave (and in three dependent steps) they kept
+    // the first stage waiting until long after the whole ring had landed; they are summed after the
+    // first stage's loads have been issued (decode at batch 32: 17.06 -> 16.88 ms per token).  With
+    // one row tile the same order measured slower (batch 1: 8.89 -> 8.97 ms), so there they stay
+    // behind the ring.
+    constexpr bool SSQ_AHEAD = NORM && MT == 2;
+    constexpr int SSQ_PASSES = NORM ? (BM * 32 + 255) / 256 : 1;
+    SsqLane ssq_pre[SSQ_AHEAD ? SSQ_PASSES : 1];
+    if constexpr (SSQ_AHEAD) {
+#pragma unroll
+        for (int pass = 0; pass < SSQ_PASSES; ++pass) {
+            const int row = min(pass * 8 + ((wg_tid & 255) >> 5), M - 1);
+            ssq_pre[pass] = ssq_lane_load(fuse.ssq_in + (size_t)row * fuse.ssq_tiles, fuse.ssq_tiles, wg_tid & 31);
+        }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // ahead of the ring, not among or behind its loads
+    }
 #pragma unroll
     for (int d = 0; d < D; ++d) load_q(q_rsrc, t0, s0 * D + d, qb[d]);
 
@@ -462,12 +480,15 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
         // the first stage) and are folded by shuffles, a fixed order; read back
         // after the K loop
 #pragma unroll
-        for (int pass = 0; pass < (BM * 32 + 255) / 256; ++pass) {
+        for (int pass = 0; pass < SSQ_PASSES; ++pass) {
             const int row = pass * 8 + (tid >> 5), p0 = tid & 31;
             float ss = 0.f;
             if (row < M) {
                 const float* pieces = fuse.ssq_in + (size_t)row * fuse.ssq_tiles;
-                ss = ssq_lane_sum(ssq_lane_load(pieces, fuse.ssq_tiles, p0), pieces, fuse.ssq_tiles, p0);
+                if constexpr (SSQ_AHEAD)
+                    ss = ssq_lane_sum(ssq_pre[pass], pieces, fuse.ssq_tiles, p0);
+                else
+                    ss = ssq_lane_sum(ssq_lane_load(pieces, fuse.ssq_tiles, p0), pieces, fuse.ssq_tiles, p0);
             }
 #pragma unroll
             for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off);
