@@ -194,6 +194,10 @@ __global__ __launch_bounds__(512) void f16_gemv_nk_kernel(const half_t* __restri
             finish(group);
             step = 0;
             ++group;
+            // two waves share a SIMD (of one workgroup of eight waves or of two of four) and the older
+            // one is served first: the priority falls with the row groups a wave has behind it, so
+            // that the younger one does not finish alone
+            set_priority_by_progress(group - first, count);
         }
     }
 }
