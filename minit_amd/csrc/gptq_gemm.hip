@@ -370,7 +370,6 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
             const int row = min(pass * 8 + ((wg_tid & 255) >> 5), M - 1);
             ssq_pre[pass] = ssq_lane_load(fuse.ssq_in + (size_t)row * fuse.ssq_tiles, fuse.ssq_tiles, wg_tid & 31);
         }
-        }
         __builtin_amdgcn_sched_barrier(0);  // ahead of the ring, not among or behind its loads
     }
 #pragma unroll
