@@ -153,6 +153,22 @@ __global__ __launch_bounds__(256) void gptq_gemv_kernel(
     }
 }
 
+// Sum over the splits in split order with eight loads in flight: a loop that loads and adds per
+// iteration is one memory round trip per split (16 splits: 6 of a 7.5 us launch).
+__device__ __forceinline__ float4_t sum_splits_in_order(const float* __restrict__ p, size_t mn, int split_k) {
+    float4_t s = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < split_k; sp += 8) {
+        float4_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)  // past the last split: that split again (a cache hit), not added
+            v[u] = *reinterpret_cast<const float4_t*>(p + (size_t)min(sp + u, split_k - 1) * mn);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (sp + u < split_k) s += v[u];
+    }
+    return s;
+}
+
 // Second stage of split-K for the kernels that do not reduce in place:
 // out[i] = fp16(sum over splits, in split order).  The kernel boundary makes
 // the partials visible without any device-scope fence or atomic.
@@ -161,16 +177,7 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const float* __res
                                                               const half_t* __restrict__ bias, int N) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
-    float4_t s = {0.f, 0.f, 0.f, 0.f};
-    int sp = 0;
-    for (; sp + 8 <= split_k; sp += 8) {
-        float4_t v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4_t*>(partial + (size_t)(sp + u) * mn + i);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
-    }
-    for (; sp < split_k; ++sp) s += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
+    const float4_t s = sum_splits_in_order(partial + i, mn, split_k);
     half4_t h = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
     if (bias) h = h + *reinterpret_cast<const half4_t*>(bias + i % N);  // N % 8 == 0: four columns of one row
     *reinterpret_cast<half4_t*>(out + i) = h;
@@ -186,11 +193,8 @@ __global__ __launch_bounds__(256) void splitk_finalize_silu_kernel(const float* 
     const size_t m = o / half_n, j = o % half_n;
     const size_t gate = m * N + j / 128 * 256 + j % 128;
     const size_t mn = (size_t)M * N;
-    float4_t g = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < split_k; ++sp) {
-        g += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + gate);
-        u += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + gate + 128);
-    }
+    const float4_t g = sum_splits_in_order(partial + gate, mn, split_k);
+    const float4_t u = sum_splits_in_order(partial + gate + 128, mn, split_k);
     half4_t gh = {(half_t)g[0], (half_t)g[1], (half_t)g[2], (half_t)g[3]};
     half4_t uh = {(half_t)u[0], (half_t)u[1], (half_t)u[2], (half_t)u[3]};
     if (bias) {  // column of the gate sum within its row: gate - m * N
@@ -211,14 +215,18 @@ __global__ __launch_bounds__(256) void splitk_finalize_residual_kernel(const flo
     __shared__ float smem[16];
     const size_t mn = (size_t)M * N;
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;  // within one row: N % 1024 == 0
-    float4_t s = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < split_k; ++sp) s += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
+    // the old value of the stream, the next norm's weight and the bias are requested ahead of the
+    // partial sums, whose wait then covers them
+    const half4_t zero4 = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+    const half4_t h_old = *reinterpret_cast<const half4_t*>(h + i);
+    const half4_t nw = fuse.xw_out ? *reinterpret_cast<const half4_t*>(fuse.next_norm_w + i % N) : zero4;
+    const half4_t b4 = fuse.bias ? *reinterpret_cast<const half4_t*>(fuse.bias + i % N) : zero4;
+    const float4_t s = sum_splits_in_order(partial + i, mn, split_k);
     half4_t y = {(half_t)s[0], (half_t)s[1], (half_t)s[2], (half_t)s[3]};
-    if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + i % N);
-    const half4_t r = *reinterpret_cast<const half4_t*>(h + i) + y;  // fp16 add, one rounding
+    if (fuse.bias) y = y + b4;
+    const half4_t r = h_old + y;  // fp16 add, one rounding
     *reinterpret_cast<half4_t*>(h + i) = r;
-    if (fuse.xw_out)
-        *reinterpret_cast<half4_t*>(fuse.xw_out + i) = norm_weighted(r, *reinterpret_cast<const half4_t*>(fuse.next_norm_w + i % N), fuse.xw_clamped);
+    if (fuse.xw_out) *reinterpret_cast<half4_t*>(fuse.xw_out + i) = norm_weighted(r, nw, fuse.xw_clamped);
     float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) ss += (float)r[e] * (float)r[e];
@@ -233,13 +241,13 @@ __global__ __launch_bounds__(256) void splitk_finalize_rope_kernel(const float* 
     const size_t mn = (size_t)M * N;
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
-    float4_t sum = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < split_k; ++sp) sum += *reinterpret_cast<const float4_t*>(partial + (size_t)sp * mn + i);
-    half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
     const int m = (int)(i / N), c = (int)(i % N);
+    // the row's position is requested ahead of the partial sums (its cos / sin hang on it)
+    const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
+    const float4_t sum = sum_splits_in_order(partial + i, mn, split_k);
+    half4_t y = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
     if (fuse.bias) y = y + *reinterpret_cast<const half4_t*>(fuse.bias + c);
     const int head = c / 128, d = c % 128;
-    const int pos = min(max(fuse.positions[m], 0), fuse.max_seq - 1);
     if (head >= fuse.q_heads + fuse.kv_heads) {  // value head: copied, cache is tiled
         half_t* dst = fuse.vt_cache + ((size_t)m * fuse.kv_heads + (head - fuse.q_heads - fuse.kv_heads)) * 128 * fuse.max_seq +
                       vt_offset(d, pos);
