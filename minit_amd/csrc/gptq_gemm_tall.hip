@@ -126,11 +126,13 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     const int pair_col = (blockIdx.x >> 1) * 256 + cg * 128 + (blockIdx.x & 1) * 64;
     const int col = (silu ? pair_col : n0 + cg * 64) + 4 * j;
 
-    const int4_t x_rsrc = tall_rsrc(x, (uint32_t)((size_t)M * K * 2));
-    const int4_t w_rsrc = tall_rsrc(qweight, (uint32_t)((size_t)(K / 8) * N * 4));
-    const int4_t s_rsrc = tall_rsrc(scales, (uint32_t)((size_t)(K / group_size) * N * 2));
-    const int4_t z_rsrc = tall_rsrc(qzeros, (uint32_t)((size_t)(K / group_size) * (N / 8) * 4));
-    const int4_t none = tall_rsrc(x, 0u);  // zero records: no traffic, zeros returned
+    // the descriptors live in fixed scalar registers; past the workgroup's last round their record count is
+    // set to zero (one scalar instruction), and a load moves nothing and returns zeros
+    int4_t x_rsrc = tall_rsrc(x, (uint32_t)((size_t)M * K * 2));
+    int4_t w_rsrc = tall_rsrc(qweight, (uint32_t)((size_t)(K / 8) * N * 4));
+    int4_t s_rsrc = tall_rsrc(scales, (uint32_t)((size_t)(K / group_size) * N * 2));
+    int4_t z_rsrc = tall_rsrc(qzeros, (uint32_t)((size_t)(K / group_size) * (N / 8) * 4));
+    const int x_bytes = x_rsrc[2], w_bytes = w_rsrc[2], s_bytes = s_rsrc[2], z_bytes = z_rsrc[2];
 
     // ---- what a lane fetches per round
     // activations: of the stage's 4 MT pieces of 1 KiB (half h, rows 8p .. 8p+7) this wave loads h = wave / 4,
@@ -155,7 +157,6 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     // group of the step whose loads are issued next / whose constants are built next
     int load_group = __builtin_amdgcn_readfirstlane(k_wave / group_size);
     int load_in_group = __builtin_amdgcn_readfirstlane(k_wave % group_size);
-    int use_in_group = load_in_group;
     // The LR loads that go with step `step`, in their fixed order: piece 0 the packed words, 1 the scales,
     // 2 the zero points (all into ring slot S), 3.. the wave's 1 KiB pieces of the activation stage of round
     // step - 1 (into buffer (step - 1) % NS).  The main loop spreads the pieces over the round's MFMAs: issued
@@ -164,11 +165,17 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     auto issue_piece = [&](auto slot, auto piece, int step) {
         constexpr int S = decltype(slot)::value, I = decltype(piece)::value;
         const bool live = step < n_rounds;
-        if constexpr (I == 0) tall_load_b128_stream(rq[S], w_off, live ? w_rsrc : none, step * 64 * N);
-        if constexpr (I == 1)
-            tall_load_b64(rs[S], s_off, live ? s_rsrc : none, __builtin_amdgcn_readfirstlane(load_group * N * 2));
+        if constexpr (I == 0) {
+            w_rsrc[2] = live ? w_bytes : 0;
+            tall_load_b128_stream(rq[S], w_off, w_rsrc, step * 64 * N);
+        }
+        if constexpr (I == 1) {
+            s_rsrc[2] = live ? s_bytes : 0;
+            tall_load_b64(rs[S], s_off, s_rsrc, __builtin_amdgcn_readfirstlane(load_group * N * 2));
+        }
         if constexpr (I == 2) {
-            tall_load_b32(rz[S], z_off, live ? z_rsrc : none, __builtin_amdgcn_readfirstlane(load_group * (N / 8) * 4));
+            z_rsrc[2] = live ? z_bytes : 0;
+            tall_load_b32(rz[S], z_off, z_rsrc, __builtin_amdgcn_readfirstlane(load_group * (N / 8) * 4));
             load_in_group += kTallRoundK;
             while (load_in_group >= group_size) {
                 load_in_group -= group_size;
@@ -178,7 +185,8 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         if constexpr (I >= 3) {
             const int stage = step - 1;
             const uint32_t base = lds_wave + (uint32_t)((S + NS - 1) % NS) * kStageBytes;
-            tall_load_to_lds(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], stage < n_rounds ? x_rsrc : none, stage * 256);
+            if constexpr (I == 3) x_rsrc[2] = stage < n_rounds ? x_bytes : 0;
+            tall_load_to_lds(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], x_rsrc, stage * 256);
         }
     };
     auto issue = [&](auto slot, int step, bool with_stage) {
@@ -195,21 +203,54 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     // point z <= 15 the fp16 values 1024 + (z + 1) and 64 + (z + 1) are 0x6400 + (z + 1) and 0x5400 +
     // 16 (z + 1) as bit patterns (one unit, one sixteenth per mantissa step), so both pairs are one
     // 24-bit multiply-add of z each.
+    auto make_const = [&](int c, const uint2_t& s, uint32_t z) {
+        const uint32_t zc = (z >> (z_shift + 4 * c)) & 0xFu;
+        const uint32_t sw = s[c >> 1];
+        cc[c].scale = as_half2((c & 1) ? __builtin_amdgcn_perm(sw, sw, 0x07060706u) : __builtin_amdgcn_perm(sw, sw, 0x05040504u));
+        cc[c].zero_lo = as_half2(zc * 0x00010001u + 0x64016401u);
+        cc[c].zero_hi = as_half2(zc * 0x00100010u + 0x54105410u);
+    };
     auto make_consts = [&](const uint2_t& s, uint32_t z) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t zc = (z >> (z_shift + 4 * c)) & 0xFu;
-            const uint32_t sw = s[c >> 1];
-            cc[c].scale = as_half2((c & 1) ? __builtin_amdgcn_perm(sw, sw, 0x07060706u) : __builtin_amdgcn_perm(sw, sw, 0x05040504u));
-            cc[c].zero_lo = as_half2(zc * 0x00010001u + 0x64016401u);
-            cc[c].zero_hi = as_half2(zc * 0x00100010u + 0x54105410u);
-        }
+        for (int c = 0; c < 4; ++c) make_const(c, s, z);
     };
     // one packed word -> the B operand of MFMA tile c: k0 .. k7 of column 4j + c
     auto dequant_piece = [&](half8_t& b, uint32_t word, int c) {
         half2_t w[4];
         dequant_word<4>(word, cc[c], regs, w);
         b = half8_t{w[0][0], w[1][0], w[2][0], w[3][0], w[0][1], w[1][1], w[2][1], w[3][1]};
+    };
+    // the same in four parts of three to five instructions (the arithmetic of dequant_word<4>), so that a
+    // wave never has more than a handful of vector instructions between two MFMAs
+    half2_t wq[4];
+    auto dequant_part = [&](auto part_c, half8_t& b, uint32_t word, int c) {
+        constexpr int part = decltype(part_c)::value;
+        // four independent instructions per part (a chain of dependent ones costs a wait state each); the
+        // empty statement at its end pins a part between the MFMAs it was written between: pure arithmetic
+        // is otherwise placed next to its use, a round later, in one block
+        if constexpr (part == 0) {
+            const uint32_t q8 = word >> 8;
+            wq[0] = as_half2((word & regs.mask_lo) | regs.magic);
+            wq[1] = as_half2((word & regs.mask_hi) | regs.magic);
+            wq[2] = as_half2((q8 & regs.mask_lo) | regs.magic);
+            wq[3] = as_half2((q8 & regs.mask_hi) | regs.magic);
+        }
+        if constexpr (part == 1) {
+            const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+            wq[0] = wq[0] - cc[c].zero_lo;
+            wq[1] = __builtin_elementwise_fma(wq[1], sixteenth, -cc[c].zero_hi);
+            wq[2] = wq[2] - cc[c].zero_lo;
+            wq[3] = __builtin_elementwise_fma(wq[3], sixteenth, -cc[c].zero_hi);
+        }
+        if constexpr (part == 2) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) wq[i] = wq[i] * cc[c].scale;
+        }
+        if constexpr (part < 3) asm volatile("" : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]));
+        if constexpr (part == 3) {
+            b = half8_t{wq[0][0], wq[1][0], wq[2][0], wq[3][0], wq[0][1], wq[1][1], wq[2][1], wq[3][1]};
+            asm volatile("" : "+v"(b));
+        }
     };
 
     // A operand of row tile rt: row rt*16 + j, chunk (ks & 1)*4 + o of the wave's half; the swizzle of
@@ -239,19 +280,13 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         __syncthreads();
         // from here on slot S is free (step r was dequantised last round) and so is the stage buffer of
         // round r - 1: the loads of step r + NS and stage r + NS - 1 go out between the MFMAs below
-        use_in_group += kTallRoundK;
-        if (use_in_group >= group_size) {  // step r + 1 lies in another group than step r
-            do use_in_group -= group_size; while (use_in_group >= group_size);
-            make_consts(rs[S1], rz[S1]);
-        }
         const int8_t* stage = smem + S * kStageBytes + (ks >> 1) * kHalfBytes + a_off;
         half8_t a[MT];
 #pragma unroll
         for (int rt = 0; rt < MT; ++rt) a[rt] = *reinterpret_cast<const half8_t*>(stage + rt * 2048);
         __builtin_amdgcn_sched_barrier(0);
-        // 2 MT pairs of MFMAs; after pair s one of the round's loads and / or the dequantisation of one packed
-        // word of step r + 1: every second pair at eight row tiles (a load) and every fourth (a word), every
-        // pair and every second at four, every pair at two
+        // 2 MT pairs of MFMAs; after pair s one of the round's loads (every second pair at eight row tiles,
+        // every pair below) and a share of the dequantisation of step r + 1
         tall_static_for<0, 2 * MT>([&](auto pair) {
             constexpr int s = decltype(pair)::value;
 #pragma unroll
@@ -260,8 +295,19 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             __builtin_amdgcn_sched_barrier(0);
             constexpr int load = MT == 8 ? ((s & 1) ? s >> 1 : -1) : s;
             if constexpr (load >= 0 && load < LR) issue_piece(slot, std::integral_constant<int, load>{}, r + NS);
-            constexpr int word = MT == 8 ? (s % 4 == 3 ? s / 4 : -1) : MT == 4 ? ((s & 1) ? s >> 1 : -1) : s;
-            if constexpr (word >= 0) dequant_piece(b[P ^ 1][word], rq[S1][word], word);
+            // the dequantisation of step r + 1 in sixteen parts over the 2 MT pairs; a column's constants right
+            // before its word, not in the wait for the first A operand -- every round, from the scales and
+            // zero points that arrive with every step: four instructions that a check for a new group would
+            // not make cheaper
+            constexpr int kParts = 8 / MT;
+            tall_static_for<s * kParts, (s + 1) * kParts>([&](auto g) {
+                constexpr int word = decltype(g)::value / 4, part = decltype(g)::value % 4;
+                if constexpr (part == 0) {
+                    make_const(word, rs[S1], rz[S1]);
+                    asm volatile("" : "+v"(cc[word].scale), "+v"(cc[word].zero_lo), "+v"(cc[word].zero_hi));
+                }
+                dequant_part(std::integral_constant<int, part>{}, b[P ^ 1][word], rq[S1][word], word);
+            });
             __builtin_amdgcn_sched_barrier(0);
         });
     };
