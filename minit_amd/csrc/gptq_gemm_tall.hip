@@ -9,7 +9,7 @@
 // A workgroup of eight waves owns 128 rows x 128 columns over a K range, walked in rounds of
 // 128 k.  Wave (cg, ks) owns all 128 rows x 64 columns (cg = 0, 1) and the ks-th 32 k of every
 // round (ks = 0..3): 8 x 4 MFMA tiles, 128 accumulator registers, so a packed word is
-// dequantised once for 128 rows and the 32 MFMAs of a 32-k step (512 cycles) outweigh its ~80
+// dequantised once for 128 rows and the 32 MFMAs of a 32-k step (512 cycles) outweigh its 84
 // vector instructions.  Lane (j, o) of a
 // wave holds columns 4j..4j+3 of the wave's 64 -- MFMA tile c takes column 4j + c -- and the
 // o-th eight k of the step: its four packed words are one 16-byte load, its four scales one
@@ -27,9 +27,11 @@
 //     load is lane-linear, the XOR swizzle that keeps the A-operand reads (16 rows x one
 //     16-byte chunk per quarter wave) free of bank conflicts is applied to the global address);
 //   * one barrier;
-//   * the 32 MFMAs of step r, with the round's seven loads and the dequantisation of step r + 1 (13 instructions per word
-//     = the bit-exact W of Dequantize, 4 to put the pairs back into k order) placed between
-//     them in four pieces.
+//   * the 32 MFMAs of step r in pairs, with the round's seven loads and the dequantisation of step r + 1
+//     (13 instructions per word = the bit-exact W of Dequantize, 4 to put the pairs back into k order, 4
+//     for the column's constants) placed between the pairs in sixteen parts of four independent
+//     instructions: two vector instructions per MFMA issue in its shadow, more cost 4.6 cycles each,
+//     and one block of 17 behind every eighth MFMA left the matrix pipe idle.
 // At the end the four waves' shares of K are added through LDS (fixed order), the tile is turned into
 // row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias), with
 // kEpilogueSiluPairs silu(gate) * up of a tile made of 64 gate and the 64 matching up columns, or,
@@ -451,9 +453,10 @@ static int tall_min_m() {
 // 57344 109 / 112; with two row tiles at 32 rows it loses (8192 x 57344 77.8 / 67.9, 28672 x 8192 48.6 / 43.5:
 // there the weight stream dominates and the small-M kernel's ring of eight loads per wave hides more
 // latency than this kernel's three rounds), so the switch is at 33 rows (MH_GEMM_TALL_MIN_M moves it).
-// The kernel runs at the power limit of the part (15-20 % faster on all-zero
-// activations); ablations of the main loop at 128 x 8192 x 28672: MFMAs alone 0.58 us per round, loads
-// alone 0.64, together 1.1-1.2.
+// (These figures predate the dequantisation in parts, which made every shape 2-6 % faster.)  A round of 128 k
+// needs 1,765 cycles whatever the data against the 1,024 of its MFMAs (instruction issue: two vector
+// instructions per MFMA are free, the loop has 2.6 plus its scalar ones), and random operands cost 13-19 %
+// of the clock on top (power).
 bool gemm_tall_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_TALL");
     if (off && *off && atoi(off)) return false;
