@@ -49,6 +49,17 @@ __device__ __forceinline__ ColumnConst make_column_const(half_t s, uint32_t z) {
     return c;
 }
 
+// The same constants from the bits of s and the zero point, without conversions: below 2048 an fp16
+// integer n + 1024 is the bit pattern 0x6400 + n, and 64 + n (n < 64) is 0x5400 + 16 n, so each pair is
+// one multiply-add.  (8-bit zero points reach 256: zero_lo still holds, zero_hi is not used there.)
+__device__ __forceinline__ ColumnConst column_const_from_bits(uint32_t sbits, uint32_t z) {
+    ColumnConst c;
+    c.scale = as_half2(sbits * 0x00010001u);
+    c.zero_lo = as_half2((z + 1u) * 0x00010001u + 0x64006400u);
+    c.zero_hi = as_half2((z + 1u) * 0x00100010u + 0x54005400u);
+    return c;
+}
+
 // Bit masks and the fp16 bias kept in registers so that each extraction is a
 // single v_and_or_b32 (VOP3 on gfx9 takes no literals; left as literals the
 // compiler splits it into v_and + v_or).  Build once per kernel.

@@ -454,8 +454,8 @@ __global__ __launch_bounds__(256 * KW) void gptq_gemm_small_kernel(
 #pragma unroll
             for (int j = 0; j < CE; ++j) {
                 const uint32_t z = (zr[j / P] >> ((zsub + j % P) * BITS)) & MASK;
-                const uint16_t sbits = (uint16_t)(sr[j / 2] >> (j % 2 * 16));
-                const ColumnConst k = make_column_const(__builtin_bit_cast(half_t, sbits), z);
+                const uint32_t sbits = (sr[j / 2] >> (j % 2 * 16)) & 0xFFFFu;
+                const ColumnConst k = column_const_from_bits(sbits, z);
                 k_scale[j] = as_u32(k.scale);
                 k_lo[j] = as_u32(k.zero_lo);
                 k_hi[j] = as_u32(k.zero_hi);

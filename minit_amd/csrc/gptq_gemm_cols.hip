@@ -50,17 +50,6 @@ constexpr int kColsStage = 8;   // steps per activation stage
 constexpr int kColsRing = 8;    // steps in flight per wave
 constexpr int kColsParts = 4;  // K ranges of a tile that is cut, when there are more tiles than CUs
 
-// (s, s), (1024 + z + 1) twice, (64 + z + 1) twice from the bits of s and the
-// zero point: below 2048 an fp16 integer n + 1024 is the bit pattern 0x6400 + n,
-// and 64 + n (n < 64) is 0x5400 + 16 n, so each pair is one multiply-add.
-__device__ __forceinline__ ColumnConst column_const_from_bits(uint32_t sbits, uint32_t z) {
-    ColumnConst c;
-    c.scale = as_half2(sbits * 0x00010001u);
-    c.zero_lo = as_half2((z + 1u) * 0x00010001u + 0x64006400u);
-    c.zero_hi = as_half2((z + 1u) * 0x00100010u + 0x54005400u);
-    return c;
-}
-
 template <int BITS, int SPG, int MROWS, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gptq_gemm_cols_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,

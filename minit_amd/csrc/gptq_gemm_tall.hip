@@ -43,8 +43,10 @@
 namespace mh {
 
 constexpr int kTallBN = 128;
-constexpr int kTallRoundK = 128;                 // four waves x one 32-k step
-constexpr int kTallThreads = 512;
+constexpr int kTallRoundK = 128;                 // K must be a multiple of this (four waves x one 32-k step)
+// K shares (waves per column group) of a workgroup: four, or two where a wave owns sixteen row tiles and
+// needs a SIMD's registers for itself
+__host__ __device__ constexpr int tall_k_shares(int mt) { return mt == 16 ? 2 : 4; }
 
 // A compile-time loop: f(integral_constant<int, S>) for S = BEGIN .. END - 1.
 template <int BEGIN, int END, class F>
@@ -84,11 +86,50 @@ __device__ __forceinline__ void tall_load_to_lds(uint32_t lds_addr, int voffset,
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
+// Two such loads behind one write of m0: the second lands 1 KiB further on in LDS through its instruction
+// offset, which the global side adds as well (the caller's voffset1 is 1 KiB short).
+__device__ __forceinline__ void tall_load_to_lds_pair(uint32_t lds_addr, int voffset0, int voffset1, const int4_t& rsrc, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
+                 "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds"
+                 :: "s"(lds_addr), "v"(voffset0), "v"(voffset1), "s"(rsrc), "s"(soffset) : "memory", "m0");
+}
 // Everything but the newest NEWEST loads has arrived; the registers read next pass through the
 // wait, so that no use can be scheduled above it.
 template <int NEWEST>
 __device__ __forceinline__ void tall_wait(uint4_t& q, uint2_t& s, uint32_t& z) {
     asm volatile("s_waitcnt vmcnt(%3)" : "+v"(q), "+v"(s), "+v"(z) : "n"(NEWEST) : "memory");
+}
+
+// The 84 vector instructions that dequantise a step (21 per packed word: code = word * 21 + u, u as in
+// dequant_op below) in the order and grouping in which they go between the MFMAs of the step before: 54
+// units of one or two instructions, never split over two MFMAs.  A packed-fp16 instruction right before an
+// MFMA costs a wait state, so each of them (the subtractions u = 9..12 and multiplications 13..16) is
+// followed by an instruction of the next word that does not depend on it (its constants 0..3, shift 4 and
+// extractions 5..8; words alternate between two sets of temporaries); the re-ordering (17..20) of word 2 is
+// held back to pair with the subtractions of word 3, whose first two multiplications stay alone.
+constexpr int kTallUnits = 54;
+constexpr signed char kTallSchedule[kTallUnits][2] = {
+    {0, -1}, {1, -1}, {2, -1}, {3, -1}, {4, -1}, {5, -1}, {6, -1}, {7, -1}, {8, -1},
+    {9, 21}, {10, 22}, {11, 23}, {12, 24}, {13, 25}, {14, 26}, {15, 27}, {16, 28}, {29, -1},
+    {17, -1}, {18, -1}, {19, -1}, {20, -1}, {30, 42}, {31, 43}, {32, 44}, {33, 45}, {34, 46},
+    {35, 47}, {36, 48}, {37, 49}, {50, -1}, {38, -1}, {39, -1}, {40, -1}, {41, -1}, {51, 63},
+    {52, 64}, {53, 65}, {54, 66}, {55, 67}, {56, 68}, {57, 69}, {58, 70}, {71, -1}, {72, 59},
+    {73, 60}, {74, 61}, {75, 62}, {76, -1}, {77, -1}, {78, 80}, {79, 81}, {82, -1}, {83, -1},
+};
+
+// The A operands are read from LDS by hand as well: the compiler waits before the first use of every one
+// of them (sixteen waits per round at sixteen row tiles), four tiles at a time are enough.
+template <int OFFSET>
+__device__ __forceinline__ void tall_lds_read(half8_t& dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET) : "memory");
+}
+// Everything but the newest NEWEST LDS reads has arrived; the operands read next pass through the wait.
+template <int NEWEST, int COUNT>
+__device__ __forceinline__ void tall_lds_wait(half8_t* a) {
+    if constexpr (COUNT == 4)
+        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]) : "n"(NEWEST) : "memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a[0]), "+v"(a[1]) : "n"(NEWEST) : "memory");
 }
 
 // MT: 16-row MFMA tiles per block of rows (8: blocks of 128 rows; 4: one block of up to 64 rows; 2: up to 32
@@ -98,30 +139,33 @@ __device__ __forceinline__ void tall_wait(uint4_t& q, uint2_t& s, uint32_t& z) {
 // 10240 30.3 against 29.0 -- what holds the kernel back at few rows is its ~105 vector instructions per
 // round, not latency.
 template <int MT, int NS>
-__global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
+__global__ __launch_bounds__(tall_k_shares(MT) * 128) void gptq_gemm_tall_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
     const half_t* __restrict__ scales, half_t* __restrict__ out, float* __restrict__ partial, int M, int N, int K,
     int group_size, int rounds_per_block, int split_k, const half_t* __restrict__ bias, int epilogue) {
     constexpr int BM = 16 * MT;
+    constexpr int KS = tall_k_shares(MT);          // waves per column group, each with 32 k of every round
+    constexpr int RK = 32 * KS;                    // k per round
+    constexpr int kThreads = 2 * KS * 64;
     constexpr int kHalfBytes = BM * 128;           // [row][64 k], chunks swizzled
-    constexpr int kStageBytes = 2 * kHalfBytes;    // the two halves of a round's 128 k
+    constexpr int kStageBytes = (RK / 64) * kHalfBytes;  // the halves of a round's k
     constexpr int PW = MT / 2;                     // 1 KiB pieces of a stage per wave
     constexpr int LR = 3 + PW;                     // loads per wave and round
     constexpr int kRegion = MT * 4096;             // a wave's accumulators in LDS
-    static_assert(MT == 2 || MT == 4 || MT == 8, "two, four or eight row tiles");
+    static_assert(MT == 2 || MT == 4 || MT == 8 || MT == 16, "two, four, eight or sixteen row tiles");
     __shared__ __attribute__((aligned(1024))) int8_t smem[NS * kStageBytes];
-    static_assert(NS * kStageBytes >= 4 * kRegion, "the reduction reuses the stages");
+    static_assert(NS * kStageBytes >= KS * kRegion, "the reduction reuses the stages");
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cg = wave & 1, ks = wave >> 1;
     const int j = lane & 15, o = lane >> 4;
     const int n0 = blockIdx.x * kTallBN, m0 = blockIdx.z * BM;
-    const int rounds_total = K / kTallRoundK;
+    const int rounds_total = K / RK;
     const int r_begin = blockIdx.y * rounds_per_block;
     const int n_rounds = min(rounds_per_block, rounds_total - r_begin);
     // this wave's 32 k of the workgroup's first round
-    const int k_wave = r_begin * kTallRoundK + ks * 32;
+    const int k_wave = r_begin * RK + ks * 32;
     // first of the lane's four columns.  kEpilogueSiluPairs (columns in blocks of 128 gate + 128 up): the
     // tile is 64 gate columns (cg = 0) and the 64 matching up columns (cg = 1) of block blockIdx.x / 2
     const bool silu = epilogue == kEpilogueSiluPairs;
@@ -145,7 +189,10 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     for (int i = 0; i < PW; ++i) {
         const int row = ((wave & 3) * PW + i) * 8 + (lane >> 3);
         const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-        x_off[i] = ((m0 + row) * K + r_begin * kTallRoundK + (wave >> 2) * 64 + chunk * 8) * 2;
+        x_off[i] = ((m0 + row) * K + r_begin * RK + (wave >> 2) * 64 + chunk * 8) * 2;
+        // the odd pieces ride on the even ones' write of m0 with an instruction offset of 1 KiB
+        // (row >= 8 there and K >= 512: the offset stays positive)
+        if (PW > 1 && (i & 1)) x_off[i] -= 1024;
     }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)smem);
     const uint32_t lds_wave = lds0 + (uint32_t)(wave >> 2) * kHalfBytes + (uint32_t)((wave & 3) * PW) * 1024u;
@@ -169,7 +216,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         const bool live = step < n_rounds;
         if constexpr (I == 0) {
             w_rsrc[2] = live ? w_bytes : 0;
-            tall_load_b128_stream(rq[S], w_off, w_rsrc, step * 64 * N);
+            tall_load_b128_stream(rq[S], w_off, w_rsrc, step * (RK / 2) * N);
         }
         if constexpr (I == 1) {
             s_rsrc[2] = live ? s_bytes : 0;
@@ -178,7 +225,7 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         if constexpr (I == 2) {
             z_rsrc[2] = live ? z_bytes : 0;
             tall_load_b32(rz[S], z_off, z_rsrc, __builtin_amdgcn_readfirstlane(load_group * (N / 8) * 4));
-            load_in_group += kTallRoundK;
+            load_in_group += RK;
             while (load_in_group >= group_size) {
                 load_in_group -= group_size;
                 ++load_group;
@@ -188,7 +235,10 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             const int stage = step - 1;
             const uint32_t base = lds_wave + (uint32_t)((S + NS - 1) % NS) * kStageBytes;
             if constexpr (I == 3) x_rsrc[2] = stage < n_rounds ? x_bytes : 0;
-            tall_load_to_lds(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], x_rsrc, stage * 256);
+            if constexpr (PW == 1)
+                tall_load_to_lds(base, x_off[0], x_rsrc, stage * (RK * 2));
+            else if constexpr ((I - 3) % 2 == 0)
+                tall_load_to_lds_pair(base + (uint32_t)(I - 3) * 1024u, x_off[I - 3], x_off[I - 2], x_rsrc, stage * (RK * 2));
         }
     };
     auto issue = [&](auto slot, int step, bool with_stage) {
@@ -222,36 +272,50 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         dequant_word<4>(word, cc[c], regs, w);
         b = half8_t{w[0][0], w[1][0], w[2][0], w[3][0], w[0][1], w[1][1], w[2][1], w[3][1]};
     };
-    // the same in four parts of three to five instructions (the arithmetic of dequant_word<4>), so that a
-    // wave never has more than a handful of vector instructions between two MFMAs
-    half2_t wq[4];
-    auto dequant_part = [&](auto part_c, half8_t& b, uint32_t word, int c) {
-        constexpr int part = decltype(part_c)::value;
-        // four independent instructions per part (a chain of dependent ones costs a wait state each); the
-        // empty statement at its end pins a part between the MFMAs it was written between: pure arithmetic
-        // is otherwise placed next to its use, a round later, in one block
-        if constexpr (part == 0) {
-            const uint32_t q8 = word >> 8;
-            wq[0] = as_half2((word & regs.mask_lo) | regs.magic);
-            wq[1] = as_half2((word & regs.mask_hi) | regs.magic);
-            wq[2] = as_half2((q8 & regs.mask_lo) | regs.magic);
-            wq[3] = as_half2((q8 & regs.mask_hi) | regs.magic);
+    // The same arithmetic (dequant_word<4>, the constants above) one instruction at a time, 21 per packed
+    // word: a wave issues one instruction of any kind in about five cycles, so whatever stands between two
+    // of its MFMAs beyond two or three instructions leaves the matrix pipe waiting.  Instruction u of word c
+    // reads packed word `word` and the step's scales and zero points; the last four write the B operand
+    // registers.  Dependent instructions are at least three apart (next to each other they cost a wait
+    // state); the empty statement pins each between the MFMAs it was written between: pure arithmetic is
+    // otherwise placed next to its use, a round later, in one block.
+    ColumnConst kc[2];
+    uint32_t zc[2], q8[2];
+    half2_t wq[2][4];
+    auto dequant_op = [&](auto op_c, uint4_t& bw, const uint4_t& q4, int c, const uint2_t& sc, uint32_t z) {
+        constexpr int u = decltype(op_c)::value % 21, e = (decltype(op_c)::value / 21) & 1;
+        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+        const uint32_t sw = sc[c >> 1], word = q4[c];
+        auto pin = [&](auto& out) { asm volatile("" : "+v"(out)); };
+        if constexpr (u == 0) { zc[e] = (z >> (z_shift + 4 * c)) & 0xFu; pin(zc[e]); }
+        if constexpr (u == 1) {
+            kc[e].scale = as_half2((c & 1) ? __builtin_amdgcn_perm(sw, sw, 0x07060706u) : __builtin_amdgcn_perm(sw, sw, 0x05040504u));
+            pin(kc[e].scale);
         }
-        if constexpr (part == 1) {
-            const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
-            wq[0] = wq[0] - cc[c].zero_lo;
-            wq[1] = __builtin_elementwise_fma(wq[1], sixteenth, -cc[c].zero_hi);
-            wq[2] = wq[2] - cc[c].zero_lo;
-            wq[3] = __builtin_elementwise_fma(wq[3], sixteenth, -cc[c].zero_hi);
+        if constexpr (u == 2) { kc[e].zero_lo = as_half2(__umul24(zc[e], 0x00010001u) + 0x64016401u); pin(kc[e].zero_lo); }
+        if constexpr (u == 3) { kc[e].zero_hi = as_half2(__umul24(zc[e], 0x00100010u) + 0x54105410u); pin(kc[e].zero_hi); }
+        if constexpr (u == 4) { q8[e] = word >> 8; pin(q8[e]); }
+        if constexpr (u >= 5 && u <= 8) {
+            constexpr int i = u - 5;
+            wq[e][i] = as_half2(((i < 2 ? word : q8[e]) & ((i & 1) ? regs.mask_hi : regs.mask_lo)) | regs.magic);
+            pin(wq[e][i]);
         }
-        if constexpr (part == 2) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) wq[i] = wq[i] * cc[c].scale;
+        if constexpr (u >= 9 && u <= 12) {
+            constexpr int i = u - 9;
+            wq[e][i] = (i & 1) ? __builtin_elementwise_fma(wq[e][i], sixteenth, -kc[e].zero_hi) : wq[e][i] - kc[e].zero_lo;
+            pin(wq[e][i]);
         }
-        if constexpr (part < 3) asm volatile("" : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]));
-        if constexpr (part == 3) {
-            b = half8_t{wq[0][0], wq[1][0], wq[2][0], wq[3][0], wq[0][1], wq[1][1], wq[2][1], wq[3][1]};
-            asm volatile("" : "+v"(b));
+        if constexpr (u >= 13 && u <= 16) {
+            wq[e][u - 13] = wq[e][u - 13] * kc[e].scale;
+            pin(wq[e][u - 13]);
+        }
+        if constexpr (u >= 17) {
+            // registers of the operand: (k0 k1) (k2 k3) (k4 k5) (k6 k7) from the pairs (k0 k4) (k1 k5) (k2 k6) (k3 k7)
+            constexpr int i = u - 17, pr = (i >> 1) * 2;
+            uint32_t r = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, wq[e][pr + 1]), __builtin_bit_cast(uint32_t, wq[e][pr]),
+                                               (i & 1) ? 0x07060302u : 0x05040100u);
+            pin(r);
+            bw[(i & 1) * 2 + (i >> 1)] = r;
         }
     };
 
@@ -263,14 +327,18 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     for (int rt = 0; rt < MT; ++rt)
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[rt][c] = float4_t{0.f, 0.f, 0.f, 0.f};
-    half8_t b[2][4];
+    uint4_t bw[2][4];  // B operands of two steps, as registers
 
     // ---- prologue: the loads of the virtual rounds -NS .. -1, then the operands of step 0
     tall_static_for<0, NS>([&](auto slot) { issue(slot, decltype(slot)::value, decltype(slot)::value != 0); });
     tall_wait<0>(rq[0], rs[0], rz[0]);
     make_consts(rs[0], rz[0]);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) dequant_piece(b[0][c], rq[0][c], c);
+    for (int c = 0; c < 4; ++c) {
+        half8_t b0;
+        dequant_piece(b0, rq[0][c], c);
+        bw[0][c] = __builtin_bit_cast(uint4_t, b0);
+    }
 
     // ---- one round: S = r % NS (ring slot, stage buffer), P = r % 2 (B operand set; NS is even)
     static_assert(NS % 2 == 0, "the B operand sets alternate with the rounds");
@@ -282,33 +350,26 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         __syncthreads();
         // from here on slot S is free (step r was dequantised last round) and so is the stage buffer of
         // round r - 1: the loads of step r + NS and stage r + NS - 1 go out between the MFMAs below
-        const int8_t* stage = smem + S * kStageBytes + (ks >> 1) * kHalfBytes + a_off;
         half8_t a[MT];
-#pragma unroll
-        for (int rt = 0; rt < MT; ++rt) a[rt] = *reinterpret_cast<const half8_t*>(stage + rt * 2048);
+        const uint32_t a_addr = lds0 + (uint32_t)(S * kStageBytes + (ks >> 1) * kHalfBytes + a_off);
+        tall_static_for<0, MT>([&](auto rt) { tall_lds_read<decltype(rt)::value * 2048>(a[decltype(rt)::value], a_addr); });
         __builtin_amdgcn_sched_barrier(0);
-        // 2 MT pairs of MFMAs; after pair s one of the round's loads (every second pair at eight row tiles,
-        // every pair below) and a share of the dequantisation of step r + 1
-        tall_static_for<0, 2 * MT>([&](auto pair) {
-            constexpr int s = decltype(pair)::value;
-#pragma unroll
-            for (int m = 2 * s; m < 2 * s + 2; ++m)
-                acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m >> 2], b[P][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
+        // 4 MT MFMAs; after MFMA m its share of the 54 units that dequantise step r + 1 and, after
+        // every fourth (second at four row tiles, every one at two), one of the round's loads
+        tall_static_for<0, 4 * MT>([&](auto mfma) {
+            constexpr int m = decltype(mfma)::value;
+            constexpr int G = MT < 4 ? MT : 4;  // row tiles per wait
+            if constexpr (m % (4 * G) == 0) tall_lds_wait<MT - (m / 4 + G), G>(&a[m / 4]);
+            acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m >> 2], __builtin_bit_cast(half8_t, bw[P][m & 3]),
+                                                                        acc[m >> 2][m & 3], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            constexpr int load = MT == 8 ? ((s & 1) ? s >> 1 : -1) : s;
+            constexpr int load = MT >= 8 ? (m % 4 == 3 ? m / 4 : -1) : MT == 4 ? (m % 2 == 1 ? m / 2 : -1) : m;
             if constexpr (load >= 0 && load < LR) issue_piece(slot, std::integral_constant<int, load>{}, r + NS);
-            // the dequantisation of step r + 1 in sixteen parts over the 2 MT pairs; a column's constants right
-            // before its word, not in the wait for the first A operand -- every round, from the scales and
-            // zero points that arrive with every step: four instructions that a check for a new group would
-            // not make cheaper
-            constexpr int kParts = 8 / MT;
-            tall_static_for<s * kParts, (s + 1) * kParts>([&](auto g) {
-                constexpr int word = decltype(g)::value / 4, part = decltype(g)::value % 4;
-                if constexpr (part == 0) {
-                    make_const(word, rs[S1], rz[S1]);
-                    asm volatile("" : "+v"(cc[word].scale), "+v"(cc[word].zero_lo), "+v"(cc[word].zero_hi));
-                }
-                dequant_part(std::integral_constant<int, part>{}, b[P ^ 1][word], rq[S1][word], word);
+            tall_static_for<m * kTallUnits / (4 * MT), (m + 1) * kTallUnits / (4 * MT)>([&](auto unit) {
+                constexpr int first = kTallSchedule[decltype(unit)::value][0], second = kTallSchedule[decltype(unit)::value][1];
+                dequant_op(std::integral_constant<int, first>{}, bw[P ^ 1][first / 21], rq[S1], first / 21, rs[S1], rz[S1]);
+                if constexpr (second >= 0)
+                    dequant_op(std::integral_constant<int, second>{}, bw[P ^ 1][second / 21], rq[S1], second / 21, rs[S1], rz[S1]);
             });
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -343,10 +404,12 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
     __syncthreads();
     if (!(ks & 1)) add((ks >> 1) * 2 + cg);
     __syncthreads();
-    if (ks == 2) put(cg);
-    __syncthreads();
-    if (ks == 0) add(cg);
-    __syncthreads();
+    if constexpr (KS == 4) {
+        if (ks == 2) put(cg);
+        __syncthreads();
+        if (ks == 0) add(cg);
+        __syncthreads();
+    }
 
     // ---- results: acc[rt][c][e] of a ks = 0 wave is row rt*16 + o*4 + e, column cg*64 + 4j + c of the tile
     if (split_k == 1) {
@@ -365,8 +428,8 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             // out[m, b*128 + h*64 + c] = silu(gate) * up of the fp16-rounded sums, b = blockIdx.x / 2, h = blockIdx.x % 2
             half_t* dst = out + (blockIdx.x >> 1) * 128 + (blockIdx.x & 1) * 64;
 #pragma unroll
-            for (int i = 0; i < (MT + 3) / 4; ++i) {
-                const int id = i * kTallThreads + tid, row = id >> 3, ch = id & 7;
+            for (int i = 0; i < (BM * 8 + kThreads - 1) / kThreads; ++i) {
+                const int id = i * kThreads + tid, row = id >> 3, ch = id & 7;
                 if (row >= BM || m0 + row >= M) continue;
                 const half8_t g = *reinterpret_cast<const half8_t*>(smem + row * kRow + ch * 16);
                 const half8_t u = *reinterpret_cast<const half8_t*>(smem + row * kRow + 128 + ch * 16);
@@ -378,15 +441,15 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
             return;
         }
 #pragma unroll
-        for (int i = 0; i < MT / 2; ++i) {
-            const int id = i * kTallThreads + tid, row = id >> 4, ch = id & 15;
+        for (int i = 0; i < BM * 16 / kThreads; ++i) {
+            const int id = i * kThreads + tid, row = id >> 4, ch = id & 15;
             const int m = m0 + row, n = n0 + ch * 8;
             if (m >= M || n >= N) continue;
             half8_t h = *reinterpret_cast<const half8_t*>(smem + row * kRow + ch * 16);
             if (bias) h = h + *reinterpret_cast<const half8_t*>(bias + n);
             *reinterpret_cast<half8_t*>(out + (size_t)m * N + n) = h;
         }
-    } else {
+    } else if constexpr (MT <= 8) {  // (sixteen row tiles: the fp32 tile does not fit the LDS; the plan never splits K there)
         constexpr int kRow = 512 + 16;
         if (ks == 0) {
 #pragma unroll
@@ -399,8 +462,8 @@ __global__ __launch_bounds__(kTallThreads) void gptq_gemm_tall_kernel(
         }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int id = i * kTallThreads + tid, row = id >> 5, ch = id & 31;
+        for (int i = 0; i < BM * 32 / kThreads; ++i) {
+            const int id = i * kThreads + tid, row = id >> 5, ch = id & 31;
             const int m = m0 + row, n = n0 + ch * 4;
             if (m >= M || n >= N) continue;
             *reinterpret_cast<float4_t*>(partial + ((size_t)blockIdx.y * M + m) * N + n) =
@@ -415,11 +478,34 @@ struct TallPlan {
     int mt, tiles_n, row_blocks, split_k, rounds_per_block;
 };
 
+// MH_GEMM_TALL_MT16: 0 never blocks of 256 rows, 1 (default) where they pad the rows no further than blocks
+// of 128 and fill the CUs without a split of K, 2 wherever K need not be split.
+static int tall_mt16_mode() {
+    static const int v = [] {
+        const char* e = getenv("MH_GEMM_TALL_MT16");
+        return e && *e ? atoi(e) : 1;
+    }();
+    return v;
+}
+
 static TallPlan plan_tall(int M, int N, int K) {
     TallPlan p;
     p.mt = M <= 32 ? 2 : M <= 64 ? 4 : 8;
-    const int bm = 16 * p.mt;
     p.tiles_n = (N + kTallBN - 1) / kTallBN;
+    if (M > 128 && tall_mt16_mode() != 0) {
+        // blocks of 256 rows: one wave per SIMD, a packed word dequantised once per 256 rows; the whole K per
+        // workgroup (its fp32 tile would not fit the LDS for a split)
+        const int blocks = (M + 255) / 256;
+        const bool same_padding = blocks * 256 == (M + 127) / 128 * 128;
+        if ((same_padding || tall_mt16_mode() == 2) && (long)p.tiles_n * blocks * 8 >= (long)compute_units() * 7) {
+            p.mt = 16;
+            p.row_blocks = blocks;
+            p.split_k = 1;
+            p.rounds_per_block = K / (32 * tall_k_shares(16));
+            return p;
+        }
+    }
+    const int bm = 16 * p.mt;
     p.row_blocks = (M + bm - 1) / bm;
     const int rounds = K / kTallRoundK;
     // one workgroup per CU (eight waves; 128 KiB of LDS at eight row tiles); a workgroup keeps at least four
@@ -487,13 +573,15 @@ int gptq_gemm_tall_launch(hipStream_t stream, const void* x, const int32_t* qwei
                     workspace ? workspace_bytes : (size_t)0);
     float* partial = need ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kTileCounterBytes) : nullptr;
 #define MH_LAUNCH_TALL(MT)                                                                                            \
-    hipLaunchKernelGGL((gptq_gemm_tall_kernel<MT, 4>), dim3(p.tiles_n, p.split_k, p.row_blocks), dim3(kTallThreads), 0, \
+    hipLaunchKernelGGL((gptq_gemm_tall_kernel<MT, 4>), dim3(p.tiles_n, p.split_k, p.row_blocks),                     \
+                       dim3(tall_k_shares(MT) * 128), 0,                                                              \
                        stream, (const half_t*)x, (const uint32_t*)qweight, (const uint32_t*)qzeros,                  \
                        (const half_t*)scales, (half_t*)out, partial, M, N, K, group_size, p.rounds_per_block,        \
                        p.split_k, bias, epilogue)
     switch (p.mt) {
         case 2: MH_LAUNCH_TALL(2); break;
         case 4: MH_LAUNCH_TALL(4); break;
+        case 16: MH_LAUNCH_TALL(16); break;
         default: MH_LAUNCH_TALL(8); break;
     }
 #undef MH_LAUNCH_TALL

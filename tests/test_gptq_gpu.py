@@ -173,7 +173,8 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
 
 
 # More than 64 rows.  K a multiple of 128: blocks of 128 rows with the weights dequantised in registers
-# (K walked in rounds of 128, a quarter per wave, the four shares added through LDS).  Other K that are
+# (K walked in rounds of 128, a quarter per wave, the four shares added through LDS), blocks of 256 rows
+# (rounds of 64, a half per wave) where they fill the CUs without padding or a split of K.  Other K that are
 # multiples of 64, from 192 rows and 192 tiles of 128 x 128: dequantised tiles staged in LDS.
 @pytest.mark.parametrize("m,k,n,group_size", [
     (65, 512, 264, 128),       # one ragged row block, ragged last column tile, four rounds
@@ -187,6 +188,9 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     (192, 6208, 12288, 64),    # K % 128 == 64 -- 2 x 96 tiles, eight waves per workgroup, K split in two
     (1000, 576, 3080, 192),    # K % 128 == 64 -- 8 x 25 tiles, groups longer than a stage
     (512, 8256, 128, 64),      # K % 128 == 64, too few tiles: the 64-row blocks of the small-M kernel
+    (256, 512, 28672, 128),    # blocks of 256 rows (224 tiles, no padding beyond blocks of 128): eight rounds of 64 k
+    (500, 384, 14400, 64),     # ... two row blocks, the second ragged, ragged last column tile, two groups per 128 k
+    (512, 1024, 14336, 256),   # ... groups longer than a round
 ])
 def test_gemm_many_rows(hip, m, k, n, group_size):
     """Rows beyond one block of 64: both kernels that dequantise a packed word once for 128 rows."""
@@ -354,7 +358,8 @@ def test_operator_api_drop_in(hip):
                                      (40, 512, 256),     # 33 to 64 rows, K >= 512: one block of 64 rows, SiLU*up in its store
                                      (40, 384, 256), (64, 256, 128),      # ... K < 512: product, then one pass
                                      (130, 1024, 384), (200, 512, 640),   # 128-row blocks, SiLU*up in their store
-                                     (128, 4096, 512)])  # ... K split over workgroups: product, then one pass
+                                     (128, 4096, 512),   # ... K split over workgroups: product, then one pass
+                                     (256, 512, 14336)])  # 256-row blocks (224 tiles), SiLU*up in their store
 def test_silu_pairs_epilogue(hip, m, k, ffn):
     """gate|up product with SiLU*up applied in the reduction: equals the plain
     product followed by silu(gate) * up on the interleaved column blocks."""
