@@ -284,7 +284,7 @@ def _run_with_bias(hip, x, qweight, qzeros, scales, bias, group_size, bits, g_id
     (4, 512, 28672, 128, 4, False), (8, 4096, 4096, 128, 4, False), (16, 4096, 1024, 128, 4, False),
     (32, 2048, 2048, 64, 4, False), (100, 1088, 1536, 64, 4, False), (130, 4160, 512, 64, 4, False),
     (200, 576, 12288, 64, 4, False), (400, 320, 6144, 64, 4, False), (192, 6208, 12288, 64, 4, False),
-    (128, 4096, 1024, 128, 4, False), (300, 1024, 1032, 128, 4, False),
+    (128, 4096, 1024, 128, 4, False), (300, 1024, 1032, 128, 4, False), (256, 512, 28672, 128, 4, False),
     (1, 2048, 2048, 128, 8, False), (24, 1024, 768, 64, 8, False), (300, 512, 512, 128, 8, False),
     (3, 768, 264, 96, 4, False), (5, 1024, 512, 512, 4, False), (6, 1024, 256, 128, 4, True),
 ])
