@@ -1,16 +1,16 @@
-// GPTQ w4a16 product for blocks of 128 rows: weights dequantised in registers, straight into
+// GPTQ w4a16 product for blocks of 128 (or 256) rows: weights dequantised in registers, straight into
 // the B operand of v_mfma_f32_16x16x32_f16, activations fetched by LDS-destination loads.
 //
 // Replaces the same reference pair as the other product kernels
-// (minit/quantize/dispatch.py:8-11 = Dequantize, then MatrixMultiply) between the small-M
-// kernel (a packed word dequantised once per 64 rows, one wave per SIMD at these sizes) and
-// several hundred rows.
+// (minit/quantize/dispatch.py:8-11 = Dequantize, then MatrixMultiply) above the small-M
+// kernel (a packed word dequantised once per 64 rows, one wave per SIMD at these sizes).
 //
 // A workgroup of eight waves owns 128 rows x 128 columns over a K range, walked in rounds of
 // 128 k.  Wave (cg, ks) owns all 128 rows x 64 columns (cg = 0, 1) and the ks-th 32 k of every
 // round (ks = 0..3): 8 x 4 MFMA tiles, 128 accumulator registers, so a packed word is
 // dequantised once for 128 rows and the 32 MFMAs of a 32-k step (512 cycles) outweigh its 84
-// vector instructions.  Lane (j, o) of a
+// vector instructions.  (Blocks of 256 rows: four waves, one per SIMD, (cg, ks) with ks = 0, 1, rounds
+// of 64 k, 16 x 4 tiles and 256 accumulators per wave, 64 MFMAs per step.)  Lane (j, o) of a
 // wave holds columns 4j..4j+3 of the wave's 64 -- MFMA tile c takes column 4j + c -- and the
 // o-th eight k of the step: its four packed words are one 16-byte load, its four scales one
 // 8-byte load, its four zero points sit in one word.
@@ -27,10 +27,10 @@
 //     load is lane-linear, the XOR swizzle that keeps the A-operand reads (16 rows x one
 //     16-byte chunk per quarter wave) free of bank conflicts is applied to the global address);
 //   * one barrier;
-//   * the 32 MFMAs of step r in pairs, with the round's seven loads and the dequantisation of step r + 1
+//   * the 32 MFMAs of step r, with the round's seven loads and the dequantisation of step r + 1
 //     (13 instructions per word = the bit-exact W of Dequantize, 4 to put the pairs back into k order, 4
-//     for the column's constants) placed between the pairs in sixteen parts of four independent
-//     instructions: two vector instructions per MFMA issue in its shadow, more cost 4.6 cycles each,
+//     for the column's constants) placed between them one or two instructions at a time
+//     (kTallSchedule): two vector instructions per MFMA issue in its shadow, more cost 4.6 cycles each,
 //     and one block of 17 behind every eighth MFMA left the matrix pipe idle.
 // At the end the four waves' shares of K are added through LDS (fixed order), the tile is turned into
 // row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias), with
