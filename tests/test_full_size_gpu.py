@@ -49,6 +49,20 @@ def mistral_weights():
     return host, dense
 
 
+def test_mistral_prefill_rows(hip, mistral_weights):
+    """The same gate and down products over a prefill's worth of rows (2000: blocks of 256 rows, the last
+    one ragged; 896 and 256 workgroups), every output against the float64 oracle."""
+    from minit_amd import synthetic
+    host, dense = mistral_weights
+    hidden, ffn, m = 4096, 14336, 2000
+    x = synthetic.activations("cfg1", f"x{m}", (m, hidden))
+    gate = _linear(hip, _dev(x), *(_dev(t) for t in host["gate"]), m, ffn, hidden).numpy()
+    assert_fp16_close(gate, x.astype(np.float64) @ dense["gate"], what=f"gate M={m}")
+    h = (gate[:, :ffn] * np.float16(0.125)).astype(np.float16)   # activations of the size the block produces
+    y = _linear(hip, _dev(h), *(_dev(t) for t in host["down"]), m, hidden, ffn).numpy()
+    assert_fp16_close(y, h.astype(np.float64) @ dense["down"], what=f"down M={m}")
+
+
 @pytest.mark.parametrize("m", [1, 8, 32, 128])
 def test_mistral_mlp_block(hip, mistral_weights, m):
     """h = SiLU(x Wg) * (x Wu), y = h Wd with K = 4096 -> 14336 -> 4096."""
