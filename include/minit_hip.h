@@ -176,7 +176,7 @@ int mh_gptq_matmul_static(mh_stream_t stream, const void* x, const int32_t* qwei
  * one launch up to 32 rows with group_size in {32, 64, 128, 256} (the epilogue runs
  * in the product's reduction) and, above 32 rows, for 4-bit weights with K a
  * multiple of 128 and at least 512 whose column tiles fill the GPU without a split
- * of K (the epilogue runs in the store of the 64- or 128-row blocks); otherwise the
+ * of K (the epilogue runs in the store of the 64-, 128- or 256-row blocks); otherwise the
  * product goes to the workspace and one more pass applies the epilogue.  The
  * workspace is always required:
  * mh_gptq_silu_pairs_workspace_bytes(M, N, K, ...) bytes, zero-filled once. */
