@@ -191,6 +191,7 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     (256, 512, 28672, 128),    # blocks of 256 rows (224 tiles, no padding beyond blocks of 128): eight rounds of 64 k
     (500, 384, 14400, 64),     # ... two row blocks, the second ragged, ragged last column tile, two groups per 128 k
     (512, 1024, 14336, 256),   # ... groups longer than a round
+    (256, 640, 28800, 32),     # ... two groups per round of 64 k, ten rounds (the ring of four wraps twice), ragged last column tile
 ])
 def test_gemm_many_rows(hip, m, k, n, group_size):
     """Rows beyond one block of 64: both kernels that dequantise a packed word once for 128 rows."""
