@@ -322,6 +322,18 @@ __global__ __launch_bounds__(tall_k_shares(MT) * 128) void gptq_gemm_tall_kernel
     // A operand of row tile rt: row rt*16 + j, chunk (ks & 1)*4 + o of the wave's half; the swizzle of
     // row rt*16 + j does not depend on rt
     const int a_off = tall_swz(j, (ks & 1) * 4 + o);
+    // Which row tile a wave keeps in accumulator rt differs between the waves that share a column group:
+    // rt ^ own, own = the first of the row tiles that the wave ends up with when the K shares are added
+    // (below): with four shares wave ks = 0 the first quarter of the row tiles, 2 the second, 1 the third, 3
+    // the fourth; with two shares a half each.  Every wave then keeps its lowest accumulators and gives away
+    // the others, and no branch decides which registers are touched.  kOwn: row tiles per owner.  (Two row
+    // tiles: wave 0 takes all, own = 0.)
+    constexpr int kOwn = MT < 4 ? MT : (KS == 4 ? MT / 4 : MT / 2);
+    const int own = MT < 4 ? 0 : KS == 4 ? (MT / 2) * (ks & 1) + (MT / 4) * (ks >> 1) : (MT / 2) * ks;
+    // LDS offset of the first of the row tiles behind accumulators [g kOwn, (g + 1) kOwn)
+    int a_group_off[MT / kOwn];
+#pragma unroll
+    for (int g = 0; g < MT / kOwn; ++g) a_group_off[g] = a_off + ((g * kOwn) ^ own) * 2048;
     float4_t acc[MT][4];
 #pragma unroll
     for (int rt = 0; rt < MT; ++rt)
@@ -351,8 +363,10 @@ __global__ __launch_bounds__(tall_k_shares(MT) * 128) void gptq_gemm_tall_kernel
         // from here on slot S is free (step r was dequantised last round) and so is the stage buffer of
         // round r - 1: the loads of step r + NS and stage r + NS - 1 go out between the MFMAs below
         half8_t a[MT];
-        const uint32_t a_addr = lds0 + (uint32_t)(S * kStageBytes + (ks >> 1) * kHalfBytes + a_off);
-        tall_static_for<0, MT>([&](auto rt) { tall_lds_read<decltype(rt)::value * 2048>(a[decltype(rt)::value], a_addr); });
+        const uint32_t a_stage = lds0 + (uint32_t)(S * kStageBytes + (ks >> 1) * kHalfBytes);
+        tall_static_for<0, MT>([&](auto rt) {
+            tall_lds_read<(decltype(rt)::value % kOwn) * 2048>(a[decltype(rt)::value], a_stage + (uint32_t)a_group_off[decltype(rt)::value / kOwn]);
+        });
         __builtin_amdgcn_sched_barrier(0);
         // 4 MT MFMAs; after MFMA m its share of the 54 units that dequantise step r + 1 and, after
         // every fourth (second at four row tiles, every one at two), one of the round's loads
@@ -384,43 +398,63 @@ __global__ __launch_bounds__(tall_k_shares(MT) * 128) void gptq_gemm_tall_kernel
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    // ---- the four quarters of K, added in a fixed order: (0 + 1) + (2 + 3)
-    // a wave's accumulators as 4 MT blocks of 1 KiB, lane-linear on both sides
-    auto put = [&](int region) {
-        float4_t* dst = reinterpret_cast<float4_t*>(smem + region * kRegion) + lane;
-#pragma unroll
-        for (int rt = 0; rt < MT; ++rt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) dst[(rt * 4 + c) * 64] = acc[rt][c];
+    // ---- the K shares of the waves, added in a fixed order: (0 + 1) + (2 + 3)
+    // Waves ks and ks ^ 1 exchange halves of their accumulators, then (four shares) ks and ks ^ 2 halves of
+    // what is left: every wave moves data at every step and ends up with kOwn row tiles, fully summed, in
+    // its lowest accumulators (row tiles own .. own + kOwn - 1).  With one wave collecting everything, three
+    // quarters of the waves sat idle for most of the 4 us behind the main loop.  a + b and b + a are the same
+    // bits, so the sums are those of the tree above whichever wave forms them.
+    // row tiles in accumulators [FIRST, FIRST + COUNT) as COUNT x 4 blocks of 1 KiB, lane-linear on both sides
+    auto put_tiles = [&](auto first, auto count, int8_t* slot) {
+        float4_t* dst = reinterpret_cast<float4_t*>(slot) + lane;
+        tall_static_for<0, decltype(count)::value * 4>([&](auto i) {
+            dst[decltype(i)::value * 64] = acc[decltype(first)::value + decltype(i)::value / 4][decltype(i)::value % 4];
+        });
     };
-    auto add = [&](int region) {
-        const float4_t* src = reinterpret_cast<const float4_t*>(smem + region * kRegion) + lane;
-#pragma unroll
-        for (int rt = 0; rt < MT; ++rt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) acc[rt][c] += src[(rt * 4 + c) * 64];
+    auto add_tiles = [&](auto first, auto count, const int8_t* slot) {
+        const float4_t* src = reinterpret_cast<const float4_t*>(slot) + lane;
+        tall_static_for<0, decltype(count)::value * 4>([&](auto i) {
+            acc[decltype(first)::value + decltype(i)::value / 4][decltype(i)::value % 4] += src[decltype(i)::value * 64];
+        });
     };
-    if (ks & 1) put((ks >> 1) * 2 + cg);
-    __syncthreads();
-    if (!(ks & 1)) add((ks >> 1) * 2 + cg);
-    __syncthreads();
-    if constexpr (KS == 4) {
+    if constexpr (MT >= 4) {
+        constexpr int H = MT / 2;
+        put_tiles(std::integral_constant<int, H>{}, std::integral_constant<int, H>{}, smem + wave * (H * 4096));
+        __syncthreads();
+        add_tiles(std::integral_constant<int, 0>{}, std::integral_constant<int, H>{}, smem + (wave ^ 2) * (H * 4096));
+        __syncthreads();
+        if constexpr (KS == 4) {
+            constexpr int Q = MT / 4;
+            put_tiles(std::integral_constant<int, Q>{}, std::integral_constant<int, Q>{}, smem + wave * (Q * 4096));
+            __syncthreads();
+            add_tiles(std::integral_constant<int, 0>{}, std::integral_constant<int, Q>{}, smem + (wave ^ 4) * (Q * 4096));
+            __syncthreads();
+        }
+    } else {
+        // two row tiles: a wave's accumulators as 4 MT blocks of 1 KiB; wave ks = 0 collects
+        auto put = [&](int region) { put_tiles(std::integral_constant<int, 0>{}, std::integral_constant<int, MT>{}, smem + region * kRegion); };
+        auto add = [&](int region) { add_tiles(std::integral_constant<int, 0>{}, std::integral_constant<int, MT>{}, smem + region * kRegion); };
+        if (ks & 1) put((ks >> 1) * 2 + cg);
+        __syncthreads();
+        if (!(ks & 1)) add((ks >> 1) * 2 + cg);
+        __syncthreads();
         if (ks == 2) put(cg);
         __syncthreads();
         if (ks == 0) add(cg);
         __syncthreads();
     }
+    const bool owner = MT >= 4 || ks == 0;  // holds sums to store
 
-    // ---- results: acc[rt][c][e] of a ks = 0 wave is row rt*16 + o*4 + e, column cg*64 + 4j + c of the tile
+    // ---- results: acc[rt][c][e], rt < kOwn, is row (own + rt)*16 + o*4 + e, column cg*64 + 4j + c of the tile
     if (split_k == 1) {
         constexpr int kRow = 256 + 16;  // bytes per tile row in LDS
-        if (ks == 0) {
+        if (owner) {
 #pragma unroll
-            for (int rt = 0; rt < MT; ++rt)
+            for (int rt = 0; rt < kOwn; ++rt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const half4_t h = {(half_t)acc[rt][0][e], (half_t)acc[rt][1][e], (half_t)acc[rt][2][e], (half_t)acc[rt][3][e]};
-                    *reinterpret_cast<half4_t*>(smem + (rt * 16 + o * 4 + e) * kRow + (cg * 64 + 4 * j) * 2) = h;
+                    *reinterpret_cast<half4_t*>(smem + ((own + rt) * 16 + o * 4 + e) * kRow + (cg * 64 + 4 * j) * 2) = h;
                 }
         }
         __syncthreads();
@@ -451,13 +485,13 @@ __global__ __launch_bounds__(tall_k_shares(MT) * 128) void gptq_gemm_tall_kernel
         }
     } else if constexpr (MT <= 8) {  // (sixteen row tiles: the fp32 tile does not fit the LDS; the plan never splits K there)
         constexpr int kRow = 512 + 16;
-        if (ks == 0) {
+        if (owner) {
 #pragma unroll
-            for (int rt = 0; rt < MT; ++rt)
+            for (int rt = 0; rt < kOwn; ++rt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float4_t v = {acc[rt][0][e], acc[rt][1][e], acc[rt][2][e], acc[rt][3][e]};
-                    *reinterpret_cast<float4_t*>(smem + (rt * 16 + o * 4 + e) * kRow + (cg * 64 + 4 * j) * 4) = v;
+                    *reinterpret_cast<float4_t*>(smem + ((own + rt) * 16 + o * 4 + e) * kRow + (cg * 64 + 4 * j) * 4) = v;
                 }
         }
         __syncthreads();
