@@ -32,8 +32,9 @@
 //     for the column's constants) placed between them one or two instructions at a time
 //     (kTallSchedule): two vector instructions per MFMA issue in its shadow, more cost 4.6 cycles each,
 //     and one block of 17 behind every eighth MFMA left the matrix pipe idle.
-// At the end the four waves' shares of K are added through LDS (fixed order), the tile is turned into
-// row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias), with
+// At the end the waves' shares of K are added through LDS in a fixed order (the waves that meet exchange
+// halves of their accumulators, so that each ends up with its own share of the row tiles), the tile is
+// turned into row-major order in LDS and leaves as 16-byte row pieces: fp16 results (plus bias), with
 // kEpilogueSiluPairs silu(gate) * up of a tile made of 64 gate and the 64 matching up columns, or,
 // with K split over blockIdx.y, fp32 partial sums for splitk_finalize_kernel.
 #include "gptq_common.h"
