@@ -111,8 +111,11 @@ __device__ __forceinline__ float load_agent(const float* p) {
 // 16-byte forms of the two above (the compiler has no vector atomics; sc1 is the
 // agent-scope cache policy it gives the scalar ones).  The load is asynchronous:
 // wait_agent_loads() must come between it and the first use of its result.
+// (The two wait states behind the store: a vector instruction that overwrites the data registers of a
+// store of more than 8 bytes within two wait states corrupts what some lanes store -- the compiler keeps
+// that distance for its own stores and cannot see into this one.)
 __device__ __forceinline__ void store_agent4(float* p, float4_t v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ float4_t load_agent4(const float* p) {
     float4_t v;
