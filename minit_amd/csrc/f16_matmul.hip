@@ -21,7 +21,10 @@ constexpr int kDenseDepth = 8;
 // the a fragment fetched at its point of use, every step waited for the load it
 // had just issued.)  Steps past the end of K re-read the last step and multiply
 // it by a zeroed a fragment.
-template <int MT, int NT>
+//
+// KS = 4: the four waves of a workgroup share one group of 16 NT columns and take a quarter of K each
+// (a weight of few rows gives too few waves for the memory system otherwise); their sums meet in LDS.
+template <int MT, int NT, int KS>
 __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __restrict__ a,
                                                             const half_t* __restrict__ b,
                                                             half_t* __restrict__ out, int M, int N, int K) {
@@ -34,15 +37,17 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
     // a wave owns NT groups of 16 output columns: above 16 rows two groups share every
     // a fragment, which halves the a traffic per byte of b (a comes from the caches,
     // but through the same vector memory path as b)
-    const int n0 = (blockIdx.x * 4 + wave) * (16 * NT);
+    const int n0 = (KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x) * (16 * NT);
     const int m0 = blockIdx.y * (16 * MT);
-    if (n0 >= N) return;
+    if (n0 >= N) return;  // the whole workgroup when its waves share the columns
+    const int steps = K / (32 * KS);  // of this wave
+    const int k_first = KS == 1 ? 0 : wave * steps * 32;
     const half_t* brow[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) brow[nt] = b + (size_t)min(n0 + nt * 16 + i16, N - 1) * K + kq * 8;
+    for (int nt = 0; nt < NT; ++nt) brow[nt] = b + (size_t)min(n0 + nt * 16 + i16, N - 1) * K + kq * 8 + k_first;
     const half_t* arow[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) arow[mt] = a + (size_t)min(m0 + mt * 16 + i16, M - 1) * K + kq * 8;
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = a + (size_t)min(m0 + mt * 16 + i16, M - 1) * K + kq * 8 + k_first;
 
     float4_t acc[MT][NT];
 #pragma unroll
@@ -50,12 +55,17 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int steps = K / 32;
     const int last = steps - 1;
+    // Workgroup i starts four i steps (128 bytes) into its K range and wraps around: started together, all
+    // workgroups ask for the same bytes of rows 2 K bytes apart at once, which fall on a fraction of the
+    // memory channels (3-8 % on weights of 8192 to 128256 rows).
+    const int first = (int)(((uint32_t)blockIdx.x * 4u) % (uint32_t)steps);
     constexpr int D = kDenseDepth;
     uint4_t bq[D][NT], aq[D][MT];
     auto load = [&](int slot, int s) {
-        const size_t off = (size_t)min(s, last) * 32;
+        int at = min(s, last) + first;
+        if (at >= steps) at -= steps;
+        const size_t off = (size_t)at * 32;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
             bq[slot][nt] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow[nt] + off));
@@ -83,6 +93,27 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt], bf[nt], acc[mt][nt], 0, 0, 0);
         }
     }
+    if constexpr (KS > 1) {
+        __shared__ float4_t sums[KS - 1][MT * NT][64];
+        if (wave > 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) sums[wave - 1][mt * NT + nt][lane] = acc[mt][nt];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < KS - 1; ++w)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float4_t v = sums[w][mt * NT + nt][lane];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[mt][nt][r] += v[r];
+                }
+    }
     // acc[mt][nt][r] is row m0 + mt*16 + kq*4 + r, column n0 + nt*16 + i16
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -96,6 +127,14 @@ __global__ __launch_bounds__(256) void f16_matmul_nk_kernel(const half_t* __rest
                 if (m < M) out[(size_t)m * N + n] = (half_t)acc[mt][nt][r];
             }
     }
+}
+
+// The waves of a workgroup share their columns and split K where the plain grid leaves CUs without a
+// workgroup and every wave still keeps a full ring of steps.
+static bool dense_share_k(unsigned workgroups, int K) {
+    static const char* off = getenv("MH_F16_NO_SHARE_K");
+    if (off && *off && atoi(off)) return false;
+    return workgroups < (unsigned)compute_units() && K % 128 == 0 && K / 128 >= kDenseDepth;
 }
 
 // One to eight rows of a (decode): a dot-product kernel.  The MFMA kernel above reads b
@@ -237,7 +276,7 @@ int f16_gemv_prepare() {
 namespace mh {
 // f16_matmul_lds.hip
 bool f16_matmul_lds_supported(int M, int N, int K);
-int f16_matmul_lds_launch(hipStream_t stream, const void* a, const void* b, void* out, int M, int N, int K);
+int f16_matmul_lds_launch(hipStream_t stream, const void* a, const void* b, void* out, int batch, int M, int N, int K);
 }  // namespace mh
 
 using namespace mh;
@@ -285,13 +324,19 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
         return MH_OK;
     }
     // more rows against a long weight: the weight streamed through LDS in whole lines
-    if (f16_matmul_lds_supported(M, N, K)) return f16_matmul_lds_launch(st, a, b, out, M, N, K);
+    if (f16_matmul_lds_supported(M, N, K)) return f16_matmul_lds_launch(st, a, b, out, 1, M, N, K);
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     const int nt = mt == 1 ? 1 : 2;  // columns per wave: 16 or 32
     dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt));
+    const bool share_k = dense_share_k(grid.x * grid.y, K);
+    if (share_k) grid.x = (N + 16 * nt - 1) / (16 * nt);
 #define MH_DENSE(MT, NT)                                                                                            \
-    hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT>), grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, \
-                       (half_t*)out, M, N, K)
+    if (share_k)                                                                                                    \
+        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 4>), grid, dim3(256), 0, st, (const half_t*)a,            \
+                           (const half_t*)b, (half_t*)out, M, N, K);                                                \
+    else                                                                                                            \
+        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 1>), grid, dim3(256), 0, st, (const half_t*)a,            \
+                           (const half_t*)b, (half_t*)out, M, N, K)
     switch (mt) {
         case 1: MH_DENSE(1, 1); break;
         case 2: MH_DENSE(2, 2); break;
@@ -325,13 +370,25 @@ extern "C" int mh_f16_matmul_nk_batched(mh_stream_t stream, const void* a, const
         MH_CHECK_LAUNCH();
         return MH_OK;
     }
+    // (the choice of kernel and tiling is that of the single product, so that a matrix of a batch gets the
+    // bits it gets alone; the LDS kernel's matrices must start on its 128-byte lines' 16-byte pieces, which
+    // `fast` has checked)
+    if (f16_matmul_lds_supported(M, N, K) && (M + 63) / 64 <= 65535)
+        return f16_matmul_lds_launch(st, a, b, out, batch, M, N, K);
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     const int nt = mt == 1 ? 1 : 2;
     dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt), batch);
     MH_REQUIRE(grid.y <= 65535, "mh_f16_matmul_nk_batched: M=%d is too large for one launch", M);
+    // the rule of the single product, so that a matrix of a batch gets the bits it gets alone
+    const bool share_k = dense_share_k(grid.x * grid.y, K);
+    if (share_k) grid.x = (N + 16 * nt - 1) / (16 * nt);
 #define MH_DENSE(MT, NT)                                                                                            \
-    hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT>), grid, dim3(256), 0, st, (const half_t*)a, (const half_t*)b, \
-                       (half_t*)out, M, N, K)
+    if (share_k)                                                                                                    \
+        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 4>), grid, dim3(256), 0, st, (const half_t*)a,            \
+                           (const half_t*)b, (half_t*)out, M, N, K);                                                \
+    else                                                                                                            \
+        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 1>), grid, dim3(256), 0, st, (const half_t*)a,            \
+                           (const half_t*)b, (half_t*)out, M, N, K)
     switch (mt) {
         case 1: MH_DENSE(1, 1); break;
         case 2: MH_DENSE(2, 2); break;

@@ -18,12 +18,10 @@
 // for all row tiles: per round two B-operand reads, 2 MT A-operand reads and 2 MT MFMAs.  Rows of
 // either operand past the end of its matrix are past the end of its buffer and read as zero.
 //
-// Measured, lm_head 128256 x 8192: 467-494 us at 9 to 64 rows (4.3-4.5 TB/s), flat in the row count,
-// against 581-636 us before.  A read-only kernel with this footprint (128-byte pieces of rows 16 KiB
-// apart) reaches 4.7 TB/s where 1 KiB runs reach 6.1-6.8; rounds of 128 k (256-byte pieces, four
-// stages of 40 KiB) measured slower, 494 against 472 us at 32 rows.  Runs of 1 KiB per row and round
-// need 32 rows per workgroup (four times the activation traffic out of L2) and a reduction over K
-// inside it, and were not tried.
+// Measured, lm_head 128256 x 8192: 346-359 us at 9 to 64 rows (5.9-6.1 TB/s), flat in the row count,
+// against 581-636 us before; 467-494 us while every workgroup started at k = 0 (see the start round
+// below).  Rounds of 128 k (256-byte pieces, four stages of 40 KiB) measured slower then, 494 against
+// 472 us at 32 rows.
 #include "common.h"
 
 namespace mh {
@@ -55,11 +53,20 @@ __global__ __launch_bounds__(kLdsThreads) void f16_matmul_nk_lds_kernel(const ha
                                                                          const half_t* __restrict__ b,
                                                                          half_t* __restrict__ out, int M, int N, int K) {
     __shared__ __attribute__((aligned(1024))) int8_t smem[kLdsStages * kLdsStageBytes];
+    // blockIdx.z: the matrix of a batch (a [batch, M, K], b [batch, N, K], out [batch, M, N])
+    a += (size_t)blockIdx.z * M * K;
+    b += (size_t)blockIdx.z * N * K;
+    out += (size_t)blockIdx.z * M * N;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, o = lane >> 4;
     const int n0 = blockIdx.x * kLdsBN, m0 = blockIdx.y * (16 * MT);
     const int rounds = K / kLdsBK;
+    // Workgroup i starts i rounds into K and wraps around.  Started together, every CU of the chip asks for
+    // the same 128 bytes of rows 2 K bytes apart at the same time, and for a K of some KiB those addresses
+    // fall on a fraction of the memory channels: lm_head 128256 x 8192 at 32 rows 471-481 us started
+    // together, 346-356 us staggered by one, seven or 37 rounds, 506-512 us staggered by 16 rounds (2 KiB).
+    const int first = (int)(blockIdx.x % (uint32_t)rounds);
 
     const int4_t w_rsrc = lds_rsrc(b, (uint32_t)((size_t)N * K * 2));
     const int4_t x_rsrc = lds_rsrc(a, (uint32_t)((size_t)M * K * 2));
@@ -80,10 +87,12 @@ __global__ __launch_bounds__(kLdsThreads) void f16_matmul_nk_lds_kernel(const ha
     auto issue_piece = [&](int i, int stage) {
         const uint32_t base = (uint32_t)(stage % kLdsStages) * kLdsStageBytes;
         const bool live = stage < rounds;
+        int at = stage + first;
+        if (at >= rounds) at -= rounds;
         if (i < 2)
-            lds_load(lds_w + base + (uint32_t)i * 1024u, off[i], live ? w_rsrc : none, stage * 128);
+            lds_load(lds_w + base + (uint32_t)i * 1024u, off[i], live ? w_rsrc : none, at * 128);
         else
-            lds_load(lds_x + base, off[2], live ? x_rsrc : none, stage * 128);
+            lds_load(lds_x + base, off[2], live ? x_rsrc : none, at * 128);
     };
 
     float4_t acc[MT];
@@ -136,18 +145,23 @@ __global__ __launch_bounds__(kLdsThreads) void f16_matmul_nk_lds_kernel(const ha
     }
 }
 
-// Shapes this kernel takes from mh_f16_matmul_nk: more rows than the dot-product kernel serves, a weight
-// long enough to give every CU a tile, whole 128-byte lines, 32-bit buffer offsets.
+// Shapes this kernel takes from mh_f16_matmul_nk: more rows than the dot-product kernel serves, whole
+// 128-byte lines, 32-bit buffer offsets.
 bool f16_matmul_lds_supported(int M, int N, int K) {
     static const char* off = getenv("MH_F16_NO_LDS");
     if (off && *off && atoi(off)) return false;
-    return M > 8 && K % kLdsBK == 0 && K >= kLdsBK * kLdsStages && N >= compute_units() * kLdsBN / 2 &&
+    // up to 16 rows against a weight that leaves CUs without a tile, the kernel with MFMA operands straight from
+    // global memory and K split over the waves is ahead (8192 x 8192 at 9 rows 35 us against 45, 4096 x 4096 at
+    // 16 rows 13 against 18); from 17 rows this one is, whatever the number of tiles (1024 x 4096 at 32 rows 17.8
+    // against 22.5, 8192 x 8192 at 64 / 256 / 1024 rows 57 / 57 / 209 against 72 / 206 / 843)
+    const bool enough = M > 16 || N >= compute_units() * kLdsBN / 2;
+    return M > 8 && K % kLdsBK == 0 && K >= kLdsBK * kLdsStages && enough &&
            (size_t)N * K * 2 + (size_t)kLdsBN * K * 2 < ((size_t)1 << 32) && (size_t)M * K * 2 < ((size_t)1 << 31);
 }
 
-int f16_matmul_lds_launch(hipStream_t stream, const void* a, const void* b, void* out, int M, int N, int K) {
+int f16_matmul_lds_launch(hipStream_t stream, const void* a, const void* b, void* out, int batch, int M, int N, int K) {
     const int mt = M <= 32 ? 2 : 4;
-    const dim3 grid((N + kLdsBN - 1) / kLdsBN, (M + 16 * mt - 1) / (16 * mt));
+    const dim3 grid((N + kLdsBN - 1) / kLdsBN, (M + 16 * mt - 1) / (16 * mt), batch);
     if (mt == 2)
         hipLaunchKernelGGL(f16_matmul_nk_lds_kernel<2>, grid, dim3(kLdsThreads), 0, stream, (const half_t*)a,
                            (const half_t*)b, (half_t*)out, M, N, K);

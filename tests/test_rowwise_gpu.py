@@ -200,7 +200,10 @@ def test_sigmoid_multiply_compose_to_silu(hip):
                                    # blocks of 64 rows, the second ragged)
                                    (9, 16390, 448), (33, 16384, 384), (64, 20000, 1024), (70, 16400, 512), (32, 32768, 2048),
                                    # 17 rows (two row tiles, the second ragged) on a ragged last tile of columns; 48 rows (four row tiles, one empty)
-                                   (17, 16390, 640), (48, 16384, 512)])
+                                   (17, 16390, 640), (48, 16384, 512),
+                                   # more than eight rows and a weight of few rows: the four waves of a workgroup split K
+                                   # (one, two and four row tiles, ragged columns, two row blocks, nine steps of 128 k per wave set)
+                                   (16, 200, 1024), (20, 1000, 2048), (100, 520, 1152), (32, 8192, 8192)])
 def test_dense_matmul_nk(hip, m, n, k):
     import minit_amd.functional as F
     rng = np.random.default_rng(10)
@@ -227,7 +230,8 @@ def test_batch_matrix_multiply(hip):
                                          (64, 70, 70, 128),    # 64 heads, four row tiles, ragged
                                          (3, 33, 129, 64),     # two row tiles, ragged columns
                                          (4, 7, 9, 20),        # K not a multiple of 32: the generic kernel
-                                         (1, 12, 300, 96)])    # a batch of one
+                                         (1, 12, 300, 96),     # a batch of one
+                                         (3, 24, 100, 1024)])  # the waves of a workgroup split K
 def test_batched_dense_product_is_one_launch_per_batch(hip, batch, m, n, k):
     """mh_f16_matmul_nk_batched against the oracle's dense product matrix by matrix, and bit for bit
     against the same matrices through mh_f16_matmul_nk one by one."""
