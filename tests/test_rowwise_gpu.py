@@ -231,7 +231,9 @@ def test_batch_matrix_multiply(hip):
                                          (3, 33, 129, 64),     # two row tiles, ragged columns
                                          (4, 7, 9, 20),        # K not a multiple of 32: the generic kernel
                                          (1, 12, 300, 96),     # a batch of one
-                                         (3, 24, 100, 1024)])  # the waves of a workgroup split K
+                                         (3, 24, 100, 1024),   # 17 rows and more, K of 384 and more: the weight through LDS
+                                         (2, 70, 130, 512),    # the same with two blocks of rows and two tiles of columns, both ragged
+                                         (3, 12, 100, 1024)])  # up to 16 rows: the waves of a workgroup split K
 def test_batched_dense_product_is_one_launch_per_batch(hip, batch, m, n, k):
     """mh_f16_matmul_nk_batched against the oracle's dense product matrix by matrix, and bit for bit
     against the same matrices through mh_f16_matmul_nk one by one."""
@@ -247,7 +249,7 @@ def test_batched_dense_product_is_one_launch_per_batch(hip, batch, m, n, k):
     for i in range(batch):
         ref = OG.dense_matmul(a[i], np.ascontiguousarray(b[i].T))
         assert_fp16_close(got[i], ref.astype(np.float64), what=f"batched nk, matrix {i}")
-        if k % 32 == 0 and m <= 64:   # same kernel, same tiling: same bits
+        if k % 32 == 0:   # same kernel, same tiling: same bits
             hip.call("mh_f16_matmul_nk", None, da.data_ptr + i * m * k * 2, db.data_ptr + i * n * k * 2,
                      one.data_ptr, m, n, k)
             np.testing.assert_array_equal(one.numpy().view(np.uint16), got[i].view(np.uint16))
