@@ -281,6 +281,34 @@ int f16_matmul_lds_launch(hipStream_t stream, const void* a, const void* b, void
 
 using namespace mh;
 
+// The MFMA kernels for `batch` matrices (K a multiple of 32, every matrix on a 16-byte boundary): the weight
+// streamed through LDS in whole lines where that kernel serves the shape, operands straight from global
+// memory otherwise.  Kernel and tiling depend on M, N and K only.
+static int launch_dense_mfma(hipStream_t st, const void* a, const void* b, void* out, int batch, int M, int N, int K) {
+    if (f16_matmul_lds_supported(M, N, K) && (M + 63) / 64 <= 65535) return f16_matmul_lds_launch(st, a, b, out, batch, M, N, K);
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    const int nt = mt == 1 ? 1 : 2;  // columns per wave: 16 or 32
+    dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt), batch);
+    MH_REQUIRE(grid.y <= 65535, "dense fp16 product: M=%d is too large for one launch", M);
+    const bool share_k = dense_share_k(grid.x * grid.y, K);
+    if (share_k) grid.x = (N + 16 * nt - 1) / (16 * nt);
+#define MH_DENSE(MT, NT)                                                                                            \
+    if (share_k)                                                                                                    \
+        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 4>), grid, dim3(256), 0, st, (const half_t*)a,            \
+                           (const half_t*)b, (half_t*)out, M, N, K);                                                \
+    else                                                                                                            \
+        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 1>), grid, dim3(256), 0, st, (const half_t*)a,            \
+                           (const half_t*)b, (half_t*)out, M, N, K)
+    switch (mt) {
+        case 1: MH_DENSE(1, 1); break;
+        case 2: MH_DENSE(2, 2); break;
+        default: MH_DENSE(4, 2); break;
+    }
+#undef MH_DENSE
+    MH_CHECK_LAUNCH();
+    return MH_OK;
+}
+
 extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b, void* out, int M, int N,
                                 int K) {
     MH_REQUIRE(M >= 0 && N >= 0 && K >= 0, "mh_f16_matmul_nk: bad shape M=%d N=%d K=%d", M, N, K);
@@ -323,28 +351,7 @@ extern "C" int mh_f16_matmul_nk(mh_stream_t stream, const void* a, const void* b
         MH_CHECK_LAUNCH();
         return MH_OK;
     }
-    // more rows against a long weight: the weight streamed through LDS in whole lines
-    if (f16_matmul_lds_supported(M, N, K)) return f16_matmul_lds_launch(st, a, b, out, 1, M, N, K);
-    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-    const int nt = mt == 1 ? 1 : 2;  // columns per wave: 16 or 32
-    dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt));
-    const bool share_k = dense_share_k(grid.x * grid.y, K);
-    if (share_k) grid.x = (N + 16 * nt - 1) / (16 * nt);
-#define MH_DENSE(MT, NT)                                                                                            \
-    if (share_k)                                                                                                    \
-        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 4>), grid, dim3(256), 0, st, (const half_t*)a,            \
-                           (const half_t*)b, (half_t*)out, M, N, K);                                                \
-    else                                                                                                            \
-        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 1>), grid, dim3(256), 0, st, (const half_t*)a,            \
-                           (const half_t*)b, (half_t*)out, M, N, K)
-    switch (mt) {
-        case 1: MH_DENSE(1, 1); break;
-        case 2: MH_DENSE(2, 2); break;
-        default: MH_DENSE(4, 2); break;
-    }
-#undef MH_DENSE
-    MH_CHECK_LAUNCH();
-    return MH_OK;
+    return launch_dense_mfma(st, a, b, out, 1, M, N, K);
 }
 
 // One launch for a batch of independent products: blockIdx.z (blockIdx.y of the generic kernel)
@@ -370,31 +377,6 @@ extern "C" int mh_f16_matmul_nk_batched(mh_stream_t stream, const void* a, const
         MH_CHECK_LAUNCH();
         return MH_OK;
     }
-    // (the choice of kernel and tiling is that of the single product, so that a matrix of a batch gets the
-    // bits it gets alone; the LDS kernel's matrices must start on its 128-byte lines' 16-byte pieces, which
-    // `fast` has checked)
-    if (f16_matmul_lds_supported(M, N, K) && (M + 63) / 64 <= 65535)
-        return f16_matmul_lds_launch(st, a, b, out, batch, M, N, K);
-    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-    const int nt = mt == 1 ? 1 : 2;
-    dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt), batch);
-    MH_REQUIRE(grid.y <= 65535, "mh_f16_matmul_nk_batched: M=%d is too large for one launch", M);
-    // the rule of the single product, so that a matrix of a batch gets the bits it gets alone
-    const bool share_k = dense_share_k(grid.x * grid.y, K);
-    if (share_k) grid.x = (N + 16 * nt - 1) / (16 * nt);
-#define MH_DENSE(MT, NT)                                                                                            \
-    if (share_k)                                                                                                    \
-        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 4>), grid, dim3(256), 0, st, (const half_t*)a,            \
-                           (const half_t*)b, (half_t*)out, M, N, K);                                                \
-    else                                                                                                            \
-        hipLaunchKernelGGL((f16_matmul_nk_kernel<MT, NT, 1>), grid, dim3(256), 0, st, (const half_t*)a,            \
-                           (const half_t*)b, (half_t*)out, M, N, K)
-    switch (mt) {
-        case 1: MH_DENSE(1, 1); break;
-        case 2: MH_DENSE(2, 2); break;
-        default: MH_DENSE(4, 2); break;
-    }
-#undef MH_DENSE
-    MH_CHECK_LAUNCH();
-    return MH_OK;
+    // the single product's choice of kernel and tiling: a matrix of a batch gets the bits it gets alone
+    return launch_dense_mfma(st, a, b, out, batch, M, N, K);
 }
