@@ -544,14 +544,22 @@ static TallPlan plan_tall(int M, int N, int K) {
     p.row_blocks = (M + bm - 1) / bm;
     const int rounds = K / kTallRoundK;
     // one workgroup per CU (eight waves; 128 KiB of LDS at eight row tiles); a workgroup keeps at least four
-    // rounds, and the fp32 partial sums (8 M N bytes per split, written and read) stay below twice the packed
-    // weights' bytes (below once: 4096 x 4096 at 128 rows 23.0 us against 19.8, 5120 x 5120 26.9 / 22.9,
-    // 1024 x 8192 21.5 / 16.9; below four times: 21.4, 23.8, 16.8)
-    long split = (long)compute_units() / ((long)p.tiles_n * p.row_blocks);
-    if (split > rounds / 4) split = rounds / 4;
-    const long traffic_cap = (long)K / (8L * (M < bm ? M : bm));
-    if (split > traffic_cap) split = traffic_cap;
-    if (split < 1) split = 1;
+    // rounds, and the fp32 partial sums (8 M N bytes per split, written and read) stay below the packed
+    // weights' bytes -- or below twice those where that shortens a workgroup's walk by a quarter or more
+    // (4096 x 4096 at 128 rows 23.0 us with two K ranges against 19.8 with four, 5120 x 5120 26.9 / 22.9,
+    // 1024 x 8192 21.5 / 16.9; below four times: 21.4, 23.8, 16.8; 4096 x 14336 at 128 rows measures the
+    // same with seven and with eight ranges and keeps seven)
+    long most = (long)compute_units() / ((long)p.tiles_n * p.row_blocks);
+    if (most > rounds / 4) most = rounds / 4;
+    const long rows = M < bm ? M : bm;
+    auto capped = [&](long per_rows) {
+        long split = (long)K / (per_rows * rows);
+        if (split > most) split = most;
+        return split < 1 ? 1L : split;
+    };
+    long split = capped(16);
+    const long relaxed = capped(8);
+    if (((rounds + relaxed - 1) / relaxed) * 4 <= ((rounds + split - 1) / split) * 3) split = relaxed;
     p.rounds_per_block = (int)((rounds + split - 1) / split);
     p.split_k = (rounds + p.rounds_per_block - 1) / p.rounds_per_block;
     return p;
