@@ -1054,7 +1054,10 @@ int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
 static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_small(kSmallMaxM, group_size); }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
-    if (gemm_tall_preferred(M, N, K, group_size, bits, kEpilogueNone)) return gemm_tall_workspace_bytes(M, N, K);
+    // Up to kSmallMaxM rows a launch with an epilogue or the norm prologue takes the small-M or the
+    // column-owner kernel where the plain product takes the 128-row-block kernel: the size covers all three.
+    const size_t tall = gemm_tall_preferred(M, N, K, group_size, bits, kEpilogueNone) ? gemm_tall_workspace_bytes(M, N, K) : 0;
+    if (M > kSmallMaxM && gemm_tall_preferred(M, N, K, group_size, bits, kEpilogueNone)) return tall;
     if (gemm_wide_preferred(M, N, K, group_size, bits, kEpilogueNone)) return gemm_wide_workspace_bytes(M, N, K);
     if (row_blocked(M, group_size)) {
         // blocks of kSmallBlockM rows in one launch; partial sums [split][M][N]
@@ -1066,10 +1069,11 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
     const GemmPlan p = plan_gemm(M, N, K, group_size, false), pb = plan_gemm(M, N, K, group_size, true);
     const int slots = p.split_k > pb.split_k ? p.split_k : pb.split_k;
     // the small-M kernel may be asked for an epilogue that goes through the partials even unsplit
-    if (slots <= 1 && !use_small(M, group_size)) return 0;
+    if (slots <= 1 && !use_small(M, group_size)) return tall;
     const size_t small = kTileCounterBytes + (size_t)slots * M * N * sizeof(float);
     const size_t cols = M <= kSmallMaxM ? gemm_cols_workspace_bytes(M, N, K) : 0;
-    return small > cols ? small : cols;
+    const size_t fused = small > cols ? small : cols;
+    return fused > tall ? fused : tall;
 }
 
 template <int BITS, int MT>

@@ -565,12 +565,27 @@ static TallPlan plan_tall(int M, int N, int K) {
     return p;
 }
 
-static int tall_min_m() {
+// MH_GEMM_TALL_MIN_M: the fewest rows that come here whatever the shape (default 33); 0: unset.
+static int tall_min_m_env() {
     static const int v = [] {
         const char* e = getenv("MH_GEMM_TALL_MIN_M");
-        return e && *e ? atoi(e) : 33;
+        return e && *e ? atoi(e) : 0;
     }();
     return v;
+}
+
+// 17 to 32 rows (two row tiles): this kernel where its workgroups are many and their walks short, i.e. where
+// a launch is made of fixed costs rather than of its weight stream.  Measured at 24 rows against the
+// small-M kernel (us, this kernel / small-M): 13824 x 5120 (240 workgroups, 18 rounds) 16.9 / 24.4, 4096 x
+// 12288 (192, 16) 15.6 / 20.1, 4096 x 28672 (224, 32) 20.1 / 23.8, 17920 x 6656 (208, 35) 24.7 / 26.0, 8192 x
+// 16384 (256, 32) 24.1 / 25.2, 8192 x 8192 16.5 / 17.5, 4096 x 4096 10.0 / 10.7; but 8192 x 28672 (224
+// workgroups, 64 rounds) 36.5 / 36.2, 28672 x 8192 (256, 56) 37.0 / 34.6, 8192 x 22016 (172, 64) 36.0 / 32.5,
+// 6656 x 17920 (140 workgroups) 29.5 / 25.4.  Up to 16 rows the small-M kernel's single row tile wins
+// nearly everywhere (8192 x 8192 12.3 against 15.7).
+static bool tall_two_row_tiles_preferred(int M, int N, int K) {
+    if (M < 17 || M > 32) return false;
+    const TallPlan p = plan_tall(M, N, K);
+    return (long)p.tiles_n * p.split_k * 8 >= (long)compute_units() * 5 && p.rounds_per_block <= 40;
 }
 
 // Measured on one box against what served these shapes before (the small-M kernel's 64-row blocks up to
@@ -580,9 +595,10 @@ static int tall_min_m() {
 // 72.0 / 113.5.  Never slower by more than 2 %, so every 4-bit product of more than 64 rows whose K is a
 // multiple of 128 comes here.  With four row tiles (33 to 64 rows) against the small-M kernel's single block
 // of 64 rows, at 64 rows: 8192 x 10240 29.0 / 41.6, 28672 x 8192 55.7 / 62.3, 4096 x 14336 23.9 / 26.3, 8192 x
-// 57344 109 / 112; with two row tiles at 32 rows it loses (8192 x 57344 77.8 / 67.9, 28672 x 8192 48.6 / 43.5:
-// there the weight stream dominates and the small-M kernel's ring of eight loads per wave hides more
-// latency than this kernel's three rounds), so the switch is at 33 rows (MH_GEMM_TALL_MIN_M moves it).
+// 57344 109 / 112; with two row tiles at 32 rows it loses on the largest shapes (8192 x 57344 77.8 / 67.9, 28672
+// x 8192 48.6 / 43.5: there the weight stream dominates and the small-M kernel's ring of eight loads per
+// wave hides more latency than this kernel's three rounds), so every shape comes here from 33 rows and
+// the shapes of tall_two_row_tiles_preferred from 17 (MH_GEMM_TALL_MIN_M sets one switch for all).
 // (These figures predate the dequantisation in parts, which made every shape 2-6 % faster.)  A round of 128 k
 // needs 1,765 cycles whatever the data against the 1,024 of its MFMAs (instruction issue: two vector
 // instructions per MFMA are free, the loop has 2.6 plus its scalar ones), and random operands cost 13-19 %
@@ -590,9 +606,12 @@ static int tall_min_m() {
 bool gemm_tall_preferred(int M, int N, int K, int group_size, int bits, int epilogue) {
     static const char* off = getenv("MH_GEMM_NO_TALL");
     if (off && *off && atoi(off)) return false;
-    return bits == 4 && epilogue == kEpilogueNone && M >= tall_min_m() && K % kTallRoundK == 0 && K >= 4 * kTallRoundK &&
-           group_size % 32 == 0 && K % group_size == 0 && N % 8 == 0 && (size_t)M * K * 2 < ((size_t)1 << 31) &&
-           (size_t)K * N / 2 < ((size_t)1 << 31);
+    if (!(bits == 4 && epilogue == kEpilogueNone && K % kTallRoundK == 0 && K >= 4 * kTallRoundK &&
+          group_size % 32 == 0 && K % group_size == 0 && N % 8 == 0 && (size_t)M * K * 2 < ((size_t)1 << 31) &&
+          (size_t)K * N / 2 < ((size_t)1 << 31)))
+        return false;
+    if (tall_min_m_env() > 0) return M >= tall_min_m_env();
+    return M >= 33 || tall_two_row_tiles_preferred(M, N, K);
 }
 
 size_t gemm_tall_workspace_bytes(int M, int N, int K) {

@@ -192,6 +192,9 @@ def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     (500, 384, 14400, 64),     # ... two row blocks, the second ragged, ragged last column tile, two groups per 128 k
     (512, 1024, 14336, 256),   # ... groups longer than a round
     (256, 640, 28800, 32),     # ... two groups per round of 64 k, ten rounds (the ring of four wraps twice), ragged last column tile
+    (24, 2048, 5120, 128),     # 17 to 32 rows where the workgroups are many and their walks short: two row tiles, 40 tiles x 4 K ranges
+    (31, 2560, 5000, 64),      # ... five K ranges of four rounds, ragged last column tile
+    (17, 512, 20488, 32),      # ... 161 tiles, K unsplit, four groups per round
 ])
 def test_gemm_many_rows(hip, m, k, n, group_size):
     """Rows beyond one block of 64: both kernels that dequantise a packed word once for 128 rows."""
@@ -360,7 +363,8 @@ def test_operator_api_drop_in(hip):
                                      (40, 384, 256), (64, 256, 128),      # ... K < 512: product, then one pass
                                      (130, 1024, 384), (200, 512, 640),   # 128-row blocks, SiLU*up in their store
                                      (128, 4096, 512),   # ... K split over workgroups: product, then one pass
-                                     (256, 512, 14336)])  # 256-row blocks (224 tiles), SiLU*up in their store
+                                     (256, 512, 14336),  # 256-row blocks (224 tiles), SiLU*up in their store
+                                     (24, 512, 14336), (32, 1024, 10240)])  # 17 to 32 rows on many short tiles: two row tiles of the 128-row-block kernel
 def test_silu_pairs_epilogue(hip, m, k, ffn):
     """gate|up product with SiLU*up applied in the reduction: equals the plain
     product followed by silu(gate) * up on the interleaved column blocks."""
