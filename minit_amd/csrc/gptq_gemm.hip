@@ -892,7 +892,7 @@ static const int kFusedReduceMaxM = [] {
 // the fp32 partial sums of a split plan and their second stage cost more than the CUs left idle
 // (8192 x 57344 at 32 rows: 14.7 MB of partial sums each way and a launch).  MH_GEMM_SMALL_KW (read at every
 // call): 2 takes it for every row count it serves, 1 never.
-static bool small_two_shares(int M, int N, int K, int group_size, int row_blocks) {
+static bool small_two_shares(int M, int N, int K, int group_size, int row_blocks, int bits) {
     // (groups of 32 would need 98 KiB of staged constants for the two shares)
     if (row_blocks != 1 || M > kSmallMaxM || group_size < 64) return false;
     const int tiles = (N + kGemmCols - 1) / kGemmCols, cus = compute_units();
@@ -900,17 +900,19 @@ static bool small_two_shares(int M, int N, int K, int group_size, int row_blocks
     if (tiles > cus || 4 * tiles < 3 * cus || stages_total < 2 || tiles > kMaxTileCounters) return false;
     const char* v = getenv("MH_GEMM_SMALL_KW");
     if (v && *v) return atoi(v) == 2;
-    return M > kFusedReduceMaxM;
+    // (8-bit weights at any row count: 8192 x 57344 at 1 / 4 / 8 rows 72.8 / 73.2 / 73.5 us against 77.1-78.5 /
+    // 78.3 / 79.8 on the balanced plan; 4-bit weights at 8 rows 51.0 against 49.1)
+    return M > kFusedReduceMaxM || bits == 8;
 }
 
-GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_blocks = 1, int group_size = 128) {
+GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_blocks = 1, int group_size = 128, int bits = 4) {
     GemmPlan p;
     p.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     p.col_tiles = (N + kGemmCols - 1) / kGemmCols;
     p.m_blocks = row_blocks;
     p.steps_total = K / 32;
     const long stages_total = (p.steps_total + kSmallDepth - 1) / kSmallDepth;
-    if (small_two_shares(M, N, K, group_size, row_blocks)) {
+    if (small_two_shares(M, N, K, group_size, row_blocks, bits)) {
         p.k_ways = 2;
         p.split_k = 1;
         p.steps_per_block = (int)((stages_total + 1) / 2 * kSmallDepth);  // stages of one share
@@ -980,8 +982,8 @@ static bool use_small(int M, int group_size) {
     return !off && M <= kSmallMaxM && (spg == 1 || spg == 2 || spg == 4 || spg == 8);
 }
 
-GemmPlan plan_gemm(int M, int N, int K, int group_size, bool allow_balanced) {
-    if (use_small(M, group_size)) return plan_gemm_small(M, N, K, allow_balanced, 1, group_size);
+GemmPlan plan_gemm(int M, int N, int K, int group_size, bool allow_balanced, int bits) {
+    if (use_small(M, group_size)) return plan_gemm_small(M, N, K, allow_balanced, 1, group_size, bits);
     GemmPlan p;
     p.mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
     const int bm = 16 * p.mt;
@@ -1030,7 +1032,7 @@ bool gemm_norm_fusion_supported(int M, int N, int K, int group_size, int bits, i
     if ((epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
         gemm_cols_preferred(M, N, K, group_size, bits, epilogue))
         return true;
-    if (M <= kFusedReduceMaxM || small_two_shares(M, N, K, group_size, 1))
+    if (M <= kFusedReduceMaxM || small_two_shares(M, N, K, group_size, 1, bits))
         return N % kGemmCols == 0 && (N + kGemmCols - 1) / kGemmCols <= kMaxTileCounters;
     return N % (epilogue == kEpilogueResidual ? 1024 : kGemmCols) == 0;
 }
@@ -1048,7 +1050,7 @@ bool gemm_bias_supported(int M, int N, int K, int group_size, int bits) {
 // Per-row pieces a kEpilogueResidual producer leaves in ssq_out for this shape.
 int gemm_residual_ssq_pieces(int M, int N, int K, int group_size, int bits) {
     if (gemm_cols_preferred(M, N, K, group_size, bits, kEpilogueResidual)) return N / 32;
-    return M <= kFusedReduceMaxM || small_two_shares(M, N, K, group_size, 1) ? N / kGemmCols : N / 1024;
+    return M <= kFusedReduceMaxM || small_two_shares(M, N, K, group_size, 1, bits) ? N / kGemmCols : N / 1024;
 }
 
 static bool row_blocked(int M, int group_size) { return M > kSmallMaxM && use_small(kSmallMaxM, group_size); }
@@ -1066,7 +1068,7 @@ size_t gemm_workspace_bytes(int M, int N, int K, int group_size, int bits) {
         return p.split_k > 1 ? kTileCounterBytes + (size_t)p.split_k * M * N * sizeof(float) : 0;
     }
     // either plan of the small-M kernel may be the one a launch takes
-    const GemmPlan p = plan_gemm(M, N, K, group_size, false), pb = plan_gemm(M, N, K, group_size, true);
+    const GemmPlan p = plan_gemm(M, N, K, group_size, false, bits), pb = plan_gemm(M, N, K, group_size, true, bits);
     const int slots = p.split_k > pb.split_k ? p.split_k : pb.split_k;
     // the small-M kernel may be asked for an epilogue that goes through the partials even unsplit
     if (slots <= 1 && !use_small(M, group_size)) return tall;
@@ -1214,7 +1216,7 @@ int gptq_gemm_launch(hipStream_t stream, const void* x, const int32_t* qweight, 
         MH_CHECK_LAUNCH();
         return MH_OK;
     }
-    const GemmPlan p = plan_gemm(M, N, K, group_size, epilogue == kEpilogueNone && fuse.ssq_in == nullptr);
+    const GemmPlan p = plan_gemm(M, N, K, group_size, epilogue == kEpilogueNone && fuse.ssq_in == nullptr, bits);
     if ((fuse.ssq_in != nullptr || epilogue == kEpilogueResidual || epilogue == kEpilogueRopeAppend) &&
         !gemm_norm_fusion_supported(M, N, K, group_size, bits, epilogue))
         return fail(MH_ERR_INVALID, "gptq gemm: RMSNorm / RoPE fusion needs M <= %d, a group of 32..256 and N %% 256 == 0 "
