@@ -930,6 +930,11 @@ GemmPlan plan_gemm_small(int M, int N, int K, bool allow_balanced, int row_block
     const long cap_unit = M > 32 && row_blocks == 1 ? 16L * M : 32L * M;
     const long traffic_cap = K / cap_unit > 1 ? K / cap_unit : 1;
     if (split > traffic_cap) split = traffic_cap;
+    // a workgroup walks two stages or more: its first stage's round trips stand in front of any arithmetic
+    // (11008 x 4096 at 2 / 8 / 12 rows, one stage per workgroup against two: 8 bit 18.1 / 20.8 / 18.4 us against
+    // 14.0 / 15.3 / 14.7, 4 bit 14.0 / 15.5 / 14.8 against 13.1 / 14.4 / 13.1; at least three: 4096 x 12288 at 12
+    // rows 12.6 -> 16.6 us)
+    if (split > stages_total / 2) split = stages_total / 2;
     if (split < 1) split = 1;
     const long spb = (stages_total + split - 1) / split;
     p.steps_per_block = (int)(spb * kSmallDepth);
