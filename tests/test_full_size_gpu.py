@@ -214,12 +214,16 @@ def test_llama70b_linear_zero_point_weights_give_zero(hip, name, k, n):
     assert not got.any(), f"{name}: {np.count_nonzero(got)} non-zero outputs"
 
 
-@pytest.mark.parametrize("m", [1, 5])
-def test_eight_bit_gate_up_shape_one_hot_rows(hip, m):
-    """8-bit weights at the gate|up shape: the balanced plan of the small-M kernel
-    (a workgroup finishes one tile and begins the next) with two packed rows per
-    8 k; one-hot rows return rows of the dequantized matrix bit for bit."""
+@pytest.mark.parametrize("m,shares", [(1, None), (5, None), (5, "1")])
+def test_eight_bit_gate_up_shape_one_hot_rows(hip, monkeypatch, m, shares):
+    """8-bit weights at the gate|up shape, two packed rows per 8 k: one workgroup of eight
+    waves per column tile whose two K halves meet in LDS (what 8-bit weights take at any
+    row count), and, with that switched off, the balanced plan of the small-M kernel (a
+    workgroup finishes one tile and begins the next); one-hot rows return rows of the
+    dequantized matrix bit for bit."""
     from minit_amd.hip import memory
+    if shares is not None:
+        monkeypatch.setenv("MH_GEMM_SMALL_KW", shares)  # read at every call
     from minit_amd.hip.tensor import HIPTensor
     k, n, bits = 8192, 57344, 8
     per, groups = 32 // bits, k // GROUP
