@@ -60,6 +60,61 @@ def wide_model():
             "final_norm": rng.normal(1, 0.1, CFG["hidden"]).astype(np.float16), "cos": cos, "sin": sin}
 
 
+def test_two_layers_at_70b_widths_eight_bit_weights(hip):
+    """The same widths on 8-bit weights (what the reference's own example ships, examples/qwen1_5_int8.py)
+    at 5 rows: gate|up (224 column tiles) then runs with the two K halves of a tile in one workgroup of
+    eight waves, norm prologue and SiLU epilogue included, which 4-bit weights take only above 8 rows."""
+    from minit_amd import synthetic
+    from minit_amd.decode import LlamaDecoder
+    cport.lib()
+    cfg = dict(CFG, bits=8)
+    batch, d = 5, CFG["head_dim"]
+    rng = np.random.default_rng(78)
+    shapes = {"qkv": (cfg["hidden"], (cfg["n_q_heads"] + 2 * cfg["n_kv_heads"]) * d),
+              "o": (cfg["n_q_heads"] * d, cfg["hidden"]),
+              "gate_up": (cfg["hidden"], 2 * cfg["ffn"]),
+              "down": (cfg["ffn"], cfg["hidden"])}
+    layers = []
+    for l in range(cfg["n_layers"]):
+        layer = {}
+        for name, (k, n) in shapes.items():
+            # zero points around the middle of the range and 16 times finer steps: the weight spread of the
+            # 4-bit model above, then the same 1/16 that keeps the projections around unit size
+            qw, qz, sc = synthetic.gptq_weights("wide70b8", f"{l}.{name}", k, n, cfg["group_size"], 8, zero_range=(120, 135))
+            layer[name] = (qw, qz, (sc.astype(np.float32) / 256).astype(np.float16), cfg["group_size"])
+        layer["input_norm"] = rng.normal(1, 0.1, cfg["hidden"]).astype(np.float16)
+        layer["post_norm"] = rng.normal(1, 0.1, cfg["hidden"]).astype(np.float16)
+        layers.append(layer)
+    cos, sin = OS.rope_tables(d, MAX_SEQ, cfg["rope_theta"])
+    model = {"config": cfg, "layers": layers,
+             "embed": rng.normal(0, 1.0, (cfg["vocab"], cfg["hidden"])).astype(np.float16),
+             "lm_head": rng.normal(0, 0.02, (cfg["vocab"], cfg["hidden"])).astype(np.float16),
+             "final_norm": rng.normal(1, 0.1, cfg["hidden"]).astype(np.float16), "cos": cos, "sin": sin}
+    shape = (batch, cfg["n_kv_heads"], MAX_SEQ, d)
+    k_cache = [rng.standard_normal(shape, np.float32).astype(np.float16) for _ in range(cfg["n_layers"])]
+    v_cache = [rng.standard_normal(shape, np.float32).astype(np.float16) for _ in range(cfg["n_layers"])]
+    tokens = rng.integers(0, cfg["vocab"], batch).astype(np.int32)
+    positions = (CONTEXT - np.arange(batch) * 3).astype(np.int32)
+    dec = LlamaDecoder(cfg, batch, MAX_SEQ)
+    dec.load_host(model, k_cache, v_cache)
+    _, got = dec.decode(tokens, positions, 1, want_logits=True)
+    ref_k, ref_v = [c.copy() for c in k_cache], [c.copy() for c in v_cache]
+    ref = OD.decode_step(model, tokens, positions, ref_k, ref_v, linear=_c_linear)
+    g, r = got.astype(np.float64), ref.astype(np.float64)
+    assert np.isfinite(g).all()
+    rel = np.linalg.norm(g - r) / np.linalg.norm(r)
+    print(f"[70B widths, 8 bit] logits rel L2 {rel:.3g}, worst |err| {np.abs(g - r).max():.3g} of {np.abs(r).max():.3g}", flush=True)
+    assert rel <= 1e-2, f"relative L2 error of the logits {rel:.3g}"
+    assert np.abs(g - r).max() <= 2e-2 * max(1.0, np.abs(r).max())
+    for layer in range(cfg["n_layers"]):
+        kc, vc = dec.k_cache[layer].numpy(), untile_v_cache(dec.v_cache[layer].numpy())
+        tol = 2e-2 if layer == 0 else 6e-2
+        for b in range(batch):
+            pos = int(positions[b])
+            assert np.abs(kc[b, :, pos].astype(np.float64) - ref_k[layer][b, :, pos].astype(np.float64)).max() <= tol
+            assert np.abs(vc[b, :, pos].astype(np.float64) - ref_v[layer][b, :, pos].astype(np.float64)).max() <= tol
+
+
 @pytest.mark.parametrize("batch", [1, 8, 32])
 def test_two_layers_at_70b_widths(hip, wide_model, batch):
     from minit_amd.decode import LlamaDecoder
