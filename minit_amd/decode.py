@@ -337,7 +337,10 @@ def bench_tokens_per_second(batches=(1, 8, 32), context=2048, tokens=128, log=pr
     bmax = max(batches)
     t0 = time.time()
     dec = LlamaDecoder(cfg, bmax, context + tokens + 8)
-    if finite:
+    if finite and cfg["bits"] == 8:
+        # 8-bit sub-words: zero points in the middle of the range and steps 16 times finer again
+        dec.load_synthetic(seed=1, prefill=context, scale_std=0.02 / 256, zero_range=(126, 127))
+    elif finite:
         dec.load_synthetic(seed=1, prefill=context, scale_std=0.02 / 16, zero_range=(6, 7))
     else:
         dec.load_synthetic(seed=1, prefill=context)
@@ -374,7 +377,10 @@ if __name__ == "__main__":
     ap.add_argument("--graph", action="store_true", help="replay one recorded step per token (HIP graph)")
     ap.add_argument("--recipe-as-given", action="store_true",
                     help="weights exactly as the benchmark recipe draws them (activations overflow fp16 after a few layers)")
+    ap.add_argument("--bits", type=int, default=4, choices=(4, 8),
+                    help="bit width of the packed weights (8: what the reference's own example ships)")
     cli = ap.parse_args()
     print(json.dumps(bench_tokens_per_second(batches=tuple(int(b) for b in cli.batches.split(",")),
                                              tokens=cli.tokens, log=lambda *a: print(*a, flush=True),
-                                             graph=cli.graph, finite=not cli.recipe_as_given)))
+                                             graph=cli.graph, finite=not cli.recipe_as_given,
+                                             config=dict(LLAMA3_70B, bits=cli.bits))))
