@@ -642,6 +642,9 @@ def main():
                 raise RuntimeError("skipped (--shapes-only)")
             from minit_amd import decode
             result["extra"]["decode_70b"] = decode.bench_tokens_per_second(batches=(1, 8, 32), tokens=128, log=log)
+            # the same model on 8-bit weights, the bit width of the reference's own example
+            result["extra"]["decode_70b_w8a16"] = decode.bench_tokens_per_second(
+                batches=(1, 32), tokens=64, log=log, config=dict(decode.LLAMA3_70B, bits=8))
         except Exception as exc:
             result["extra"]["decode_70b_error"] = str(exc)
 
