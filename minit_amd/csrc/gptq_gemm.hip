@@ -1107,8 +1107,8 @@ static void launch_gemm_small(hipStream_t stream, const GemmPlan& p, const void*
     // epilogue runs in the launch at any row count, small_two_shares)
     // (a plain product of five to eight rows whose tiles have more than sixteen contributors goes to the second
     // stage all the same: one workgroup reading that many partial tiles is slower than a launch that spreads
-    // them over the chip -- 11008 x 4096 at 5-8 rows 14.0-14.2 -> 12.1-12.7 us, 14336 x 4096 17.0-17.3 -> 13.8-14.9;
-    // with sixteen contributors, 28672 x 8192, 26.3-27.5 us in the kernel against 28.3-30.2)
+    // them over the chip -- 14336 x 4096 at 5-8 rows, 28 contributors, 17.0-17.3 -> 14.2-14.9 us; with sixteen
+    // contributors, 28672 x 8192, 26.3-27.5 us in the kernel against 28.3-30.2)
     const bool many_contributors = epilogue == kEpilogueNone && fuse.ssq_in == nullptr && p.stream_units == 0 &&
                                    M > 4 && p.split_k > 16;
     unsigned* counters = ((M <= kFusedReduceMaxM || (p.k_ways == 2 && p.split_k == 1)) && p.col_tiles <= kMaxTileCounters &&
