@@ -162,7 +162,9 @@ def test_gemm_matches_oracle(hip, m):
 @pytest.mark.parametrize("m,k,n,group_size,bits", [
     (8, 1536, 512, 64, 8), (33, 4096, 256, 32, 4),
     # group sizes the small-M kernel does not serve go to the staged MFMA kernel
-    (5, 1024, 264, 512, 4), (40, 1536, 256, 96, 4), (130, 1024, 520, 512, 4)])
+    (5, 1024, 264, 512, 4), (40, 1536, 256, 96, 4), (130, 1024, 520, 512, 4),
+    # five to eight rows, 28 K ranges per tile: their sums are added by the second stage; four rows: in the kernel
+    (6, 14336, 512, 128, 4), (7, 14336, 512, 128, 8), (4, 14336, 512, 128, 4)])
 def test_gemm_other_layouts(hip, m, k, n, group_size, bits):
     from minit_amd import synthetic
     qweight, qzeros, scales = _weights(k, n, group_size, bits, seed=8)
