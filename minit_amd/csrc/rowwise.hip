@@ -1,8 +1,10 @@
 // RMSNorm, softmax (+ fused causal mask), row reductions, RoPE and SiLU*up.
 //
 // All of these are HBM-bound: one pass over the data where the row fits in
-// registers, 16-byte loads, wave64 shuffle reductions (common.h), one row per
-// workgroup so a launch has as many workgroups as rows.  The view convention is
+// registers, 16-byte loads, wave64 shuffle reductions (common.h).  A row belongs to
+// 16, 64 or all 256 threads of a workgroup by its length (up to 128, 2048, 8192
+// elements), so that short rows do not leave most of a workgroup idle; longer rows
+// are walked twice by one workgroup, the second time out of the caches.  The view convention is
 // the reference's: a tensor is seen as [a, b, c] and the operation runs along b
 // (minit/cuda/dispatch.py:430-478).  c == 1 with 16-bit data takes the
 // vectorised path; anything else takes the strided path.
@@ -32,6 +34,29 @@ __device__ __forceinline__ uint4 pack8(const float* f) {
     return raw;
 }
 
+// Sum / maximum over the LANES threads that share a row: the whole workgroup through LDS, or 16 / 64
+// neighbouring lanes of a wave by shuffles.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v, float* smem) {
+    if constexpr (LANES == kRowThreads) {
+        return block_sum(v, smem);
+    } else {
+#pragma unroll
+        for (int off = LANES / 2; off > 0; off >>= 1) v += __shfl_xor(v, off);
+        return v;
+    }
+}
+template <int LANES>
+__device__ __forceinline__ float group_max(float v, float* smem) {
+    if constexpr (LANES == kRowThreads) {
+        return block_max(v, smem);
+    } else {
+#pragma unroll
+        for (int off = LANES / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+        return v;
+    }
+}
+
 // 16-byte accesses to data that is touched once: keep them from displacing what other
 // workgroups reuse.
 __device__ __forceinline__ uint4 stream_load(const uint4* p) {
@@ -46,11 +71,13 @@ __device__ __forceinline__ void stream_store(uint4* p, const uint4& v) {
 // out = T( x / sqrt(sum(x^2)/b + eps) * w ), fp32 inside
 // (minit/cuda/kernel/cuda/rms_norm.py:69-89).
 
-template <typename T>
+template <typename T, int LANES>
 __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
-    const T* __restrict__ in, const T* __restrict__ weight, T* __restrict__ out, size_t b, float eps) {
+    const T* __restrict__ in, const T* __restrict__ weight, T* __restrict__ out, size_t a, size_t b, float eps) {
     __shared__ float smem[16];
-    const size_t row = blockIdx.x;
+    const size_t row = (size_t)blockIdx.x * (kRowThreads / LANES) + threadIdx.x / LANES;
+    const int lane = threadIdx.x % LANES;
+    if (LANES < kRowThreads && row >= a) return;  // whole groups of LANES threads
     const uint4* src = reinterpret_cast<const uint4*>(in + row * b);
     const uint4* wsrc = reinterpret_cast<const uint4*>(weight);
     uint4* dst = reinterpret_cast<uint4*>(out + row * b);
@@ -61,7 +88,7 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
     // once (streaming hint), the weight by every row (it stays cached)
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
-        const int v = c * kRowThreads + threadIdx.x;
+        const int v = c * LANES + lane;
         if (v < nvec) {
             regs[c] = stream_load(src + v);
             wregs[c] = wsrc[v];
@@ -69,7 +96,7 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
     }
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
-        const int v = c * kRowThreads + threadIdx.x;
+        const int v = c * LANES + lane;
         if (v < nvec) {
             float f[8];
             unpack8<T>(regs[c], f);
@@ -77,14 +104,14 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
             for (int i = 0; i < 8; ++i) ss += f[i] * f[i];
         }
     }
-    ss = block_sum(ss, smem);
+    ss = group_sum<LANES>(ss, smem);
     const float rms = sqrtf(ss / (float)b + eps);
     // 16-bit storage: one division per row; x * (1 / rms) differs from x / rms by an fp32 ulp at most,
     // far below the storage type's step.  fp32 storage keeps the reference's x / rms * w.
     const float inv = 1.0f / rms;
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
-        const int v = c * kRowThreads + threadIdx.x;
+        const int v = c * LANES + lane;
         if (v < nvec) {
             float f[8], w[8];
             unpack8<T>(regs[c], f);
@@ -93,6 +120,39 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
             for (int i = 0; i < 8; ++i) f[i] = sizeof(T) == 2 ? f[i] * inv * w[i] : f[i] / rms * w[i];
             stream_store(dst + v, pack8<T>(f));
         }
+    }
+}
+
+// Rows too long for the registers of a workgroup (more than 8192 elements): the row is walked twice with
+// 16-byte loads, the second time out of the caches (plain loads first, streaming loads and stores last).
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_wide_kernel(
+    const T* __restrict__ in, const T* __restrict__ weight, T* __restrict__ out, size_t b, float eps) {
+    __shared__ float smem[16];
+    const size_t row = blockIdx.x;
+    const uint4* src = reinterpret_cast<const uint4*>(in + row * b);
+    const uint4* wsrc = reinterpret_cast<const uint4*>(weight);
+    uint4* dst = reinterpret_cast<uint4*>(out + row * b);
+    const size_t nvec = b / kRowVec;
+    float ss = 0.f;
+#pragma unroll 4
+    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+        float f[8];
+        unpack8<T>(src[v], f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += f[i] * f[i];
+    }
+    ss = block_sum(ss, smem);
+    const float rms = sqrtf(ss / (float)b + eps);
+    const float inv = 1.0f / rms;
+#pragma unroll 4
+    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+        float f[8], w[8];
+        unpack8<T>(stream_load(src + v), f);
+        unpack8<T>(wsrc[v], w);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = sizeof(T) == 2 ? f[i] * inv * w[i] : f[i] / rms * w[i];
+        stream_store(dst + v, pack8<T>(f));
     }
 }
 
@@ -125,11 +185,13 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_strided_kernel(
 // scaled score is rounded to T as the separate divide kernel would, and
 // positions j > offset + i contribute exp(-inf) = 0.
 
-template <typename T, bool CAUSAL>
+template <typename T, bool CAUSAL, int LANES>
 __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
-    const T* __restrict__ in, T* __restrict__ out, size_t b, size_t s, size_t offset, float scale) {
+    const T* __restrict__ in, T* __restrict__ out, size_t a, size_t b, size_t s, size_t offset, float scale) {
     __shared__ float smem[16];
-    const size_t row = blockIdx.x;
+    const size_t row = (size_t)blockIdx.x * (kRowThreads / LANES) + threadIdx.x / LANES;
+    const int lane = threadIdx.x % LANES;
+    if (LANES < kRowThreads && row >= a) return;
     const uint4* src = reinterpret_cast<const uint4*>(in + row * b);
     uint4* dst = reinterpret_cast<uint4*>(out + row * b);
     const int nvec = (int)(b / kRowVec);
@@ -138,7 +200,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
     float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
-        const int v = c * kRowThreads + threadIdx.x;
+        const int v = c * LANES + lane;
         if (v < nvec) {
             const uint4 raw = stream_load(src + v);
             unpack8<T>(raw, vals[c]);
@@ -154,11 +216,11 @@ __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
             }
         }
     }
-    mx = block_max(mx, smem);
+    mx = group_max<LANES>(mx, smem);
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
-        const int v = c * kRowThreads + threadIdx.x;
+        const int v = c * LANES + lane;
         if (v < nvec) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -170,16 +232,67 @@ __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
             }
         }
     }
-    sum = block_sum(sum, smem);
+    sum = group_sum<LANES>(sum, smem);
     const float inv = 1.0f / sum;  // one division per row for 16-bit storage
 #pragma unroll
     for (int c = 0; c < kRowMaxChunks; ++c) {
-        const int v = c * kRowThreads + threadIdx.x;
+        const int v = c * LANES + lane;
         if (v < nvec) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) vals[c][i] = sizeof(T) == 2 ? vals[c][i] * inv : vals[c][i] / sum;
             stream_store(dst + v, pack8<T>(vals[c]));
         }
+    }
+}
+
+// Rows of more than 8192 elements: maximum, sum and store in three walks over the row with 16-byte loads, the
+// second and third out of the caches; the arithmetic of softmax_rows_kernel.
+template <typename T, bool CAUSAL>
+__global__ __launch_bounds__(kRowThreads) void softmax_wide_kernel(
+    const T* __restrict__ in, T* __restrict__ out, size_t b, size_t s, size_t offset, float scale) {
+    __shared__ float smem[16];
+    const size_t row = blockIdx.x;
+    const uint4* src = reinterpret_cast<const uint4*>(in + row * b);
+    uint4* dst = reinterpret_cast<uint4*>(out + row * b);
+    const size_t nvec = b / kRowVec;
+    const long limit = CAUSAL ? (long)(offset + row % s) : (long)b;
+    auto fetch = [&](size_t v, bool last, float* x) {
+        unpack8<T>(last ? stream_load(src + v) : src[v], x);
+        if (CAUSAL) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (scale != 1.f) x[i] = Cvt<T>::to_f32(Cvt<T>::from_f32(x[i] * scale));
+                if ((long)v * 8 + i > limit) x[i] = -INFINITY;
+            }
+        }
+    };
+    auto expd = [](float d) { return sizeof(T) == 2 ? __builtin_amdgcn_exp2f(d * 1.44269504088896340736f) : expf(d); };
+    float mx = -INFINITY;
+#pragma unroll 4
+    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+        float x[8];
+        fetch(v, false, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) mx = fmaxf(mx, x[i]);
+    }
+    mx = block_max(mx, smem);
+    float sum = 0.f;
+#pragma unroll 4
+    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+        float x[8];
+        fetch(v, false, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += expd(x[i] - mx);
+    }
+    sum = block_sum(sum, smem);
+    const float inv = 1.0f / sum;
+#pragma unroll 4
+    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+        float x[8];
+        fetch(v, true, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = sizeof(T) == 2 ? expd(x[i] - mx) * inv : expd(x[i] - mx) / sum;
+        stream_store(dst + v, pack8<T>(x));
     }
 }
 
@@ -224,28 +337,30 @@ __device__ __forceinline__ T mean_of_sum(float sum, size_t b) {
     return Cvt<T>::from_f32(s / n);
 }
 
-template <typename T, bool IS_MAX, bool MEAN = false>
+template <typename T, bool IS_MAX, bool MEAN, int LANES>
 __global__ __launch_bounds__(kRowThreads) void reduce_rows_kernel(const T* __restrict__ in,
-                                                                 T* __restrict__ out, size_t b) {
+                                                                 T* __restrict__ out, size_t a, size_t b) {
     __shared__ float smem[16];
-    const size_t row = blockIdx.x;
+    const size_t row = (size_t)blockIdx.x * (kRowThreads / LANES) + threadIdx.x / LANES;
+    const int lane = threadIdx.x % LANES;
+    if (LANES < kRowThreads && row >= a) return;
     const T* src = in + row * b;
     float acc = IS_MAX ? -INFINITY : 0.f;
     const size_t nvec = (sizeof(T) == 2 && (uintptr_t)src % 16 == 0) ? b / kRowVec : 0;
     const uint4* vsrc = reinterpret_cast<const uint4*>(src);
-    for (size_t v = threadIdx.x; v < nvec; v += blockDim.x) {
+    for (size_t v = lane; v < nvec; v += LANES) {
         float f[8];
         const uint4 raw = vsrc[v];
         unpack8<T>(raw, f);
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc = IS_MAX ? fmaxf(acc, f[i]) : acc + f[i];
     }
-    for (size_t j = nvec * kRowVec + threadIdx.x; j < b; j += blockDim.x) {
+    for (size_t j = nvec * kRowVec + lane; j < b; j += LANES) {
         const float f = Cvt<T>::to_f32(src[j]);
         acc = IS_MAX ? fmaxf(acc, f) : acc + f;
     }
-    acc = IS_MAX ? block_max(acc, smem) : block_sum(acc, smem);
-    if (threadIdx.x == 0) out[row] = MEAN ? mean_of_sum<T>(acc, b) : Cvt<T>::from_f32(acc);
+    acc = IS_MAX ? group_max<LANES>(acc, smem) : group_sum<LANES>(acc, smem);
+    if (lane == 0) out[row] = MEAN ? mean_of_sum<T>(acc, b) : Cvt<T>::from_f32(acc);
 }
 
 // c > 1: one thread per output element, coalesced across c.
@@ -384,17 +499,36 @@ static unsigned grid_for(size_t work_items, int per_block) {
     return (unsigned)blocks;
 }
 
-static bool rows_fast_path(const void* in, const void* out, size_t b, size_t c, size_t elem) {
-    return c == 1 && elem == 2 && b % kRowVec == 0 && b <= (size_t)kRowThreads * kRowVec * kRowMaxChunks &&
-           ((uintptr_t)in | (uintptr_t)out) % 16 == 0;
+// Contiguous rows of 16-bit elements in whole 16-byte pieces: the vectorised kernels.
+static bool rows_vector_path(const void* in, const void* out, size_t b, size_t c, size_t elem) {
+    return c == 1 && elem == 2 && b % kRowVec == 0 && ((uintptr_t)in | (uintptr_t)out) % 16 == 0;
+}
+static bool rows_fit_registers(size_t b) { return b <= (size_t)kRowThreads * kRowVec * kRowMaxChunks; }
+// Threads per row: 16 up to 128 elements, 64 up to 2048 (one to four 16-byte pieces per lane), else the workgroup.
+static int rows_lanes(size_t b) { return b <= 16 * kRowVec ? 16 : b <= 64 * kRowVec * kRowMaxChunks ? 64 : kRowThreads; }
+static unsigned rows_grid(size_t a, int lanes) {
+    const size_t per = kRowThreads / lanes;
+    return (unsigned)((a + per - 1) / per);
 }
 
 template <typename T>
 static int rms_norm_t(hipStream_t st, const void* in, const void* weight, void* out, size_t a, size_t b,
                       size_t c, float eps) {
-    if (rows_fast_path(in, out, b, c, sizeof(T)) && (uintptr_t)weight % 16 == 0) {
-        hipLaunchKernelGGL(rms_norm_rows_kernel<T>, dim3((unsigned)a), dim3(kRowThreads), 0, st, (const T*)in,
-                           (const T*)weight, (T*)out, b, eps);
+    if (rows_vector_path(in, out, b, c, sizeof(T)) && (uintptr_t)weight % 16 == 0) {
+        const int lanes = rows_lanes(b);
+#define MH_RMS_ROWS(LANES)                                                                                           \
+    hipLaunchKernelGGL((rms_norm_rows_kernel<T, LANES>), dim3(rows_grid(a, LANES)), dim3(kRowThreads), 0, st, (const T*)in, \
+                       (const T*)weight, (T*)out, a, b, eps)
+        if (!rows_fit_registers(b))
+            hipLaunchKernelGGL(rms_norm_wide_kernel<T>, dim3((unsigned)a), dim3(kRowThreads), 0, st, (const T*)in,
+                               (const T*)weight, (T*)out, b, eps);
+        else if (lanes == 16)
+            MH_RMS_ROWS(16);
+        else if (lanes == 64)
+            MH_RMS_ROWS(64);
+        else
+            MH_RMS_ROWS(kRowThreads);
+#undef MH_RMS_ROWS
     } else {
         hipLaunchKernelGGL(rms_norm_strided_kernel<T>, dim3(grid_for(a * c, 1)), dim3(kRowThreads), 0, st,
                            (const T*)in, (const T*)weight, (T*)out, a, b, c, eps);
@@ -406,9 +540,21 @@ static int rms_norm_t(hipStream_t st, const void* in, const void* weight, void* 
 template <typename T, bool CAUSAL>
 static int softmax_t(hipStream_t st, const void* in, void* out, size_t a, size_t b, size_t c, size_t s,
                      size_t offset, float scale) {
-    if (rows_fast_path(in, out, b, c, sizeof(T))) {
-        hipLaunchKernelGGL((softmax_rows_kernel<T, CAUSAL>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
-                           (const T*)in, (T*)out, b, s, offset, scale);
+    if (rows_vector_path(in, out, b, c, sizeof(T))) {
+        const int lanes = rows_lanes(b);
+#define MH_SOFTMAX_ROWS(LANES)                                                                                       \
+    hipLaunchKernelGGL((softmax_rows_kernel<T, CAUSAL, LANES>), dim3(rows_grid(a, LANES)), dim3(kRowThreads), 0, st, \
+                       (const T*)in, (T*)out, a, b, s, offset, scale)
+        if (!rows_fit_registers(b))
+            hipLaunchKernelGGL((softmax_wide_kernel<T, CAUSAL>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
+                               (const T*)in, (T*)out, b, s, offset, scale);
+        else if (lanes == 16)
+            MH_SOFTMAX_ROWS(16);
+        else if (lanes == 64)
+            MH_SOFTMAX_ROWS(64);
+        else
+            MH_SOFTMAX_ROWS(kRowThreads);
+#undef MH_SOFTMAX_ROWS
     } else {
         hipLaunchKernelGGL((softmax_strided_kernel<T, CAUSAL>), dim3(grid_for(a * c, 1)), dim3(kRowThreads), 0,
                            st, (const T*)in, (T*)out, a, b, c, s, offset, scale);
@@ -420,8 +566,17 @@ static int softmax_t(hipStream_t st, const void* in, void* out, size_t a, size_t
 template <typename T, bool IS_MAX, bool MEAN = false>
 static int reduce_t(hipStream_t st, const void* in, void* out, size_t a, size_t b, size_t c) {
     if (c == 1) {
-        hipLaunchKernelGGL((reduce_rows_kernel<T, IS_MAX, MEAN>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
-                           (const T*)in, (T*)out, b);
+        const int lanes = rows_lanes(b);
+#define MH_REDUCE_ROWS(LANES)                                                                                        \
+    hipLaunchKernelGGL((reduce_rows_kernel<T, IS_MAX, MEAN, LANES>), dim3(rows_grid(a, LANES)), dim3(kRowThreads), 0, \
+                       st, (const T*)in, (T*)out, a, b)
+        if (lanes == 16)
+            MH_REDUCE_ROWS(16);
+        else if (lanes == 64)
+            MH_REDUCE_ROWS(64);
+        else
+            MH_REDUCE_ROWS(kRowThreads);
+#undef MH_REDUCE_ROWS
     } else {
         hipLaunchKernelGGL((reduce_strided_kernel<T, IS_MAX, MEAN>), dim3(grid_for(a * c, 256)), dim3(256), 0, st,
                            (const T*)in, (T*)out, a, b, c);

@@ -33,6 +33,12 @@ def _assert_ulp(got, ref, ulps=1.0, atol=1e-6, what=""):
     ((3, 5, 264), 2),
     ((2, 100, 6), 1),       # normalise a middle axis (strided path)
     ((7, 33), 1),           # not a multiple of the vector width
+    ((37, 128), 1),         # 16 threads per row, 16 rows per workgroup, the last workgroup part empty
+    ((2, 19, 64), 2),       # ... half of the 16 threads of a row without a piece
+    ((21, 520), 1),         # 64 threads per row, two pieces per lane, the second part empty
+    ((9, 2048), 1),         # ... four pieces per lane
+    ((5, 16384), 1),        # longer than the registers of a workgroup: two walks over the row
+    ((3, 28680), 1),        # ... a length that is no multiple of the workgroup's stride
 ])
 def test_rms_norm(hip, shape, axis):
     import minit_amd.functional as F
@@ -91,6 +97,11 @@ def test_rope_scalar_path(hip):
     ((2, 3, 40), 2),
     ((4, 50, 3), 1),          # strided
     ((2, 16384), 1),          # longer than the register-resident path
+    ((3, 128264), 1),         # ... a vocabulary-sized row, no multiple of the workgroup's stride
+    ((37, 128), 1),           # 16 threads per row
+    ((2, 19, 72), 2),         # ... nine of them with a piece
+    ((21, 520), 1),           # 64 threads per row, two pieces per lane
+    ((9, 2048), 1),           # ... four pieces per lane
 ])
 def test_softmax(hip, shape, axis):
     import minit_amd.functional as F
@@ -111,7 +122,10 @@ def test_softmax_with_minus_inf(hip):
     _assert_ulp(got, O.softmax(x, 1), what="softmax -inf")
 
 
-@pytest.mark.parametrize("b,n,s,offset", [(2, 3, 8, 24), (16, 32, 1, 1023), (1, 2, 16, 0)])
+@pytest.mark.parametrize("b,n,s,offset", [(2, 3, 8, 24), (16, 32, 1, 1023), (1, 2, 16, 0),
+                                          (2, 3, 40, 88),       # rows of 128: 16 threads per row
+                                          (1, 2, 100, 412),     # rows of 512: 64 threads per row
+                                          (1, 1, 5, 9003)])     # rows of 9008: three walks over the row
 def test_softmax_causal(hip, b, n, s, offset):
     from minit_amd.hip.tensor import HIPTensor
     t = offset + s
@@ -130,7 +144,8 @@ def test_softmax_causal(hip, b, n, s, offset):
     _assert_ulp(out.numpy(), O.masked_softmax(xs, offset), what="causal softmax scaled")
 
 
-@pytest.mark.parametrize("shape,axis", [((512, 4096), 1), ((512, 1024), 1), ((3, 77, 5), 1), ((9, 13), 1)])
+@pytest.mark.parametrize("shape,axis", [((512, 4096), 1), ((512, 1024), 1), ((3, 77, 5), 1), ((9, 13), 1),
+                                        ((37, 128), 1), ((35, 100), 1), ((21, 520), 1), ((5, 16392), 1)])
 def test_sum_max(hip, shape, axis):
     import minit_amd.functional as F
     x = np.random.default_rng(8).normal(0, 3, size=shape).astype(np.float16)
