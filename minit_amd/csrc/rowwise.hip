@@ -13,6 +13,7 @@
 namespace mh {
 
 constexpr int kRowThreads = 256;
+constexpr int kWideThreads = 1024;  // workgroup of the kernels for rows beyond the registers of kRowThreads threads
 constexpr int kRowVec = 8;        // 16-bit elements per 16-byte load
 constexpr int kRowMaxChunks = 4;  // register-resident rows: b <= 256 * 8 * 4 = 8192
 
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_rows_kernel(
 // Rows too long for the registers of a workgroup (more than 8192 elements): the row is walked twice with
 // 16-byte loads, the second time out of the caches (plain loads first, streaming loads and stores last).
 template <typename T>
-__global__ __launch_bounds__(kRowThreads) void rms_norm_wide_kernel(
+__global__ __launch_bounds__(kWideThreads) void rms_norm_wide_kernel(
     const T* __restrict__ in, const T* __restrict__ weight, T* __restrict__ out, size_t b, float eps) {
     __shared__ float smem[16];
     const size_t row = blockIdx.x;
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_wide_kernel(
     const size_t nvec = b / kRowVec;
     float ss = 0.f;
 #pragma unroll 4
-    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+    for (size_t v = threadIdx.x; v < nvec; v += kWideThreads) {
         float f[8];
         unpack8<T>(src[v], f);
 #pragma unroll
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_wide_kernel(
     const float rms = sqrtf(ss / (float)b + eps);
     const float inv = 1.0f / rms;
 #pragma unroll 4
-    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+    for (size_t v = threadIdx.x; v < nvec; v += kWideThreads) {
         float f[8], w[8];
         unpack8<T>(stream_load(src + v), f);
         unpack8<T>(wsrc[v], w);
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_rows_kernel(
 // Rows of more than 8192 elements: maximum, sum and store in three walks over the row with 16-byte loads, the
 // second and third out of the caches; the arithmetic of softmax_rows_kernel.
 template <typename T, bool CAUSAL>
-__global__ __launch_bounds__(kRowThreads) void softmax_wide_kernel(
+__global__ __launch_bounds__(kWideThreads) void softmax_wide_kernel(
     const T* __restrict__ in, T* __restrict__ out, size_t b, size_t s, size_t offset, float scale) {
     __shared__ float smem[16];
     const size_t row = blockIdx.x;
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_wide_kernel(
     auto expd = [](float d) { return sizeof(T) == 2 ? __builtin_amdgcn_exp2f(d * 1.44269504088896340736f) : expf(d); };
     float mx = -INFINITY;
 #pragma unroll 4
-    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+    for (size_t v = threadIdx.x; v < nvec; v += kWideThreads) {
         float x[8];
         fetch(v, false, x);
 #pragma unroll
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_wide_kernel(
     mx = block_max(mx, smem);
     float sum = 0.f;
 #pragma unroll 4
-    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+    for (size_t v = threadIdx.x; v < nvec; v += kWideThreads) {
         float x[8];
         fetch(v, false, x);
 #pragma unroll
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_wide_kernel(
     sum = block_sum(sum, smem);
     const float inv = 1.0f / sum;
 #pragma unroll 4
-    for (size_t v = threadIdx.x; v < nvec; v += kRowThreads) {
+    for (size_t v = threadIdx.x; v < nvec; v += kWideThreads) {
         float x[8];
         fetch(v, true, x);
 #pragma unroll
@@ -520,7 +521,7 @@ static int rms_norm_t(hipStream_t st, const void* in, const void* weight, void* 
     hipLaunchKernelGGL((rms_norm_rows_kernel<T, LANES>), dim3(rows_grid(a, LANES)), dim3(kRowThreads), 0, st, (const T*)in, \
                        (const T*)weight, (T*)out, a, b, eps)
         if (!rows_fit_registers(b))
-            hipLaunchKernelGGL(rms_norm_wide_kernel<T>, dim3((unsigned)a), dim3(kRowThreads), 0, st, (const T*)in,
+            hipLaunchKernelGGL(rms_norm_wide_kernel<T>, dim3((unsigned)a), dim3(kWideThreads), 0, st, (const T*)in,
                                (const T*)weight, (T*)out, b, eps);
         else if (lanes == 16)
             MH_RMS_ROWS(16);
@@ -546,7 +547,7 @@ static int softmax_t(hipStream_t st, const void* in, void* out, size_t a, size_t
     hipLaunchKernelGGL((softmax_rows_kernel<T, CAUSAL, LANES>), dim3(rows_grid(a, LANES)), dim3(kRowThreads), 0, st, \
                        (const T*)in, (T*)out, a, b, s, offset, scale)
         if (!rows_fit_registers(b))
-            hipLaunchKernelGGL((softmax_wide_kernel<T, CAUSAL>), dim3((unsigned)a), dim3(kRowThreads), 0, st,
+            hipLaunchKernelGGL((softmax_wide_kernel<T, CAUSAL>), dim3((unsigned)a), dim3(kWideThreads), 0, st,
                                (const T*)in, (T*)out, b, s, offset, scale);
         else if (lanes == 16)
             MH_SOFTMAX_ROWS(16);
