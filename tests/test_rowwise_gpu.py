@@ -37,6 +37,7 @@ def _assert_ulp(got, ref, ulps=1.0, atol=1e-6, what=""):
     ((2, 19, 64), 2),       # ... half of the 16 threads of a row without a piece
     ((21, 520), 1),         # 64 threads per row, two pieces per lane, the second part empty
     ((9, 2048), 1),         # ... four pieces per lane
+    ((6, 2056), 1),         # ... five of up to eight pieces per lane, the fifth for one lane only
     ((5, 16384), 1),        # longer than the registers of a workgroup: two walks over the row
     ((3, 28680), 1),        # ... a length that is no multiple of the workgroup's stride
 ])
@@ -102,6 +103,7 @@ def test_rope_scalar_path(hip):
     ((2, 19, 72), 2),         # ... nine of them with a piece
     ((21, 520), 1),           # 64 threads per row, two pieces per lane
     ((9, 2048), 1),           # ... four pieces per lane
+    ((6, 3080), 1),           # ... seven of up to eight pieces per lane
 ])
 def test_softmax(hip, shape, axis):
     import minit_amd.functional as F
