@@ -147,7 +147,8 @@ def test_softmax_causal(hip, b, n, s, offset):
 
 
 @pytest.mark.parametrize("shape,axis", [((512, 4096), 1), ((512, 1024), 1), ((3, 77, 5), 1), ((9, 13), 1),
-                                        ((37, 128), 1), ((35, 100), 1), ((21, 520), 1), ((5, 16392), 1)])
+                                        ((37, 128), 1), ((35, 100), 1), ((21, 520), 1), ((5, 16392), 1),
+                                        ((3, 40011), 1)])   # a workgroup of 1024 threads per row, scalar tail
 def test_sum_max(hip, shape, axis):
     import minit_amd.functional as F
     x = np.random.default_rng(8).normal(0, 3, size=shape).astype(np.float16)
